@@ -1,0 +1,220 @@
+/*
+ * mi355_layer.h -- C ABI of libmi355_layer.so: hand-written gfx950 (MI355X) kernels for the
+ * transformer-layer hot path (attention core forward/backward/decode, rotary, RMSNorm, SwiGLU).
+ *
+ * The reference (Aleph-Alpha/scaling) is pure Python; it has no FFI for this path.  Each entry
+ * point below names the reference call site (path under src/scaling/) whose arithmetic it
+ * replaces.  A Python host binds these with ctypes; nothing here depends on libtorch.
+ *
+ * Conventions
+ *   - every function returns MI_OK (0) or a negative mi_status; it never throws, aborts or
+ *     synchronises the device.  mi_last_error() returns a thread-local description of the last
+ *     failure on the calling thread.
+ *   - all kernels are launched asynchronously on `stream` (a hipStream_t passed as void*;
+ *     NULL = the default stream).
+ *   - the library allocates no device memory and keeps no mutable global state: scratch space is
+ *     passed in by the caller (see the *_workspace_bytes helpers), so calls are re-entrant.
+ *   - tensors: innermost dimension contiguous, base pointers 16-byte aligned, every stride
+ *     (given in ELEMENTS) a multiple of 8 elements for 16-bit types (4 for fp32).
+ *   - "token" axes are the flattened (batch seq) axis of the reference's [b, s, ...] tensors;
+ *     cumulative sequence lengths are int32 offsets on that axis exactly as produced by
+ *     transformer/data/utils.py:40-74.
+ */
+#ifndef MI355_LAYER_H
+#define MI355_LAYER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_LAYER_VERSION 100
+
+typedef enum mi_status {
+    MI_OK = 0,
+    MI_E_NULL = -1,        /* a required pointer is NULL */
+    MI_E_DTYPE = -2,       /* dtype code not supported by this entry point */
+    MI_E_SHAPE = -3,       /* size / head_dim / head-count combination not supported */
+    MI_E_ALIGN = -4,       /* pointer or stride violates the alignment contract */
+    MI_E_WORKSPACE = -5,   /* workspace missing or too small */
+    MI_E_LAUNCH = -6,      /* the HIP runtime refused the launch (mi_last_error has details) */
+    MI_E_ARCH = -7         /* current device is not gfx950 */
+} mi_status;
+
+typedef enum mi_dtype { MI_BF16 = 0, MI_F16 = 1, MI_F32 = 2 } mi_dtype;
+
+int mi_version(void);
+const char* mi_last_error(void);
+const char* mi_status_string(int status);
+/* MI_OK when the current HIP device is a gfx950 part, MI_E_ARCH otherwise. */
+int mi_check_device(void);
+
+/* ------------------------------------------------------------------------------------------
+ * RMSNorm.  Replaces core/nn/norm/rms_norm.py:47-50:  y = x * rsqrt(mean(x^2, -1) + eps) * weight.
+ * Arithmetic in fp32, one rounding to `dtype` on store.  x, y: [n_rows, hidden]; weight: [hidden].
+ * rstd (optional, may be NULL): fp32 [n_rows], receives rsqrt(mean(x^2)+eps).
+ * Algorithmic HBM bytes: fwd 2*n_rows*hidden*e, bwd 3*n_rows*hidden*e (e = element size).
+ * ------------------------------------------------------------------------------------------ */
+int mi_rmsnorm_fwd(const void* x, const void* weight, void* y, float* rstd,
+                   int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
+
+/* Backward of the above (what autograd derives from rms_norm.py:47-50):
+ *   dx = rstd * (dy*w) - x * rstd^3 * mean(dy*w*x),   dweight = sum_rows dy * x * rstd.
+ * rstd is recomputed from x.  `workspace` holds per-block fp32 partial sums of dweight and must be
+ * at least mi_rmsnorm_bwd_workspace_bytes(n_rows, hidden) bytes; the partials are reduced in a
+ * fixed order (bit-reproducible).  dweight is written in `dtype`. */
+size_t mi_rmsnorm_bwd_workspace_bytes(int64_t n_rows, int64_t hidden);
+int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dweight,
+                   void* workspace, size_t workspace_bytes,
+                   int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * SwiGLU activation.  Replaces core/nn/mlp.py:248-249:  out = silu(a) * gate, elementwise over
+ * n_elem contiguous elements.  Backward: da = dout*gate*sig(a)*(1 + a*(1 - sig(a))), dgate = dout*silu(a).
+ * Algorithmic HBM bytes: fwd 3*n_elem*e, bwd 5*n_elem*e.
+ * ------------------------------------------------------------------------------------------ */
+int mi_swiglu_fwd(const void* a, const void* gate, void* out, int64_t n_elem, int dtype, void* stream);
+int mi_swiglu_bwd(const void* a, const void* gate, const void* dout, void* da, void* dgate,
+                  int64_t n_elem, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Rotary embedding (rotate-half pairing i <-> i + rot_dim/2), stand-alone kernel.
+ * Replaces core/nn/rotary.py:117-139 / :176-213 (cos/sin row gather by position id, then
+ * x*cos + rotate_half(x)*sin on the first rot_dim features, the rest copied).
+ * x, out: [n_tokens, n_heads, head_dim] with element strides (token, head); out may alias x.
+ * cos, sin: [table_rows, rot_dim] contiguous, in `table_dtype` (the reference keeps them in the
+ * module dtype).  position_ids: int64 [n_tokens] or NULL (then token t of every sequence uses
+ * row t % seq_len_for_null_ids).  inverse != 0 rotates by the negative angle (= the backward).
+ * Algorithmic HBM bytes: 2*n_tokens*n_heads*head_dim*e + table rows touched + 8*n_tokens.
+ * ------------------------------------------------------------------------------------------ */
+int mi_rotary(const void* x, void* out, const void* cos, const void* sin, const int64_t* position_ids,
+              int64_t n_tokens, int32_t n_heads, int32_t head_dim, int32_t rot_dim,
+              int64_t x_stride_token, int64_t x_stride_head, int64_t out_stride_token, int64_t out_stride_head,
+              int64_t table_rows, int64_t seq_len_for_null_ids, int inverse,
+              int dtype, int table_dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Attention core.  Replaces core/nn/attention/attention.py:108-213 (multi_head_attention) with
+ * core/nn/masked_softmax/masked_softmax.py:14-34 as softmax and :76-105 as mask, plus repeat_kv
+ * (:60-69) and, when cos/sin are given, the rotary call at :836-845.  Interface precedent for a
+ * fused kernel inside the reference: flash_attention(), attention.py:216-271.
+ *
+ * Layout: q [total_q, n_q_heads, head_dim], k/v [total_k, n_kv_heads, head_dim], o like q, element
+ * strides (token, head) per tensor.  Query head h reads kv head h / (n_q_heads / n_kv_heads).
+ * Mask predicate (never materialised): query token t of document j (cu_seqlens_q[j] <= t <
+ * cu_seqlens_q[j+1]) may attend key token u iff cu_seqlens_k[j] <= u < cu_seqlens_k[j+1] and, when
+ * causal, (u - cu_seqlens_k[j]) <= (t - cu_seqlens_q[j]) + (len_k - len_q).  For len_k == len_q this
+ * is exactly the reference's block-diagonal lower-triangular mask; for len_q == 1 it is the
+ * unmasked cached-decode case.  Softmax is evaluated in fp32 with scores scaled by softmax_scale
+ * (= query_key_scaling_factor * masked_softmax.scale); probabilities are rounded to bf16 before
+ * P*V as in the reference (attention.py:211).  A row without any allowed key yields zeros.
+ * lse: fp32 [n_q_heads, total_q], natural-log sum-exp of the scaled scores (needed by backward).
+ *
+ * Fused rotary (optional): if rotary_cos != NULL, q and k are rotated on load (rotate-half, the
+ * whole head_dim; tables [rotary_table_rows, head_dim] in the I/O dtype; position ids int64 per
+ * token, required).  Supported: dtype MI_BF16, head_dim in {64, 128}.
+ * Algorithmic work: 4 * head_dim * n_q_heads * P flop forward, 10 * head_dim * n_q_heads * P backward,
+ * P = number of allowed (query, key) pairs per head.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct mi_attn_args {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    float* lse;
+    const int32_t* cu_seqlens_q;   /* device, [n_docs + 1] */
+    const int32_t* cu_seqlens_k;   /* device, [n_docs + 1]; NULL = same as cu_seqlens_q */
+    int32_t n_docs;
+    int32_t causal;
+    int64_t total_q;
+    int64_t total_k;
+    int32_t n_q_heads;
+    int32_t n_kv_heads;
+    int32_t head_dim;
+    int32_t dtype;
+    int64_t q_stride_token, q_stride_head;
+    int64_t k_stride_token, k_stride_head;
+    int64_t v_stride_token, v_stride_head;
+    int64_t o_stride_token, o_stride_head;
+    float softmax_scale;
+    int32_t reserved0;
+    /* optional fused rotary */
+    const void* rotary_cos;
+    const void* rotary_sin;
+    const int64_t* position_ids_q;
+    const int64_t* position_ids_k;
+    int64_t rotary_table_rows;
+    void* stream;
+} mi_attn_args;
+
+int mi_attn_fwd(const mi_attn_args* args);
+
+/* Backward of mi_attn_fwd.  Extra inputs: o and lse from the forward, d_o (layout/strides of o).
+ * Outputs dq (strides of q), dk, dv (strides given).  GQA: dk/dv are summed over the query heads of
+ * each group inside the kernel, in a fixed order (no atomics; bit-reproducible).
+ * workspace: fp32 scratch of mi_attn_bwd_workspace_bytes() bytes (row sums of d_o * o). */
+typedef struct mi_attn_bwd_args {
+    mi_attn_args fwd;              /* q,k,v,o,lse,cu_seqlens,... as in the forward call */
+    const void* d_o;
+    void* dq;
+    void* dk;
+    void* dv;
+    int64_t dk_stride_token, dk_stride_head;
+    int64_t dv_stride_token, dv_stride_head;
+    void* workspace;
+    size_t workspace_bytes;
+} mi_attn_bwd_args;
+
+size_t mi_attn_bwd_workspace_bytes(int64_t total_q, int32_t n_q_heads, int32_t head_dim);
+int mi_attn_bwd(const mi_attn_bwd_args* args);
+
+/* ------------------------------------------------------------------------------------------
+ * Decode attention over a pre-allocated KV cache (one new query token per sequence).
+ * Replaces the cache branch attention.py:852-873 followed by multi_head_attention with a
+ * [1,1,1,1] all-false mask: softmax over every cached key.  The reference grows the cache by
+ * torch.cat per step and supports batch 1 only; here the cache is [batch, max_ctx, n_kv_heads,
+ * head_dim] (element strides batch/token/head), holds post-rotary K, and ctx_len[b] (int32, device)
+ * gives the number of valid keys of sequence b INCLUDING the token appended in this call.
+ *
+ * If k_new/v_new != NULL the kernel first appends them at position ctx_len[b]-1 (in-place append
+ * instead of torch.cat); with rotary_cos != NULL it rotates q and k_new by position_ids[b] before
+ * use/append (fused rotary).  q, o: [batch, n_q_heads, head_dim] contiguous.
+ * The key axis is split into n_splits chunks processed by different workgroups and merged by a
+ * second kernel; workspace = mi_attn_decode_workspace_bytes() bytes of fp32 scratch.
+ * Algorithmic HBM bytes: 2 * sum_b ctx_len[b] * n_kv_heads * head_dim * e  (K and V read once).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct mi_decode_args {
+    const void* q;
+    void* k_cache;
+    void* v_cache;
+    void* o;
+    const int32_t* ctx_len;        /* device, [batch] */
+    const void* k_new;             /* [batch, n_kv_heads, head_dim] or NULL */
+    const void* v_new;
+    const void* rotary_cos;        /* [rotary_table_rows, head_dim] or NULL */
+    const void* rotary_sin;
+    const int64_t* position_ids;   /* device, [batch]; required with rotary */
+    int64_t rotary_table_rows;
+    int32_t batch;
+    int32_t max_ctx;
+    int32_t n_q_heads;
+    int32_t n_kv_heads;
+    int32_t head_dim;
+    int32_t dtype;
+    int64_t cache_stride_batch, cache_stride_token, cache_stride_head;
+    float softmax_scale;
+    int32_t n_splits;              /* 0 = let the library choose */
+    void* workspace;
+    size_t workspace_bytes;
+    void* stream;
+} mi_decode_args;
+
+size_t mi_attn_decode_workspace_bytes(int32_t batch, int32_t n_q_heads, int32_t head_dim, int32_t max_ctx);
+int mi_attn_decode(const mi_decode_args* args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_LAYER_H */

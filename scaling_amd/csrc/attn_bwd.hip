@@ -1,0 +1,473 @@
+// Attention backward for gfx950 (bf16 MFMA, fp32 softmax recomputation from the saved log-sum-exp).
+//
+// Three kernels, no atomics, fixed summation order (bit-reproducible):
+//   1. delta[h][t] = sum_d dO[t][h][d] * O[t][h][d]
+//   2. dK/dV: a workgroup owns 128 keys of one KV head (32 per wavefront, K and V fragments stay in
+//      registers), loops over the query heads of the group and over 64-query tiles staged in LDS:
+//          S = Q K^T,  P = exp2(S*c - lse),  dP = dO V^T,  dS = P * (dP - delta)
+//          dV^T += dO^T P        dK^T += Q^T dS         (P / dS feed the MFMA straight from registers)
+//   3. dQ: a workgroup owns 128 queries of one head (32 per wavefront, Q and dO fragments in registers),
+//      loops over 64-key tiles:  S^T = K Q^T, dP^T = V dO^T, dS^T, dQ^T += K^T dS^T.
+// Operands whose contraction index is a token index are kept in LDS transposed and "chunk ordered"
+// (see attn_common.h) so that score tiles can be consumed in their accumulator layout.
+#include "attn_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// ---------------------------------------------------------------------------------------------
+// 1. delta
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_bwd_delta_kernel(const AttnParams p) {
+    constexpr int LPR = 16;  // lanes per (token, head) row, 8 elements each
+    const int64_t row = ((int64_t)blockIdx.x * kThreads + threadIdx.x) / LPR;
+    const int c = threadIdx.x % LPR;
+    const int64_t n_rows = (int64_t)p.total_q * p.nq;
+    float acc = 0.f;
+    const bool ok = row < n_rows && c < D / 8;
+    const int64_t t = ok ? row / p.nq : 0;
+    const int h = ok ? (int)(row % p.nq) : 0;
+    if (ok) {
+        const uint4 a = *reinterpret_cast<const uint4*>(p.o + t * p.o_st + (int64_t)h * p.o_sh + 8 * c);
+        const uint4 b = *reinterpret_cast<const uint4*>(p.d_o + t * p.o_st + (int64_t)h * p.o_sh + 8 * c);
+        float fa[8], fb[8];
+        Elem<__bf16>::unpack(a, fa);
+        Elem<__bf16>::unpack(b, fb);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc += fa[i] * fb[i];
+    }
+    acc = group_sum<LPR>(acc);
+    if (ok && c == 0) p.delta[(int64_t)h * p.total_q + t] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// helpers shared by kernels 2 and 3: stage a 64-token tile (row-major, padded) and its transposed
+// chunk-ordered copy from a thread-owned block of 4 tokens x 8 features
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ void load_quad(uint4 (&raw)[4], const __bf16* base, int64_t stride, int tok0, int total,
+                                          int quad, int dg) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int tok = tok0 + 4 * quad + j;
+        tok = tok < total ? tok : total - 1;
+        raw[j] = *reinterpret_cast<const uint4*>(base + (int64_t)tok * stride + 8 * dg);
+    }
+}
+
+template <int STR>
+__device__ __forceinline__ void store_rows(const uint4 (&raw)[4], uint16_t* rm, int quad, int dg) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(rm + (4 * quad + j) * STR + 8 * dg) = raw[j];
+}
+
+__device__ __forceinline__ void store_transposed(const uint4 (&raw)[4], char* tr, int quad, int dg) {
+    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&raw[0]);
+    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&raw[1]);
+    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&raw[2]);
+    const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&raw[3]);
+#pragma unroll
+    for (int dd = 0; dd < 8; ++dd) {
+        uint32_t lo, hi;
+        if (dd & 1) {
+            lo = (w0[dd >> 1] >> 16) | (w1[dd >> 1] & 0xffff0000u);
+            hi = (w2[dd >> 1] >> 16) | (w3[dd >> 1] & 0xffff0000u);
+        } else {
+            lo = (w0[dd >> 1] & 0xffffu) | (w1[dd >> 1] << 16);
+            hi = (w2[dd >> 1] & 0xffffu) | (w3[dd >> 1] << 16);
+        }
+        *reinterpret_cast<uint2*>(tr + chunk_quad_offset<64>(8 * dg + dd, quad)) = make_uint2(lo, hi);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 2. dK / dV
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(const AttnParams p) {
+    constexpr int BNK = 128;              // keys per workgroup (32 per wavefront)
+    constexpr int BQ = 64;                // queries per tile
+    constexpr int STR = D + 8;
+    constexpr int KS = D / 16;
+    constexpr int DT = D / 32;
+    constexpr int ITEMS = 16 * (D / 8);
+
+    __shared__ __attribute__((aligned(16))) uint16_t q_rm[BQ * STR];
+    __shared__ __attribute__((aligned(16))) uint16_t do_rm[BQ * STR];
+    __shared__ __attribute__((aligned(16))) uint16_t q_tr[D * BQ];
+    __shared__ __attribute__((aligned(16))) uint16_t do_tr[D * BQ];
+    __shared__ __attribute__((aligned(16))) float lse_lds[BQ];
+    __shared__ __attribute__((aligned(16))) float delta_lds[BQ];
+    __shared__ int range_lds[8];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+
+    const int nkb = (p.total_k + BNK - 1) / BNK;
+    const int work = xcd_remap(blockIdx.x, gridDim.x);
+    const int kb = work % nkb;            // early key blocks (most queries under a causal mask) first
+    const int kvh = work / nkb;
+    const int key = kb * BNK + wave * 32 + l32;
+
+    int qlo, qhi;
+    query_range(p, key, qlo, qhi);
+    int wmin = qhi > qlo ? qlo : 0x7fffffff, wmax = qhi > qlo ? qhi : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        wmin = min(wmin, __shfl_xor(wmin, off, 64));
+        wmax = max(wmax, __shfl_xor(wmax, off, 64));
+    }
+    if (lane == 0) { range_lds[wave] = wmin; range_lds[4 + wave] = wmax; }
+
+    // K and V fragments (B operands: column = key, contraction = feature)
+    bf16x8_t kf[KS], vf[KS];
+    {
+        const int kl = key < p.total_k ? key : p.total_k - 1;
+        const __bf16* kr = p.k + (int64_t)kl * p.k_st + (int64_t)kvh * p.k_sh + 8 * g;
+        const __bf16* vr = p.v + (int64_t)kl * p.v_st + (int64_t)kvh * p.v_sh + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            kf[ks] = *reinterpret_cast<const bf16x8_t*>(kr + 16 * ks);
+            vf[ks] = *reinterpret_cast<const bf16x8_t*>(vr + 16 * ks);
+        }
+    }
+    __syncthreads();
+    int bmin = min(min(range_lds[0], range_lds[1]), min(range_lds[2], range_lds[3]));
+    int bmax = max(max(range_lds[4], range_lds[5]), max(range_lds[6], range_lds[7]));
+    if (bmax <= bmin) { bmin = 0; bmax = 0; }
+    const int qt0 = bmin & ~(BQ - 1);
+    const int n_tiles = (bmax - qt0 + BQ - 1) / BQ;
+
+    f32x16_t dk_acc[DT], dv_acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dk_acc[dt][r] = 0.f; dv_acc[dt][r] = 0.f; }
+
+    const int quad = tid / (D / 8), dg = tid % (D / 8);
+    uint4 qraw[4], doraw[4];
+    float stat = 0.f;
+
+    const int total_iters = n_tiles * p.n_rep;
+    auto load_tile = [&](int iter) {
+        const int rep = iter / n_tiles, qt = qt0 + (iter % n_tiles) * BQ;
+        const int head = kvh * p.n_rep + rep;
+        if (tid < ITEMS) {
+            load_quad<D>(qraw, p.q + (int64_t)head * p.q_sh, p.q_st, qt, p.total_q, quad, dg);
+            load_quad<D>(doraw, p.d_o + (int64_t)head * p.o_sh, p.o_st, qt, p.total_q, quad, dg);
+        }
+        if (tid < 2 * BQ) {
+            int tok = qt + (tid & (BQ - 1));
+            tok = tok < p.total_q ? tok : p.total_q - 1;
+            const float* src = (tid < BQ) ? p.lse : p.delta;
+            stat = src[(int64_t)head * p.total_q + tok];
+            if (tid < BQ) stat *= 1.4426950408889634f;  // log-sum-exp in the exp2 domain
+        }
+    };
+    auto store_tile = [&]() {
+        if (tid < ITEMS) {
+            store_rows<STR>(qraw, q_rm, quad, dg);
+            store_rows<STR>(doraw, do_rm, quad, dg);
+            store_transposed(qraw, reinterpret_cast<char*>(q_tr), quad, dg);
+            store_transposed(doraw, reinterpret_cast<char*>(do_tr), quad, dg);
+        }
+        if (tid < BQ) lse_lds[tid] = stat;
+        else if (tid < 2 * BQ) delta_lds[tid - BQ] = stat;
+    };
+
+    if (total_iters > 0) {
+        load_tile(0);
+        store_tile();
+    }
+    __syncthreads();
+
+    for (int iter = 0; iter < total_iters; ++iter) {
+        const int qt = qt0 + (iter % n_tiles) * BQ;
+        if (iter + 1 < total_iters) load_tile(iter + 1);
+
+        const bool wave_active = (qt < wmax) && (qt + BQ > wmin);
+        if (wave_active) {
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                const int qs = qt + 32 * sub;
+                if (!((qs < wmax) && (qs + 32 > wmin))) continue;
+                f32x16_t s_acc, dp_acc;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { s_acc[r] = 0.f; dp_acc[r] = 0.f; }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(q_rm + (32 * sub + l32) * STR + 16 * ks + 8 * g);
+                    const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(do_rm + (32 * sub + l32) * STR + 16 * ks + 8 * g);
+                    s_acc = mfma_32x32x16(aq, kf[ks], s_acc);
+                    dp_acc = mfma_32x32x16(ad, vf[ks], dp_acc);
+                }
+                // rows of the accumulators are queries qs + 8a + 4g + c, the column is this lane's key
+                bf16x8_t pf[2], dsf[2];
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(lse_lds + 32 * sub + 8 * a + 4 * g);
+                    const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(delta_lds + 32 * sub + 8 * a + 4 * g);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int r = 4 * a + c;
+                        const int qi = qs + 8 * a + 4 * g + c;
+                        float pv = fast_exp2(s_acc[r] * p.scale_log2 - l4[c]);
+                        if (qi < qlo || qi >= qhi) pv = 0.f;
+                        const float ds = pv * (dp_acc[r] - d4[c]);
+                        pf[a >> 1][4 * (a & 1) + c] = (__bf16)pv;
+                        dsf[a >> 1][4 * (a & 1) + c] = (__bf16)ds;
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const bf16x8_t adt = *reinterpret_cast<const bf16x8_t*>(
+                            reinterpret_cast<const char*>(do_tr) + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
+                        const bf16x8_t aqt = *reinterpret_cast<const bf16x8_t*>(
+                            reinterpret_cast<const char*>(q_tr) + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
+                        dv_acc[dt] = mfma_32x32x16(adt, pf[m], dv_acc[dt]);
+                        dk_acc[dt] = mfma_32x32x16(aqt, dsf[m], dk_acc[dt]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (iter + 1 < total_iters) store_tile();
+        __syncthreads();
+    }
+
+    if (key < p.total_k) {
+        __bf16* dkr = p.dk + (int64_t)key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * g;
+        __bf16* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const uint32_t k0 = pack_bf16x2(dk_acc[dt][4 * a] * p.scale, dk_acc[dt][4 * a + 1] * p.scale);
+                const uint32_t k1 = pack_bf16x2(dk_acc[dt][4 * a + 2] * p.scale, dk_acc[dt][4 * a + 3] * p.scale);
+                *reinterpret_cast<uint2*>(dkr + 32 * dt + 8 * a) = make_uint2(k0, k1);
+                const uint32_t v0 = pack_bf16x2(dv_acc[dt][4 * a], dv_acc[dt][4 * a + 1]);
+                const uint32_t v1 = pack_bf16x2(dv_acc[dt][4 * a + 2], dv_acc[dt][4 * a + 3]);
+                *reinterpret_cast<uint2*>(dvr + 32 * dt + 8 * a) = make_uint2(v0, v1);
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 3. dQ
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnParams p) {
+    constexpr int BM = 128;
+    constexpr int BN = 64;
+    constexpr int STR = D + 8;
+    constexpr int KS = D / 16;
+    constexpr int DT = D / 32;
+    constexpr int ITEMS = 16 * (D / 8);
+
+    __shared__ __attribute__((aligned(16))) uint16_t k_rm[BN * STR];
+    __shared__ __attribute__((aligned(16))) uint16_t v_rm[BN * STR];
+    __shared__ __attribute__((aligned(16))) uint16_t k_tr[D * BN];
+    __shared__ int range_lds[8];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+
+    const int nqb = (p.total_q + BM - 1) / BM;
+    const int work = xcd_remap(blockIdx.x, gridDim.x);
+    const int rep = work % p.n_rep;
+    const int qb = nqb - 1 - (work / p.n_rep) % nqb;
+    const int kvh = work / (p.n_rep * nqb);
+    const int head = kvh * p.n_rep + rep;
+    const int tq = qb * BM + wave * 32 + l32;
+
+    int klo, khi;
+    key_range(p, tq, klo, khi);
+    int wmin = khi > klo ? klo : 0x7fffffff, wmax = khi > klo ? khi : 0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        wmin = min(wmin, __shfl_xor(wmin, off, 64));
+        wmax = max(wmax, __shfl_xor(wmax, off, 64));
+    }
+    if (lane == 0) { range_lds[wave] = wmin; range_lds[4 + wave] = wmax; }
+
+    const int tl = tq < p.total_q ? tq : p.total_q - 1;
+    bf16x8_t qf[KS], dof[KS];
+    {
+        const __bf16* qr = p.q + (int64_t)tl * p.q_st + (int64_t)head * p.q_sh + 8 * g;
+        const __bf16* dr = p.d_o + (int64_t)tl * p.o_st + (int64_t)head * p.o_sh + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qf[ks] = *reinterpret_cast<const bf16x8_t*>(qr + 16 * ks);
+            dof[ks] = *reinterpret_cast<const bf16x8_t*>(dr + 16 * ks);
+        }
+    }
+    const float lse2 = p.lse[(int64_t)head * p.total_q + tl] * 1.4426950408889634f;
+    const float delta = p.delta[(int64_t)head * p.total_q + tl];
+
+    __syncthreads();
+    int bmin = min(min(range_lds[0], range_lds[1]), min(range_lds[2], range_lds[3]));
+    int bmax = max(max(range_lds[4], range_lds[5]), max(range_lds[6], range_lds[7]));
+    if (bmax <= bmin) { bmin = 0; bmax = 0; }
+    const int kt0 = bmin & ~(BN - 1);
+    const int n_tiles = (bmax - kt0 + BN - 1) / BN;
+
+    f32x16_t dq_acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq_acc[dt][r] = 0.f;
+
+    const int quad = tid / (D / 8), dg = tid % (D / 8);
+    uint4 kraw[4], vraw[4];
+    const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
+    const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
+
+    auto load_tile = [&](int kt) {
+        if (tid < ITEMS) {
+            load_quad<D>(kraw, kbase, p.k_st, kt, p.total_k, quad, dg);
+            load_quad<D>(vraw, vbase, p.v_st, kt, p.total_k, quad, dg);
+        }
+    };
+    auto store_tile = [&]() {
+        if (tid < ITEMS) {
+            store_rows<STR>(kraw, k_rm, quad, dg);
+            store_rows<STR>(vraw, v_rm, quad, dg);
+            store_transposed(kraw, reinterpret_cast<char*>(k_tr), quad, dg);
+        }
+    };
+
+    if (n_tiles > 0) {
+        load_tile(kt0);
+        store_tile();
+    }
+    __syncthreads();
+
+    for (int it = 0; it < n_tiles; ++it) {
+        const int kt = kt0 + it * BN;
+        if (it + 1 < n_tiles) load_tile(kt + BN);
+
+        const bool wave_active = (kt < wmax) && (kt + BN > wmin);
+        if (wave_active) {
+            f32x16_t s_acc[2], dp_acc[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { s_acc[t][r] = 0.f; dp_acc[t][r] = 0.f; }
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(k_rm + (32 * t + l32) * STR + 16 * ks + 8 * g);
+                    const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(v_rm + (32 * t + l32) * STR + 16 * ks + 8 * g);
+                    s_acc[t] = mfma_32x32x16(ak, qf[ks], s_acc[t]);
+                    dp_acc[t] = mfma_32x32x16(av, dof[ks], dp_acc[t]);
+                }
+            }
+            bf16x8_t dsf[4];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kj = kt + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
+                    float pv = fast_exp2(s_acc[t][r] * p.scale_log2 - lse2);
+                    if (kj < klo || kj >= khi) pv = 0.f;
+                    const float ds = pv * (dp_acc[t][r] - delta);
+                    dsf[2 * t + (r >> 3)][r & 7] = (__bf16)ds;
+                }
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const bf16x8_t akt = *reinterpret_cast<const bf16x8_t*>(
+                        reinterpret_cast<const char*>(k_tr) + chunk_unit_offset<64>(32 * dt + l32, m, g));
+                    dq_acc[dt] = mfma_32x32x16(akt, dsf[m], dq_acc[dt]);
+                }
+            }
+        }
+        __syncthreads();
+        if (it + 1 < n_tiles) store_tile();
+        __syncthreads();
+    }
+
+    if (tq < p.total_q) {
+        __bf16* dqr = p.dq + (int64_t)tq * p.q_st + (int64_t)head * p.q_sh + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const uint32_t w0 = pack_bf16x2(dq_acc[dt][4 * a] * p.scale, dq_acc[dt][4 * a + 1] * p.scale);
+                const uint32_t w1 = pack_bf16x2(dq_acc[dt][4 * a + 2] * p.scale, dq_acc[dt][4 * a + 3] * p.scale);
+                *reinterpret_cast<uint2*>(dqr + 32 * dt + 8 * a) = make_uint2(w0, w1);
+            }
+    }
+}
+
+template <int D> int launch_bwd(const AttnParams& p, hipStream_t st) {
+    {
+        const int64_t rows = (int64_t)p.total_q * p.nq;
+        const int64_t blocks = (rows * 16 + kThreads - 1) / kThreads;
+        if (blocks > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_bwd: grid too large");
+        attn_bwd_delta_kernel<D><<<dim3((unsigned)blocks), dim3(kThreads), 0, st>>>(p);
+        int rc = mi_check_launch("attn_bwd_delta");
+        if (rc != MI_OK) return rc;
+    }
+    {
+        const int64_t grid = (((int64_t)p.total_k + 127) / 128) * p.nkv;
+        attn_bwd_dkdv_kernel<D><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
+        int rc = mi_check_launch("attn_bwd_dkdv");
+        if (rc != MI_OK) return rc;
+    }
+    {
+        const int64_t grid = (((int64_t)p.total_q + 127) / 128) * p.nq;
+        attn_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
+        return mi_check_launch("attn_bwd_dq");
+    }
+}
+
+}  // namespace
+
+int mi_attn_validate(const mi_attn_args* a, const char* who);
+void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p);
+
+extern "C" size_t mi_attn_bwd_workspace_bytes(int64_t total_q, int32_t n_q_heads, int32_t head_dim) {
+    (void)head_dim;
+    if (total_q <= 0 || n_q_heads <= 0) return 0;
+    return (size_t)total_q * (size_t)n_q_heads * sizeof(float);
+}
+
+extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
+    if (!b) return mi_fail(MI_E_NULL, "attn_bwd: args is null");
+    const mi_attn_args* a = &b->fwd;
+    int rc = mi_attn_validate(a, "attn_bwd");
+    if (rc != MI_OK) return rc;
+    if (a->rotary_cos) return mi_fail(MI_E_SHAPE, "attn_bwd: takes already rotated q/k (rotary is not fused into the backward)");
+    if (!a->o || !a->lse || !b->d_o || !b->dq || !b->dk || !b->dv)
+        return mi_fail(MI_E_NULL, "attn_bwd: o, lse, d_o, dq, dk, dv are required");
+    if (!mi_aligned16(a->o) || !mi_aligned16(b->d_o) || !mi_aligned16(b->dq) || !mi_aligned16(b->dk) || !mi_aligned16(b->dv))
+        return mi_fail(MI_E_ALIGN, "attn_bwd: tensors must be 16-byte aligned");
+    if (a->o_stride_token % 8 || a->o_stride_head % 8 || b->dk_stride_token % 8 || b->dk_stride_head % 8 ||
+        b->dv_stride_token % 8 || b->dv_stride_head % 8)
+        return mi_fail(MI_E_ALIGN, "attn_bwd: strides must be multiples of 8 elements");
+    if (a->total_q == 0) return MI_OK;
+    const size_t need = mi_attn_bwd_workspace_bytes(a->total_q, a->n_q_heads, a->head_dim);
+    if (!b->workspace || b->workspace_bytes < need || !mi_aligned16(b->workspace))
+        return mi_fail(MI_E_WORKSPACE, "attn_bwd: workspace needs %zu bytes (16-byte aligned), got %zu", need, b->workspace_bytes);
+    AttnParams p;
+    mi_attn_fill_params(a, &p);
+    p.d_o = (const __bf16*)b->d_o; p.dq = (__bf16*)b->dq; p.dk = (__bf16*)b->dk; p.dv = (__bf16*)b->dv;
+    p.dk_st = b->dk_stride_token; p.dk_sh = b->dk_stride_head;
+    p.dv_st = b->dv_stride_token; p.dv_sh = b->dv_stride_head;
+    p.delta = (float*)b->workspace;
+    hipStream_t st = (hipStream_t)a->stream;
+    switch (a->head_dim) {
+        case 32: return launch_bwd<32>(p, st);
+        case 64: return launch_bwd<64>(p, st);
+        case 96: return launch_bwd<96>(p, st);
+        case 128: return launch_bwd<128>(p, st);
+        default: return mi_fail(MI_E_SHAPE, "attn_bwd: head_dim %d unsupported", a->head_dim);
+    }
+}

@@ -1,0 +1,132 @@
+// Shared pieces of the gfx950 attention kernels: parameter block, document lookup, mask ranges,
+// MFMA wrapper and the LDS layouts used to feed v_mfma_f32_32x32x16_bf16.
+//
+// MFMA 32x32x16 (bf16) register layout, wavefront of 64 lanes, lane = 32*g + l32:
+//   A operand (32 x 16): lane holds row l32,    k = 8*g + 0..7   (8 bf16 = 4 VGPRs)
+//   B operand (16 x 32): lane holds column l32, k = 8*g + 0..7
+//   C / D     (32 x 32): lane holds column l32, rows 8*(r/4) + 4*g + (r%4) for r = 0..15 (16 fp32 VGPRs)
+// Because A and B use the same k assignment, any permutation of the contraction index that is applied
+// to both operands leaves the product unchanged.  The kernels rely on that: a C tile is re-used
+// directly as the B operand of the next product (contraction over its rows) with the k slot (g, i)
+// standing for row 8*(i/4) + 4*g + (i%4) of a 16-row chunk, and the matching A operand is stored in
+// LDS in exactly that order ("chunk order", see chunk_pos below).
+#pragma once
+#include "common.h"
+
+struct AttnParams {
+    const __bf16* q; const __bf16* k; const __bf16* v; __bf16* o; float* lse;
+    const int32_t* cu_q; const int32_t* cu_k;
+    int n_docs; int causal;
+    int total_q; int total_k;
+    int nq; int nkv; int n_rep;
+    int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;
+    float scale_log2;   // softmax_scale * log2(e)
+    const __bf16* cos; const __bf16* sin; const int64_t* pos_q; const int64_t* pos_k; int table_rows;
+    // backward only
+    const __bf16* d_o; __bf16* dq; __bf16* dk; __bf16* dv; float* delta;
+    int64_t dk_st, dk_sh, dv_st, dv_sh;
+    float scale;        // softmax_scale
+};
+
+__device__ __forceinline__ f32x16_t mfma_32x32x16(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// index j with cu[j] <= t < cu[j+1]  (cu has n_docs + 1 non-decreasing entries, cu[0] = 0)
+__device__ __forceinline__ int find_doc(const int32_t* __restrict__ cu, int n_docs, int t) {
+    int lo = 0, hi = n_docs;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (cu[mid] <= t) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// allowed keys of query token t: [klo, khi) on the flattened key axis (empty when khi <= klo)
+__device__ __forceinline__ void key_range(const AttnParams& p, int t, int& klo, int& khi) {
+    if (t >= p.total_q) { klo = 0; khi = 0; return; }
+    const int j = find_doc(p.cu_q, p.n_docs, t);
+    const int qs = p.cu_q[j], qe = p.cu_q[j + 1];
+    const int ks = p.cu_k[j], ke = p.cu_k[j + 1];
+    klo = ks;
+    khi = ke;
+    if (p.causal) {
+        const int lim = ks + (t - qs) + (ke - ks) - (qe - qs) + 1;
+        khi = lim < ke ? lim : ke;
+    }
+    if (khi < klo) khi = klo;
+}
+
+// allowed queries of key token u: [qlo, qhi) on the flattened query axis (mirror image of key_range)
+__device__ __forceinline__ void query_range(const AttnParams& p, int u, int& qlo, int& qhi) {
+    if (u >= p.total_k) { qlo = 0; qhi = 0; return; }
+    const int j = find_doc(p.cu_k, p.n_docs, u);
+    const int qs = p.cu_q[j], qe = p.cu_q[j + 1];
+    const int ks = p.cu_k[j], ke = p.cu_k[j + 1];
+    qlo = qs;
+    qhi = qe;
+    if (p.causal) {
+        // (u - ks) <= (t - qs) + (len_k - len_q)   <=>   t >= qs + (u - ks) - (len_k - len_q)
+        const int lim = qs + (u - ks) - ((ke - ks) - (qe - qs));
+        qlo = lim > qs ? lim : qs;
+    }
+    if (qlo > qhi) qlo = qhi;
+}
+
+// ---- "chunk order" LDS layout for operands whose contraction index is the row index of a C tile ----
+// A [R rows][N contraction] matrix (N multiple of 16) is stored row-major with 16-byte units XOR-
+// swizzled per row; inside each 16-wide chunk the contraction indices are permuted so that lane
+// group g finds its 8 k-slots contiguous:  unit (2*m + g) of row r holds indices
+// 16*m + {4g..4g+3, 8+4g..8+4g+3}.
+__device__ __forceinline__ int swz(int row) { return ((row >> 1) + (row >> 4)) & 7; }
+
+// byte offset of the 8-byte group holding contraction indices 4*quad .. 4*quad+3 (quad = index / 4)
+template <int N> __device__ __forceinline__ int chunk_quad_offset(int row, int quad) {
+    static_assert(N == 64, "one row = 8 swizzled units of 16 bytes");
+    const int m = quad >> 2, kq = quad & 3;
+    const int unit = 2 * m + (kq & 1);
+    return row * (N * 2) + ((unit ^ swz(row)) << 4) + ((kq >> 1) << 3);
+}
+
+// byte offset of the 16-byte unit read by lane group g for chunk m of row `row`
+template <int N> __device__ __forceinline__ int chunk_unit_offset(int row, int m, int g) {
+    static_assert(N == 64, "one row = 8 swizzled units of 16 bytes");
+    return row * (N * 2) + (((2 * m + g) ^ swz(row)) << 4);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    bf16x2_t p;
+    p[0] = (__bf16)lo;
+    p[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, p);
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// rotate-half rotary applied to a (first-half, second-half) pair of 8-element vectors; cos/sin hold
+// the table values of the first-half columns (both table halves are equal by construction)
+__device__ __forceinline__ void rotate_pair(uint4& lo, uint4& hi, const uint4& c, const uint4& s, float sign) {
+    uint32_t* l = reinterpret_cast<uint32_t*>(&lo);
+    uint32_t* h = reinterpret_cast<uint32_t*>(&hi);
+    const uint32_t* cw = reinterpret_cast<const uint32_t*>(&c);
+    const uint32_t* sw = reinterpret_cast<const uint32_t*>(&s);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float x0a = bf16_lo(l[i]), x0b = bf16_hi(l[i]);
+        const float x1a = bf16_lo(h[i]), x1b = bf16_hi(h[i]);
+        const float ca = bf16_lo(cw[i]), cb = bf16_hi(cw[i]);
+        const float sa = sign * bf16_lo(sw[i]), sb = sign * bf16_hi(sw[i]);
+        l[i] = pack_bf16x2(x0a * ca - x1a * sa, x0b * cb - x1b * sb);
+        h[i] = pack_bf16x2(x1a * ca + x0a * sa, x1b * cb + x0b * sb);
+    }
+}
+
+// maps the linear workgroup id to a work item so that the workgroups an XCD receives (ids congruent
+// modulo 8) form one contiguous range of work items (neighbouring items share K/V in that XCD's L2)
+__device__ __forceinline__ int xcd_remap(int linear, int total) {
+    if ((total & 7) != 0) return linear;
+    return (linear & 7) * (total >> 3) + (linear >> 3);
+}

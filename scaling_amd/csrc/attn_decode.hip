@@ -1,0 +1,354 @@
+// Decode attention over a pre-allocated KV cache for gfx950: one query token per sequence, HBM-bound.
+//
+// Grid = batch x KV heads x key splits.  All query heads of a GQA group are processed by the same
+// workgroup, so every cached K/V element is read from HBM exactly once.  Each wavefront streams its
+// own 32-key chunks:
+//     S^T[key][head]  = K * Q^T     v_mfma_f32_16x16x32_bf16, A = K rows loaded straight from global
+//                                   memory in operand layout, B = Q^T (heads of the group, zero padded)
+//     online softmax over keys      the lane's column is a head; 8 in-lane keys + 2 lane exchanges
+//     O^T[d][head]   += V^T * P^T   A = V^T read from a transposed per-wavefront LDS copy of the chunk
+// Partial (max, sum, O) per split go to a workspace and are merged by a second kernel.
+// A small first kernel appends the new K/V row in place (instead of the reference's torch.cat) and
+// applies rotary to it; the query is rotated while its fragments are loaded.
+#include "attn_common.h"
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kChunk = 32;           // keys per wavefront and iteration
+constexpr int kMaxSplits = 32;
+
+struct DecodeParams {
+    const __bf16* q; __bf16* kc; __bf16* vc; __bf16* o;
+    const int32_t* ctx_len;
+    const __bf16* k_new; const __bf16* v_new;
+    const __bf16* cos; const __bf16* sin; const int64_t* pos; int table_rows;
+    int batch, max_ctx, nq, nkv, n_rep, n_splits;
+    int64_t c_sb, c_st, c_sh;
+    float scale_log2;
+    float* ws_o;   // [batch][nq][n_splits][D]
+    float* ws_ml;  // [batch][nq][n_splits][2]
+};
+
+__device__ __forceinline__ f32x4v mfma_16x16x32(bf16x8_t a, bf16x8_t b, f32x4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// ---- in-place append of the new K/V row (optionally rotated) -------------------------------------
+template <int D>
+__global__ void decode_append_kernel(const DecodeParams p) {
+    // one thread per (batch, kv head, 8-feature vector of the first half)
+    constexpr int HV = D / 16;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= p.batch * p.nkv * HV) return;
+    const int c = idx % HV, kvh = (idx / HV) % p.nkv, b = idx / (HV * p.nkv);
+    const int ctx = p.ctx_len[b];
+    if (ctx < 1 || ctx > p.max_ctx) return;
+    const int64_t src = ((int64_t)b * p.nkv + kvh) * D + 8 * c;
+    const int64_t dst = (int64_t)b * p.c_sb + (int64_t)(ctx - 1) * p.c_st + (int64_t)kvh * p.c_sh + 8 * c;
+    uint4 lo = *reinterpret_cast<const uint4*>(p.k_new + src);
+    uint4 hi = *reinterpret_cast<const uint4*>(p.k_new + src + D / 2);
+    if (p.cos != nullptr) {
+        int64_t pos = p.pos[b];
+        pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+        const uint4 cv = *reinterpret_cast<const uint4*>(p.cos + pos * D + 8 * c);
+        const uint4 sv = *reinterpret_cast<const uint4*>(p.sin + pos * D + 8 * c);
+        rotate_pair(lo, hi, cv, sv, 1.0f);
+    }
+    *reinterpret_cast<uint4*>(p.kc + dst) = lo;
+    *reinterpret_cast<uint4*>(p.kc + dst + D / 2) = hi;
+    *reinterpret_cast<uint4*>(p.vc + dst) = *reinterpret_cast<const uint4*>(p.v_new + src);
+    *reinterpret_cast<uint4*>(p.vc + dst + D / 2) = *reinterpret_cast<const uint4*>(p.v_new + src + D / 2);
+}
+
+// ---- split kernel ----------------------------------------------------------------------------------
+template <int D, bool ROT>
+__global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeParams p) {
+    constexpr int KS = D / 32;          // contraction steps of Q K^T (32 features each)
+    constexpr int DT = D / 16;          // 16-row tiles of O^T
+    constexpr int VROW = kChunk + 8;    // padded row of the transposed V chunk (elements)
+    constexpr int V_ITEMS = 8 * (D / 8);  // (key quad, feature group) items of a 32-key chunk
+    constexpr int V_PER_LANE = V_ITEMS / 64;
+
+    __shared__ __attribute__((aligned(16))) uint16_t vt_lds[4][D * VROW];
+    __shared__ float wm_lds[4][16];
+    __shared__ float wl_lds[4][16];
+    __shared__ float wo_lds[4][16][D + 1];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l16 = lane & 15, G = lane >> 4;
+
+    const int split = blockIdx.x % p.n_splits;
+    const int kvh = (blockIdx.x / p.n_splits) % p.nkv;
+    const int b = blockIdx.x / (p.n_splits * p.nkv);
+
+    int ctx = p.ctx_len[b];
+    ctx = ctx < 0 ? 0 : (ctx > p.max_ctx ? p.max_ctx : ctx);
+    // keys of this split: [s0, s1), split length rounded up to whole workgroup iterations
+    int per = (ctx + p.n_splits - 1) / p.n_splits;
+    per = (per + 4 * kChunk - 1) / (4 * kChunk) * (4 * kChunk);
+    const int s0 = split * per;
+    const int s1 = min(ctx, s0 + per);
+    const int n_iter = s1 > s0 ? (s1 - s0 + 4 * kChunk - 1) / (4 * kChunk) : 0;
+
+    // Q^T fragments: column = head slot l16 (valid when < n_rep), contraction = features 32*ks + 8*G + i
+    bf16x8_t qf[KS];
+    {
+        const int hs = l16 < p.n_rep ? l16 : 0;
+        const __bf16* qr = p.q + ((int64_t)b * p.nq + kvh * p.n_rep + hs) * D + 8 * G;
+        uint4 raw[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qr + 32 * ks);
+        if constexpr (ROT) {
+            int64_t pos = p.pos[b];
+            pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+#pragma unroll
+            for (int ks = 0; ks < KS / 2; ++ks) {
+                const uint4 cv = *reinterpret_cast<const uint4*>(p.cos + pos * D + 32 * ks + 8 * G);
+                const uint4 sv = *reinterpret_cast<const uint4*>(p.sin + pos * D + 32 * ks + 8 * G);
+                rotate_pair(raw[ks], raw[ks + KS / 2], cv, sv, 1.0f);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (l16 >= p.n_rep) raw[ks] = make_uint4(0, 0, 0, 0);
+            qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
+        }
+    }
+
+    f32x4v o_acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o_acc[dt] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    float m_i = -INFINITY, l_i = 0.f;
+
+    const __bf16* kbase = p.kc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
+    const __bf16* vbase = p.vc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
+    char* vt = reinterpret_cast<char*>(vt_lds[wave]);
+
+    for (int it = 0; it < n_iter; ++it) {
+        const int key0 = s0 + (4 * it + wave) * kChunk;
+        const bool active = key0 < s1;          // wave-uniform
+        bf16x8_t kf[2][KS];
+        uint4 vraw[V_PER_LANE][4];
+        if (active) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                int tok = key0 + 16 * t + l16;
+                tok = tok < s1 ? tok : s1 - 1;
+                const __bf16* kr = kbase + (int64_t)tok * p.c_st + 8 * G;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) kf[t][ks] = *reinterpret_cast<const bf16x8_t*>(kr + 32 * ks);
+            }
+#pragma unroll
+            for (int j = 0; j < V_PER_LANE; ++j) {
+                const int item = lane + 64 * j;
+                const int quad = item / (D / 8), dg = item % (D / 8);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int tok = key0 + 4 * quad + r;
+                    tok = tok < s1 ? tok : s1 - 1;
+                    vraw[j][r] = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.c_st + 8 * dg);
+                }
+            }
+        }
+        __syncthreads();  // every wavefront is done reading its LDS chunk of the previous iteration
+        bf16x8_t pf;
+        float alpha = 1.f;
+        if (active) {
+            f32x4v s_acc[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                s_acc[t] = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) s_acc[t] = mfma_16x16x32(kf[t][ks], qf[ks], s_acc[t]);
+            }
+            // rows: keys key0 + 16*t + 4*G + r; column: head slot l16
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (key0 + 16 * t + 4 * G + r >= s1) s_acc[t][r] = -INFINITY;
+                    mx = fmaxf(mx, s_acc[t][r]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_i, mx * p.scale_log2);   // finite: the chunk holds >= 1 valid key
+            alpha = fast_exp2(m_i - m_new);
+            m_i = m_new;
+            float rs = 0.f;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float e = fast_exp2(s_acc[t][r] * p.scale_log2 - m_new);
+                    rs += e;
+                    pf[4 * t + r] = (__bf16)e;   // slot (G, i): key 16*(i/4) + 4*G + (i%4)
+                }
+            l_i = l_i * alpha + rs;
+            // transposed, slot-ordered copy of the V chunk: row = feature, 8 slots of lane group G contiguous
+#pragma unroll
+            for (int j = 0; j < V_PER_LANE; ++j) {
+                const int item = lane + 64 * j;
+                const int quad = item / (D / 8), dg = item % (D / 8);
+                const int col = 8 * (quad & 3) + 4 * (quad >> 2);
+                const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&vraw[j][0]);
+                const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&vraw[j][1]);
+                const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&vraw[j][2]);
+                const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&vraw[j][3]);
+#pragma unroll
+                for (int dd = 0; dd < 8; ++dd) {
+                    uint32_t lo, hi;
+                    if (dd & 1) {
+                        lo = (w0[dd >> 1] >> 16) | (w1[dd >> 1] & 0xffff0000u);
+                        hi = (w2[dd >> 1] >> 16) | (w3[dd >> 1] & 0xffff0000u);
+                    } else {
+                        lo = (w0[dd >> 1] & 0xffffu) | (w1[dd >> 1] << 16);
+                        hi = (w2[dd >> 1] & 0xffffu) | (w3[dd >> 1] << 16);
+                    }
+                    *reinterpret_cast<uint2*>(vt + ((8 * dg + dd) * VROW + col) * 2) = make_uint2(lo, hi);
+                }
+            }
+        }
+        __syncthreads();
+        if (active) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(vt + ((16 * dt + l16) * VROW + 8 * G) * 2);
+                o_acc[dt] = o_acc[dt] * alpha;
+                o_acc[dt] = mfma_16x16x32(a, pf, o_acc[dt]);
+            }
+        }
+    }
+
+    // ---- merge the four wavefronts, emit the split partial -----------------------------------------
+    l_i += __shfl_xor(l_i, 16, 64);
+    l_i += __shfl_xor(l_i, 32, 64);
+    __syncthreads();
+    if (G == 0) { wm_lds[wave][l16] = m_i; wl_lds[wave][l16] = l_i; }
+    if (l16 < p.n_rep) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) wo_lds[wave][l16][16 * dt + 4 * G + r] = o_acc[dt][r];
+    }
+    __syncthreads();
+    for (int idx = tid; idx < p.n_rep * D; idx += kThreads) {
+        const int hs = idx / D, d = idx % D;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, wm_lds[w][hs]);
+        float L = 0.f, O = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float wm = wm_lds[w][hs];
+            const float f = wm == -INFINITY ? 0.f : fast_exp2(wm - M);
+            L += f * wl_lds[w][hs];
+            O += f * wo_lds[w][hs][d];
+        }
+        const int64_t slot = ((int64_t)b * p.nq + kvh * p.n_rep + hs) * p.n_splits + split;
+        p.ws_o[slot * D + d] = O;
+        if (d == 0) { p.ws_ml[slot * 2] = M; p.ws_ml[slot * 2 + 1] = L; }
+    }
+}
+
+// ---- merge of the splits ------------------------------------------------------------------------------
+template <int D>
+__global__ void decode_merge_kernel(const DecodeParams p) {
+    // one thread per (batch, head, feature)
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.batch * p.nq * D) return;
+    const int d = (int)(idx % D);
+    const int64_t bh = idx / D;
+    float M = -INFINITY;
+    for (int s = 0; s < p.n_splits; ++s) M = fmaxf(M, p.ws_ml[(bh * p.n_splits + s) * 2]);
+    float L = 0.f, O = 0.f;
+    for (int s = 0; s < p.n_splits; ++s) {
+        const float m = p.ws_ml[(bh * p.n_splits + s) * 2];
+        const float f = m == -INFINITY ? 0.f : fast_exp2(m - M);
+        L += f * p.ws_ml[(bh * p.n_splits + s) * 2 + 1];
+        O += f * p.ws_o[(bh * p.n_splits + s) * D + d];
+    }
+    p.o[bh * D + d] = (__bf16)(L > 0.f ? O / L : 0.f);
+}
+
+int choose_splits(int batch, int nkv, int max_ctx) {
+    const int64_t pairs = (int64_t)batch * nkv;
+    int64_t s = (1024 + pairs - 1) / pairs;
+    const int64_t by_len = ((int64_t)max_ctx + 4 * kChunk - 1) / (4 * kChunk);
+    if (s > by_len) s = by_len;
+    if (s > kMaxSplits) s = kMaxSplits;
+    if (s < 1) s = 1;
+    return (int)s;
+}
+
+template <int D> int launch_decode(const DecodeParams& p, bool append, bool rot, hipStream_t st) {
+    if (append) {
+        const int n = p.batch * p.nkv * (D / 16);
+        decode_append_kernel<D><<<dim3((n + 127) / 128), dim3(128), 0, st>>>(p);
+        int rc = mi_check_launch("decode_append");
+        if (rc != MI_OK) return rc;
+    }
+    const unsigned grid = (unsigned)p.batch * p.nkv * p.n_splits;
+    if (rot) {
+        if constexpr (D == 64 || D == 128) decode_split_kernel<D, true><<<dim3(grid), dim3(kThreads), 0, st>>>(p);
+        else return mi_fail(MI_E_SHAPE, "attn_decode: fused rotary needs head_dim 64 or 128");
+    } else {
+        decode_split_kernel<D, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p);
+    }
+    int rc = mi_check_launch("decode_split");
+    if (rc != MI_OK) return rc;
+    const int64_t n = (int64_t)p.batch * p.nq * D;
+    decode_merge_kernel<D><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(p);
+    return mi_check_launch("decode_merge");
+}
+
+}  // namespace
+
+extern "C" size_t mi_attn_decode_workspace_bytes(int32_t batch, int32_t n_q_heads, int32_t head_dim, int32_t max_ctx) {
+    (void)max_ctx;
+    if (batch <= 0 || n_q_heads <= 0 || head_dim <= 0) return 0;
+    return (size_t)batch * n_q_heads * kMaxSplits * (size_t)(head_dim + 2) * sizeof(float);
+}
+
+extern "C" int mi_attn_decode(const mi_decode_args* a) {
+    if (!a) return mi_fail(MI_E_NULL, "attn_decode: args is null");
+    if (!a->q || !a->k_cache || !a->v_cache || !a->o || !a->ctx_len) return mi_fail(MI_E_NULL, "attn_decode: q, caches, o and ctx_len are required");
+    if (a->dtype != MI_BF16) return mi_fail(MI_E_DTYPE, "attn_decode: only bf16 is supported");
+    if (a->head_dim != 64 && a->head_dim != 128) return mi_fail(MI_E_SHAPE, "attn_decode: head_dim %d unsupported (64, 128)", a->head_dim);
+    if (a->batch <= 0 || a->max_ctx <= 0 || a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0 ||
+        a->n_q_heads / a->n_kv_heads > 16)
+        return mi_fail(MI_E_SHAPE, "attn_decode: bad batch/head configuration (group size must be <= 16)");
+    if ((a->k_new == nullptr) != (a->v_new == nullptr)) return mi_fail(MI_E_NULL, "attn_decode: k_new and v_new go together");
+    const bool rot = a->rotary_cos != nullptr || a->rotary_sin != nullptr;
+    if (rot && (!a->rotary_cos || !a->rotary_sin || !a->position_ids || a->rotary_table_rows <= 0))
+        return mi_fail(MI_E_NULL, "attn_decode: fused rotary needs cos, sin, position ids and the table size");
+    if (!mi_aligned16(a->q) || !mi_aligned16(a->k_cache) || !mi_aligned16(a->v_cache) || !mi_aligned16(a->o) ||
+        (a->k_new && (!mi_aligned16(a->k_new) || !mi_aligned16(a->v_new))) ||
+        (rot && (!mi_aligned16(a->rotary_cos) || !mi_aligned16(a->rotary_sin))))
+        return mi_fail(MI_E_ALIGN, "attn_decode: tensors must be 16-byte aligned");
+    if (a->cache_stride_batch % 8 || a->cache_stride_token % 8 || a->cache_stride_head % 8)
+        return mi_fail(MI_E_ALIGN, "attn_decode: cache strides must be multiples of 8 elements");
+    if (!(a->softmax_scale > 0.f)) return mi_fail(MI_E_SHAPE, "attn_decode: softmax_scale must be positive");
+    int splits = a->n_splits > 0 ? a->n_splits : choose_splits(a->batch, a->n_kv_heads, a->max_ctx);
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    const size_t need = (size_t)a->batch * a->n_q_heads * splits * (size_t)(a->head_dim + 2) * sizeof(float);
+    if (!a->workspace || a->workspace_bytes < need || !mi_aligned16(a->workspace))
+        return mi_fail(MI_E_WORKSPACE, "attn_decode: workspace needs %zu bytes (16-byte aligned), got %zu", need, a->workspace_bytes);
+    DecodeParams p{};
+    p.q = (const __bf16*)a->q; p.kc = (__bf16*)a->k_cache; p.vc = (__bf16*)a->v_cache; p.o = (__bf16*)a->o;
+    p.ctx_len = a->ctx_len; p.k_new = (const __bf16*)a->k_new; p.v_new = (const __bf16*)a->v_new;
+    p.cos = (const __bf16*)a->rotary_cos; p.sin = (const __bf16*)a->rotary_sin; p.pos = a->position_ids;
+    p.table_rows = (int)a->rotary_table_rows;
+    p.batch = a->batch; p.max_ctx = a->max_ctx; p.nq = a->n_q_heads; p.nkv = a->n_kv_heads;
+    p.n_rep = a->n_q_heads / a->n_kv_heads; p.n_splits = splits;
+    p.c_sb = a->cache_stride_batch; p.c_st = a->cache_stride_token; p.c_sh = a->cache_stride_head;
+    p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
+    p.ws_o = (float*)a->workspace;
+    p.ws_ml = p.ws_o + (size_t)a->batch * a->n_q_heads * splits * a->head_dim;
+    hipStream_t st = (hipStream_t)a->stream;
+    if (a->head_dim == 64) return launch_decode<64>(p, a->k_new != nullptr, rot, st);
+    return launch_decode<128>(p, a->k_new != nullptr, rot, st);
+}

@@ -1,0 +1,354 @@
+// Attention forward for gfx950 (bf16 MFMA, fp32 online softmax, causal / packed-document masks, GQA).
+//
+// Workgroup = 4 wavefronts; wavefront w owns QG groups of 32 consecutive query tokens of one head.
+// Keys/values stream through LDS in tiles of 64 tokens (double buffered, one barrier per tile).
+// Per tile and query group:
+//     S^T = K * Q^T            A = K tile rows from LDS, B = Q fragment held in registers
+//     online softmax           each lane owns ONE query (C column), so the row max / sum are in-lane
+//                              reductions plus a single exchange with lane ^ 32
+//     O^T += V^T * P^T         B = P^T taken straight from the S^T accumulators (no LDS round trip),
+//                              A = V^T read from a transposed, chunk-ordered LDS copy of the V tile
+// The mask is a per-lane key interval [klo, khi) derived from the cumulative sequence lengths; tiles
+// outside the union of the intervals are never loaded, tiles inside every interval skip the compare.
+#include "attn_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int BN = 64;  // keys per tile
+
+template <int D, int QG, bool ROT>
+__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnParams p) {
+    constexpr int BM = 128 * QG;
+    constexpr int KSTR = D + 8;           // padded K row (elements): conflict-free 128-bit row reads
+    constexpr int KS = D / 16;            // contraction steps of Q K^T
+    constexpr int DT = D / 32;            // 32-row tiles of O^T
+    constexpr int KV_VECS = D / 32;       // 128-bit K vectors per thread and tile
+    constexpr int V_ITEMS = 16 * (D / 8); // (key quad, 8-column group) items of a V tile
+    static_assert(D % 32 == 0 && D <= 128, "head_dim must be 32, 64, 96 or 128");
+
+    __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KSTR];
+    __shared__ __attribute__((aligned(16))) uint16_t vt_lds[2][D * BN];
+    __shared__ int range_lds[8];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+
+    // ---- work item ---------------------------------------------------------------------------
+    const int nqb = (p.total_q + BM - 1) / BM;
+    const int work = xcd_remap(blockIdx.x, gridDim.x);
+    const int rep = work % p.n_rep;
+    const int qb = nqb - 1 - (work / p.n_rep) % nqb;   // long (late) query blocks first
+    const int kvh = work / (p.n_rep * nqb);
+    const int head = kvh * p.n_rep + rep;
+    const int q0 = qb * BM + wave * (32 * QG);
+
+    // ---- per-lane query, mask interval, Q fragments ------------------------------------------
+    int tq[QG], klo[QG], khi[QG];
+    bf16x8_t qf[QG][KS];
+    int wmin = 0x7fffffff, wmax = 0;
+#pragma unroll
+    for (int i = 0; i < QG; ++i) {
+        tq[i] = q0 + 32 * i + l32;
+        key_range(p, tq[i], klo[i], khi[i]);
+        if (khi[i] > klo[i]) {
+            wmin = min(wmin, klo[i]);
+            wmax = max(wmax, khi[i]);
+        }
+        const int tl = tq[i] < p.total_q ? tq[i] : p.total_q - 1;
+        const __bf16* qrow = p.q + (int64_t)tl * p.q_st + (int64_t)head * p.q_sh + 8 * g;
+        uint4 raw[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qrow + 16 * ks);
+        if constexpr (ROT) {
+            int64_t pos = p.pos_q[tl];
+            pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+            const __bf16* cr = p.cos + pos * D + 8 * g;
+            const __bf16* sr = p.sin + pos * D + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < KS / 2; ++ks) {
+                const uint4 c = *reinterpret_cast<const uint4*>(cr + 16 * ks);
+                const uint4 s = *reinterpret_cast<const uint4*>(sr + 16 * ks);
+                rotate_pair(raw[ks], raw[ks + KS / 2], c, s, 1.0f);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[i][ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
+    }
+    // wave and block key ranges
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        wmin = min(wmin, __shfl_xor(wmin, off, 64));
+        wmax = max(wmax, __shfl_xor(wmax, off, 64));
+    }
+    if (lane == 0) { range_lds[wave] = wmin; range_lds[4 + wave] = wmax; }
+    __syncthreads();
+    int bmin = min(min(range_lds[0], range_lds[1]), min(range_lds[2], range_lds[3]));
+    int bmax = max(max(range_lds[4], range_lds[5]), max(range_lds[6], range_lds[7]));
+    if (bmax <= bmin) { bmin = 0; bmax = 0; }
+    const int kt0 = bmin & ~(BN - 1);
+    const int n_tiles = (bmax - kt0 + BN - 1) / BN;
+
+    // ---- accumulators ----------------------------------------------------------------------
+    f32x16_t o_acc[QG][DT];
+    float m_i[QG], l_i[QG];
+#pragma unroll
+    for (int i = 0; i < QG; ++i) {
+        m_i[i] = -INFINITY;
+        l_i[i] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o_acc[i][dt][r] = 0.f;
+    }
+
+    // ---- tile loaders ----------------------------------------------------------------------
+    uint4 kraw[KV_VECS];
+    uint4 vraw[4];
+    uint4 craw[ROT ? KV_VECS / 2 : 1], sraw[ROT ? KV_VECS / 2 : 1];  // rotary table rows of the K tile
+    const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
+    const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
+    const int v_kg = tid / (D / 8), v_dg = tid % (D / 8);
+
+    auto load_tile = [&](int kt) {
+        if constexpr (!ROT) {
+#pragma unroll
+            for (int j = 0; j < KV_VECS; ++j) {
+                const int idx = tid + kThreads * j;
+                const int row = idx / (D / 8), c = idx % (D / 8);
+                int tok = kt + row;
+                tok = tok < p.total_k ? tok : p.total_k - 1;
+                kraw[j] = *reinterpret_cast<const uint4*>(kbase + (int64_t)tok * p.k_st + 8 * c);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < KV_VECS / 2; ++j) {
+                const int idx = tid + kThreads * j;
+                const int row = idx / (D / 16), c = idx % (D / 16);
+                int tok = kt + row;
+                tok = tok < p.total_k ? tok : p.total_k - 1;
+                const __bf16* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
+                kraw[2 * j] = *reinterpret_cast<const uint4*>(kr);
+                kraw[2 * j + 1] = *reinterpret_cast<const uint4*>(kr + D / 2);
+                int64_t pos = p.pos_k[tok];
+                pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+                craw[j] = *reinterpret_cast<const uint4*>(p.cos + pos * D + 8 * c);
+                sraw[j] = *reinterpret_cast<const uint4*>(p.sin + pos * D + 8 * c);
+            }
+        }
+        if (tid < V_ITEMS) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int tok = kt + 4 * v_kg + j;
+                tok = tok < p.total_k ? tok : p.total_k - 1;
+                vraw[j] = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.v_st + 8 * v_dg);
+            }
+        }
+    };
+
+    auto store_tile = [&](int buf) {
+        uint16_t* ks = k_lds[buf];
+        if constexpr (!ROT) {
+#pragma unroll
+            for (int j = 0; j < KV_VECS; ++j) {
+                const int idx = tid + kThreads * j;
+                const int row = idx / (D / 8), c = idx % (D / 8);
+                *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[j];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < KV_VECS / 2; ++j) {
+                const int idx = tid + kThreads * j;
+                const int row = idx / (D / 16), c = idx % (D / 16);
+                rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);  // rotate after the MFMA section
+                *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[2 * j];
+                *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c + D / 2) = kraw[2 * j + 1];
+            }
+        }
+        if (tid < V_ITEMS) {
+            char* vt = reinterpret_cast<char*>(vt_lds[buf]);
+            const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&vraw[0]);
+            const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&vraw[1]);
+            const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&vraw[2]);
+            const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&vraw[3]);
+#pragma unroll
+            for (int dd = 0; dd < 8; ++dd) {
+                uint32_t lo, hi;
+                if (dd & 1) {
+                    lo = (w0[dd >> 1] >> 16) | (w1[dd >> 1] & 0xffff0000u);
+                    hi = (w2[dd >> 1] >> 16) | (w3[dd >> 1] & 0xffff0000u);
+                } else {
+                    lo = (w0[dd >> 1] & 0xffffu) | (w1[dd >> 1] << 16);
+                    hi = (w2[dd >> 1] & 0xffffu) | (w3[dd >> 1] << 16);
+                }
+                *reinterpret_cast<uint2*>(vt + chunk_quad_offset<BN>(8 * v_dg + dd, v_kg)) = make_uint2(lo, hi);
+            }
+        }
+    };
+
+    // ---- main loop ---------------------------------------------------------------------------
+    if (n_tiles > 0) {
+        load_tile(kt0);
+        store_tile(0);
+    }
+    __syncthreads();
+
+    for (int it = 0; it < n_tiles; ++it) {
+        const int kt = kt0 + it * BN;
+        const int buf = it & 1;
+        if (it + 1 < n_tiles) load_tile(kt + BN);
+
+        const bool wave_active = (kt < wmax) && (kt + BN > wmin);
+        if (wave_active) {
+            const uint16_t* ks = k_lds[buf];
+            const char* vt = reinterpret_cast<const char*>(vt_lds[buf]);
+
+            f32x16_t s_acc[QG][2];
+#pragma unroll
+            for (int i = 0; i < QG; ++i)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s_acc[i][t][r] = 0.f;
+
+#pragma unroll
+            for (int ksi = 0; ksi < KS; ++ksi) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks + (32 * t + l32) * KSTR + 16 * ksi + 8 * g);
+#pragma unroll
+                    for (int i = 0; i < QG; ++i) s_acc[i][t] = mfma_32x32x16(a, qf[i][ksi], s_acc[i][t]);
+                }
+            }
+
+            bf16x8_t pf[QG][4];
+#pragma unroll
+            for (int i = 0; i < QG; ++i) {
+                const bool need_mask = __any((kt < klo[i]) || (kt + BN > khi[i]));
+                if (need_mask) {
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int key = kt + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
+                            if (key < klo[i] || key >= khi[i]) s_acc[i][t][r] = -INFINITY;
+                        }
+                }
+                float mx = -INFINITY;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[i][t][r]);
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float m_new = fmaxf(m_i[i], mx * p.scale_log2);
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = fast_exp2(m_i[i] - m_use);
+                m_i[i] = m_new;
+                float rs = 0.f;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const float e = fast_exp2(s_acc[i][t][r] * p.scale_log2 - m_use);
+                        s_acc[i][t][r] = e;
+                        rs += e;
+                    }
+                l_i[i] = l_i[i] * alpha + rs;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o_acc[i][dt][r] *= alpha;
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const int t = m >> 1, r0 = 8 * (m & 1);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pf[i][m][e] = (__bf16)s_acc[i][t][r0 + e];
+                }
+            }
+
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(vt + chunk_unit_offset<BN>(32 * dt + l32, m, g));
+#pragma unroll
+                    for (int i = 0; i < QG; ++i) o_acc[i][dt] = mfma_32x32x16(a, pf[i][m], o_acc[i][dt]);
+                }
+            }
+        }
+
+        if (it + 1 < n_tiles) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue ------------------------------------------------------------------------------
+#pragma unroll
+    for (int i = 0; i < QG; ++i) {
+        const float l_tot = l_i[i] + __shfl_xor(l_i[i], 32, 64);
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        if (tq[i] < p.total_q) {
+            __bf16* orow = p.o + (int64_t)tq[i] * p.o_st + (int64_t)head * p.o_sh + 4 * g;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const uint32_t w0 = pack_bf16x2(o_acc[i][dt][4 * a] * inv, o_acc[i][dt][4 * a + 1] * inv);
+                    const uint32_t w1 = pack_bf16x2(o_acc[i][dt][4 * a + 2] * inv, o_acc[i][dt][4 * a + 3] * inv);
+                    *reinterpret_cast<uint2*>(orow + 32 * dt + 8 * a) = make_uint2(w0, w1);
+                }
+            if (g == 0 && p.lse != nullptr) {
+                const float lse = l_tot > 0.f ? (m_i[i] + __log2f(l_tot)) * 0.6931471805599453f : INFINITY;
+                p.lse[(int64_t)head * p.total_q + tq[i]] = lse;
+            }
+        }
+    }
+}
+
+template <int D, int QG, bool ROT> int launch(const AttnParams& p, hipStream_t st) {
+    constexpr int BM = 128 * QG;
+    const int64_t nqb = ((int64_t)p.total_q + BM - 1) / BM;
+    const int64_t grid = nqb * p.nq;
+    if (grid > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_fwd: grid too large");
+    attn_fwd_kernel<D, QG, ROT><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
+    return mi_check_launch("attn_fwd");
+}
+
+template <int D> int launch_d(const AttnParams& p, bool rot, int qg, hipStream_t st) {
+    if (rot) {
+        if constexpr (D == 64 || D == 128) {
+            return qg == 2 ? launch<D, 2, true>(p, st) : launch<D, 1, true>(p, st);
+        } else {
+            return mi_fail(MI_E_SHAPE, "attn_fwd: fused rotary needs head_dim 64 or 128");
+        }
+    }
+    return qg == 2 ? launch<D, 2, false>(p, st) : launch<D, 1, false>(p, st);
+}
+
+}  // namespace
+
+int mi_attn_validate(const mi_attn_args* a, const char* who);
+void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p);
+
+extern "C" int mi_attn_fwd(const mi_attn_args* a) {
+    int rc = mi_attn_validate(a, "attn_fwd");
+    if (rc != MI_OK) return rc;
+    if (!a->o) return mi_fail(MI_E_NULL, "attn_fwd: o is null");
+    if (!mi_aligned16(a->o) || a->o_stride_token % 8 || a->o_stride_head % 8)
+        return mi_fail(MI_E_ALIGN, "attn_fwd: o must be 16-byte aligned with strides multiple of 8");
+    if (a->total_q == 0) return MI_OK;
+    AttnParams p;
+    mi_attn_fill_params(a, &p);
+    const bool rot = a->rotary_cos != nullptr;
+    // two query groups per wavefront halve the LDS traffic per MFMA; worth it once the grid still
+    // fills the chip
+    const int64_t blocks_qg2 = (((int64_t)p.total_q + 255) / 256) * p.nq;
+    const int qg = blocks_qg2 >= 512 ? 2 : 1;
+    hipStream_t st = (hipStream_t)a->stream;
+    switch (a->head_dim) {
+        case 32: return launch_d<32>(p, rot, qg, st);
+        case 64: return launch_d<64>(p, rot, qg, st);
+        case 96: return launch_d<96>(p, rot, qg, st);
+        case 128: return launch_d<128>(p, rot, qg, st);
+        default: return mi_fail(MI_E_SHAPE, "attn_fwd: head_dim %d unsupported (32, 64, 96, 128)", a->head_dim);
+    }
+}

@@ -1,0 +1,61 @@
+"""Builds libmi355_layer.so (gfx950 only) from the HIP sources in this directory.
+
+Usage: python -m scaling_amd.csrc.build      (or scaling_amd.csrc.build.build() from Python)
+Each .hip file is one translation unit; objects go to ./build/, the library next to the sources.
+"""
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libmi355_layer.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+SOURCES = ["abi.hip", "rmsnorm.hip", "swiglu.hip", "rotary.hip", "attn_host.hip", "attn_fwd.hip", "attn_bwd.hip",
+           "attn_decode.hip"]
+# packed fp32 VALU instructions stay disabled for every device translation unit
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; libmi355_layer.so cannot be built")
+    return exe
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, cwd=HERE, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), proc.stdout, proc.stderr))
+    return proc
+
+
+def build(verbose: bool = False, jobs: int = 8) -> str:
+    hipcc = _hipcc()
+    obj_dir = os.path.join(HERE, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        _run([hipcc] + FLAGS + ["-c", src, "-o", obj])
+        if verbose:
+            print("compiled", src, flush=True)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs)
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print("linked", LIB_PATH, flush=True)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build(verbose=True)
+    sys.exit(0)

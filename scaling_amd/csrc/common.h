@@ -1,0 +1,96 @@
+// Shared device/host helpers for the gfx950 kernels of libmi355_layer.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include "../../include/mi355_layer.h"
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+#define MI_WAVE 64
+
+// ---- host side error plumbing -------------------------------------------------------------
+void mi_set_error(const char* fmt, ...);
+int mi_fail(int status, const char* fmt, ...);
+int mi_check_launch(const char* what);
+
+static inline bool mi_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- element type traits: 8 x 16-bit or 4 x fp32 per 128-bit access --------------------------
+template <typename T> struct Elem;
+
+template <> struct Elem<__bf16> {
+    static constexpr int kVec = 8;
+    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ uint4 pack(const float* f) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bf16x2_t p;
+            p[0] = (__bf16)f[2 * i];
+            p[1] = (__bf16)f[2 * i + 1];
+            w[i] = __builtin_bit_cast(uint32_t, p);
+        }
+        return make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    static __device__ __forceinline__ float load1(const __bf16* p) { return (float)*p; }
+    static __device__ __forceinline__ void store1(__bf16* p, float v) { *p = (__bf16)v; }
+};
+
+template <> struct Elem<_Float16> {
+    static constexpr int kVec = 8;
+    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+        f16x8_t h = __builtin_bit_cast(f16x8_t, u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)h[i];
+    }
+    static __device__ __forceinline__ uint4 pack(const float* f) {
+        f16x8_t h;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[i] = (_Float16)f[i];
+        return __builtin_bit_cast(uint4, h);
+    }
+    static __device__ __forceinline__ float load1(const _Float16* p) { return (float)*p; }
+    static __device__ __forceinline__ void store1(_Float16* p, float v) { *p = (_Float16)v; }
+};
+
+template <> struct Elem<float> {
+    static constexpr int kVec = 4;
+    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+        f[0] = __uint_as_float(u.x); f[1] = __uint_as_float(u.y);
+        f[2] = __uint_as_float(u.z); f[3] = __uint_as_float(u.w);
+    }
+    static __device__ __forceinline__ uint4 pack(const float* f) {
+        return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+    }
+    static __device__ __forceinline__ float load1(const float* p) { return *p; }
+    static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+};
+
+// ---- wavefront reductions (64 lanes) -------------------------------------------------------
+template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, MI_WAVE);
+    return v;
+}
+
+#define MI_DISPATCH_DTYPE(dtype, ...)                                       \
+    switch (dtype) {                                                        \
+        case MI_BF16: { using T = __bf16; __VA_ARGS__; break; }             \
+        case MI_F16: { using T = _Float16; __VA_ARGS__; break; }            \
+        case MI_F32: { using T = float; __VA_ARGS__; break; }               \
+        default: return mi_fail(MI_E_DTYPE, "unsupported dtype code %d", (int)(dtype)); \
+    }

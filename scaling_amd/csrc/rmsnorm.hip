@@ -1,0 +1,303 @@
+// RMSNorm forward / backward for gfx950: single pass over HBM, 128-bit accesses, fp32 math.
+//
+// A row is owned by TPR threads (16 / 64 lanes of one wavefront, or a whole 256-thread block for very
+// wide rows); each thread keeps CH 128-bit vectors of the row in registers, so x (and dy) are read
+// from HBM exactly once.  Rows handled by a wavefront need no block barrier, so the memory pipeline
+// stays full.  The weight gradient is accumulated in registers across a block's rows, combined in
+// LDS in a fixed order, written as one fp32 partial row per block and reduced by a second kernel.
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kMaxBwdBlocks = 512;
+
+template <int TPR> __device__ __forceinline__ float row_sum(float v, float* lds) {
+    if constexpr (TPR <= 64) {
+        return group_sum<TPR>(v);
+    } else {
+        v = group_sum<64>(v);
+        const int wave = threadIdx.x >> 6;
+        __syncthreads();  // protect lds from the previous use
+        if ((threadIdx.x & 63) == 0) lds[wave] = v;
+        __syncthreads();
+        return lds[0] + lds[1] + lds[2] + lds[3];
+    }
+}
+
+template <typename T, int TPR, int CH>
+__global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                              T* __restrict__ y, float* __restrict__ rstd_out,
+                                                              int64_t n_rows, int hidden, float eps) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int RPB = kBlock / TPR;
+    __shared__ float lds[4];
+    const int tr = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+    const bool row_ok = row < n_rows;
+    const int vecs = hidden / V;
+    const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
+    uint4 raw[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int v = c * TPR + tr;
+        raw[c] = (row_ok && v < vecs) ? xr[v] : make_uint4(0, 0, 0, 0);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        float f[V];
+        Elem<T>::unpack(raw[c], f);
+#pragma unroll
+        for (int i = 0; i < V; ++i) ss += f[i] * f[i];
+    }
+    ss = row_sum<TPR>(ss, lds);
+    const float rstd = rsqrtf(ss / (float)hidden + eps);
+    if (rstd_out != nullptr && row_ok && tr == 0) rstd_out[row] = rstd;
+    if (!row_ok) return;
+    const uint4* wr = reinterpret_cast<const uint4*>(w);
+    uint4* yr = reinterpret_cast<uint4*>(y + row * hidden);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int v = c * TPR + tr;
+        if (v < vecs) {
+            float f[V], g[V];
+            Elem<T>::unpack(raw[c], f);
+            Elem<T>::unpack(wr[v], g);
+#pragma unroll
+            for (int i = 0; i < V; ++i) f[i] = (f[i] * rstd) * g[i];
+            yr[v] = Elem<T>::pack(f);
+        }
+    }
+}
+
+template <typename T, int TPR, int CH>
+__global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                              const T* __restrict__ dy, T* __restrict__ dx,
+                                                              float* __restrict__ dw_partial, int64_t n_rows,
+                                                              int hidden, float eps) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int RPB = kBlock / TPR;
+    extern __shared__ float dw_lds[];  // [hidden]
+    __shared__ float lds[4];
+    const int tr = threadIdx.x % TPR;
+    const int rg = threadIdx.x / TPR;
+    const int vecs = hidden / V;
+    const float inv_h = 1.0f / (float)hidden;
+
+    float wf[CH][V];
+    float acc[CH][V];
+    const uint4* wr = reinterpret_cast<const uint4*>(w);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int v = c * TPR + tr;
+        uint4 u = (v < vecs) ? wr[v] : make_uint4(0, 0, 0, 0);
+        Elem<T>::unpack(u, wf[c]);
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[c][i] = 0.f;
+    }
+
+    const int64_t row_step = (int64_t)gridDim.x * RPB;
+    // every thread of the block runs the same number of iterations (barriers inside row_sum for TPR=256)
+    const int64_t iters = (n_rows + row_step - 1) / row_step;
+    for (int64_t it = 0; it < iters; ++it) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
+        const uint4* gr = reinterpret_cast<const uint4*>(dy + (row_ok ? row : 0) * hidden);
+        uint4 xraw[CH], graw[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int v = c * TPR + tr;
+            const bool ok = row_ok && v < vecs;
+            xraw[c] = ok ? xr[v] : make_uint4(0, 0, 0, 0);
+            graw[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
+        }
+        float ss = 0.f, dot = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float xf[V], gf[V];
+            Elem<T>::unpack(xraw[c], xf);
+            Elem<T>::unpack(graw[c], gf);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                ss += xf[i] * xf[i];
+                dot += gf[i] * wf[c][i] * xf[i];
+            }
+        }
+        ss = row_sum<TPR>(ss, lds);
+        dot = row_sum<TPR>(dot, lds);
+        const float rstd = rsqrtf(ss * inv_h + eps);
+        const float coef = dot * inv_h * rstd * rstd * rstd;
+        if (row_ok) {
+            uint4* dxr = reinterpret_cast<uint4*>(dx + row * hidden);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+                    float xf[V], gf[V], o[V];
+                    Elem<T>::unpack(xraw[c], xf);
+                    Elem<T>::unpack(graw[c], gf);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        o[i] = rstd * (gf[i] * wf[c][i]) - xf[i] * coef;
+                        acc[c][i] += gf[i] * (xf[i] * rstd);
+                    }
+                    dxr[v] = Elem<T>::pack(o);
+                }
+            }
+        }
+    }
+
+    // combine the row groups of this block in a fixed order, then emit one partial row
+    for (int i = threadIdx.x; i < hidden; i += kBlock) dw_lds[i] = 0.f;
+    __syncthreads();
+    for (int g = 0; g < RPB; ++g) {
+        if (rg == g) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) dw_lds[v * V + i] += acc[c][i];
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out = dw_partial + (int64_t)blockIdx.x * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kBlock) out[i] = dw_lds[i];
+}
+
+// dw[col] = sum_p partial[p][col]; 16 columns x 16 row groups per block, fixed summation order.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw,
+                                                                    int n_partial, int hidden) {
+    __shared__ float lds[16][17];
+    const int cl = threadIdx.x % 16, pg = threadIdx.x / 16;
+    const int col = blockIdx.x * 16 + cl;
+    float s = 0.f;
+    if (col < hidden)
+        for (int p = pg; p < n_partial; p += 16) s += partial[(int64_t)p * hidden + col];
+    lds[pg][cl] = s;
+    __syncthreads();
+    if (pg == 0 && col < hidden) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t += lds[i][cl];
+        Elem<T>::store1(dw + col, t);
+    }
+}
+
+struct Plan { int tpr; int ch; };
+
+template <typename T> bool make_plan(int64_t hidden, Plan* p) {
+    constexpr int V = Elem<T>::kVec;
+    if (hidden <= 0 || hidden % V != 0) return false;
+    const int64_t vecs = hidden / V;
+    int tpr, ch;
+    if (vecs <= 16) { tpr = 16; ch = 1; }
+    else if (vecs <= 64 * 8) { tpr = 64; ch = (int)((vecs + 63) / 64); }
+    else if (vecs <= 256 * 8) { tpr = 256; ch = (int)((vecs + 255) / 256); }
+    else return false;
+    int c = 1;
+    while (c < ch) c *= 2;
+    p->tpr = tpr; p->ch = c;
+    return true;
+}
+
+int bwd_blocks(int64_t n_rows, int tpr) {
+    const int64_t rpb = kBlock / tpr;
+    int64_t b = (n_rows + rpb - 1) / rpb;
+    if (b > kMaxBwdBlocks) b = kMaxBwdBlocks;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+template <int TPRV, int CHV> struct PlanTag { static constexpr int TPR = TPRV; static constexpr int CH = CHV; };
+
+// calls f(PlanTag<tpr, ch>{}) for the instantiated (threads per row, vectors per thread) pair
+template <typename F> bool dispatch_plan(const Plan& plan, F&& f) {
+#define RMS_CASE(TPRV, CHV) if (plan.tpr == TPRV && plan.ch == CHV) { f(PlanTag<TPRV, CHV>{}); return true; }
+    RMS_CASE(16, 1)
+    RMS_CASE(64, 1) RMS_CASE(64, 2) RMS_CASE(64, 4) RMS_CASE(64, 8)
+    RMS_CASE(256, 4) RMS_CASE(256, 8)
+#undef RMS_CASE
+    return false;
+}
+
+template <typename T>
+int launch_fwd(const void* x, const void* w, void* y, float* rstd, int64_t n_rows, int64_t hidden, float eps,
+               hipStream_t st) {
+    Plan plan;
+    if (!make_plan<T>(hidden, &plan))
+        return mi_fail(MI_E_SHAPE, "rmsnorm: hidden=%lld unsupported (must be a multiple of %d and <= %d)",
+                       (long long)hidden, Elem<T>::kVec, 256 * 8 * Elem<T>::kVec);
+    const bool launched = dispatch_plan(plan, [&](auto tag) {
+        constexpr int TPR = decltype(tag)::TPR;
+        constexpr int CH = decltype(tag)::CH;
+        const int rpb = kBlock / TPR;
+        const unsigned grid = (unsigned)((n_rows + rpb - 1) / rpb);
+        rmsnorm_fwd_kernel<T, TPR, CH><<<dim3(grid), dim3(kBlock), 0, st>>>((const T*)x, (const T*)w, (T*)y, rstd, n_rows,
+                                                                            (int)hidden, eps);
+    });
+    if (!launched) return mi_fail(MI_E_SHAPE, "rmsnorm: no kernel for hidden=%lld", (long long)hidden);
+    return mi_check_launch("rmsnorm_fwd");
+}
+
+template <typename T>
+int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, void* ws, size_t ws_bytes,
+               int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
+    Plan plan;
+    if (!make_plan<T>(hidden, &plan))
+        return mi_fail(MI_E_SHAPE, "rmsnorm: hidden=%lld unsupported", (long long)hidden);
+    const int blocks = bwd_blocks(n_rows, plan.tpr);
+    if (ws == nullptr || ws_bytes < (size_t)blocks * hidden * sizeof(float))
+        return mi_fail(MI_E_WORKSPACE, "rmsnorm_bwd: workspace needs %zu bytes, got %zu",
+                       (size_t)blocks * hidden * sizeof(float), ws_bytes);
+    const bool launched = dispatch_plan(plan, [&](auto tag) {
+        constexpr int TPR = decltype(tag)::TPR;
+        constexpr int CH = decltype(tag)::CH;
+        rmsnorm_bwd_kernel<T, TPR, CH><<<dim3(blocks), dim3(kBlock), hidden * sizeof(float), st>>>(
+            (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps);
+    });
+    if (!launched) return mi_fail(MI_E_SHAPE, "rmsnorm: no kernel for hidden=%lld", (long long)hidden);
+    int rc = mi_check_launch("rmsnorm_bwd");
+    if (rc != MI_OK) return rc;
+    rmsnorm_dw_reduce_kernel<T><<<dim3((unsigned)((hidden + 15) / 16)), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw,
+                                                                                               blocks, (int)hidden);
+    return mi_check_launch("rmsnorm_dw_reduce");
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_rmsnorm_fwd(const void* x, const void* weight, void* y, float* rstd, int64_t n_rows, int64_t hidden, float eps,
+                   int dtype, void* stream) {
+    if (!x || !weight || !y) return mi_fail(MI_E_NULL, "rmsnorm_fwd: null pointer");
+    if (n_rows < 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "rmsnorm_fwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
+    if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(y)) return mi_fail(MI_E_ALIGN, "rmsnorm_fwd: pointers must be 16-byte aligned");
+    if (n_rows == 0) return MI_OK;
+    MI_DISPATCH_DTYPE(dtype, return launch_fwd<T>(x, weight, y, rstd, n_rows, hidden, eps, (hipStream_t)stream));
+    return MI_OK;
+}
+
+size_t mi_rmsnorm_bwd_workspace_bytes(int64_t n_rows, int64_t hidden) {
+    (void)n_rows;
+    return (size_t)kMaxBwdBlocks * (size_t)(hidden > 0 ? hidden : 0) * sizeof(float);
+}
+
+int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dweight, void* workspace,
+                   size_t workspace_bytes, int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream) {
+    if (!x || !weight || !dy || !dx || !dweight) return mi_fail(MI_E_NULL, "rmsnorm_bwd: null pointer");
+    if (n_rows <= 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "rmsnorm_bwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
+    if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(dy) || !mi_aligned16(dx) || !mi_aligned16(workspace))
+        return mi_fail(MI_E_ALIGN, "rmsnorm_bwd: pointers must be 16-byte aligned");
+    if (hidden * sizeof(float) > 160 * 1024 - 64) return mi_fail(MI_E_SHAPE, "rmsnorm_bwd: hidden too large for LDS");
+    MI_DISPATCH_DTYPE(dtype, return launch_bwd<T>(x, weight, dy, dx, dweight, workspace, workspace_bytes, n_rows, hidden,
+                                                  eps, (hipStream_t)stream));
+    return MI_OK;
+}
+
+}  // extern "C"

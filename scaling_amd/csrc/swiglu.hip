@@ -1,0 +1,132 @@
+// SwiGLU activation forward / backward for gfx950: elementwise, 128-bit accesses, fp32 math.
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 2;  // 128-bit vectors per thread and tensor
+
+__device__ __forceinline__ float sigmoid_f(float a) { return 1.0f / (1.0f + __expf(-a)); }
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_fwd_kernel(const T* __restrict__ a, const T* __restrict__ g,
+                                                             T* __restrict__ out, int64_t n_vec, int64_t n_elem) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t base = ((int64_t)blockIdx.x * kBlock) * kUnroll + threadIdx.x;
+    uint4 ra[kUnroll], rg[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = base + (int64_t)u * kBlock;
+        if (v < n_vec) {
+            ra[u] = reinterpret_cast<const uint4*>(a)[v];
+            rg[u] = reinterpret_cast<const uint4*>(g)[v];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = base + (int64_t)u * kBlock;
+        if (v < n_vec) {
+            float fa[V], fg[V];
+            Elem<T>::unpack(ra[u], fa);
+            Elem<T>::unpack(rg[u], fg);
+#pragma unroll
+            for (int i = 0; i < V; ++i) fa[i] = (fa[i] * sigmoid_f(fa[i])) * fg[i];
+            reinterpret_cast<uint4*>(out)[v] = Elem<T>::pack(fa);
+        }
+    }
+    // scalar tail (n_elem not a multiple of the vector width): handled by the last block
+    if (blockIdx.x == gridDim.x - 1) {
+        for (int64_t i = n_vec * V + threadIdx.x; i < n_elem; i += kBlock) {
+            const float x = Elem<T>::load1(a + i);
+            Elem<T>::store1(out + i, (x * sigmoid_f(x)) * Elem<T>::load1(g + i));
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const T* __restrict__ a, const T* __restrict__ g,
+                                                             const T* __restrict__ dout, T* __restrict__ da,
+                                                             T* __restrict__ dg, int64_t n_vec, int64_t n_elem) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t base = ((int64_t)blockIdx.x * kBlock) * kUnroll + threadIdx.x;
+    uint4 ra[kUnroll], rg[kUnroll], rd[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = base + (int64_t)u * kBlock;
+        if (v < n_vec) {
+            ra[u] = reinterpret_cast<const uint4*>(a)[v];
+            rg[u] = reinterpret_cast<const uint4*>(g)[v];
+            rd[u] = reinterpret_cast<const uint4*>(dout)[v];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = base + (int64_t)u * kBlock;
+        if (v < n_vec) {
+            float fa[V], fg[V], fd[V], oa[V], og[V];
+            Elem<T>::unpack(ra[u], fa);
+            Elem<T>::unpack(rg[u], fg);
+            Elem<T>::unpack(rd[u], fd);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const float s = sigmoid_f(fa[i]);
+                oa[i] = fd[i] * fg[i] * s * (1.0f + fa[i] * (1.0f - s));
+                og[i] = fd[i] * (fa[i] * s);
+            }
+            reinterpret_cast<uint4*>(da)[v] = Elem<T>::pack(oa);
+            reinterpret_cast<uint4*>(dg)[v] = Elem<T>::pack(og);
+        }
+    }
+    if (blockIdx.x == gridDim.x - 1) {
+        for (int64_t i = n_vec * V + threadIdx.x; i < n_elem; i += kBlock) {
+            const float x = Elem<T>::load1(a + i), gg = Elem<T>::load1(g + i), d = Elem<T>::load1(dout + i);
+            const float s = sigmoid_f(x);
+            Elem<T>::store1(da + i, d * gg * s * (1.0f + x * (1.0f - s)));
+            Elem<T>::store1(dg + i, d * (x * s));
+        }
+    }
+}
+
+template <typename T> unsigned grid_for(int64_t n_elem, int64_t* n_vec) {
+    *n_vec = n_elem / Elem<T>::kVec;
+    int64_t blocks = (*n_vec + (int64_t)kBlock * kUnroll - 1) / ((int64_t)kBlock * kUnroll);
+    if (blocks < 1) blocks = 1;
+    return (unsigned)blocks;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_swiglu_fwd(const void* a, const void* gate, void* out, int64_t n_elem, int dtype, void* stream) {
+    if (!a || !gate || !out) return mi_fail(MI_E_NULL, "swiglu_fwd: null pointer");
+    if (n_elem < 0) return mi_fail(MI_E_SHAPE, "swiglu_fwd: negative size");
+    if (!mi_aligned16(a) || !mi_aligned16(gate) || !mi_aligned16(out)) return mi_fail(MI_E_ALIGN, "swiglu_fwd: pointers must be 16-byte aligned");
+    if (n_elem == 0) return MI_OK;
+    if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "swiglu_fwd: too many elements");
+    MI_DISPATCH_DTYPE(dtype, {
+        int64_t n_vec;
+        const unsigned grid = grid_for<T>(n_elem, &n_vec);
+        swiglu_fwd_kernel<T><<<dim3(grid), dim3(kBlock), 0, (hipStream_t)stream>>>((const T*)a, (const T*)gate, (T*)out, n_vec, n_elem);
+    });
+    return mi_check_launch("swiglu_fwd");
+}
+
+int mi_swiglu_bwd(const void* a, const void* gate, const void* dout, void* da, void* dgate, int64_t n_elem, int dtype,
+                  void* stream) {
+    if (!a || !gate || !dout || !da || !dgate) return mi_fail(MI_E_NULL, "swiglu_bwd: null pointer");
+    if (n_elem < 0) return mi_fail(MI_E_SHAPE, "swiglu_bwd: negative size");
+    if (!mi_aligned16(a) || !mi_aligned16(gate) || !mi_aligned16(dout) || !mi_aligned16(da) || !mi_aligned16(dgate))
+        return mi_fail(MI_E_ALIGN, "swiglu_bwd: pointers must be 16-byte aligned");
+    if (n_elem == 0) return MI_OK;
+    if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "swiglu_bwd: too many elements");
+    MI_DISPATCH_DTYPE(dtype, {
+        int64_t n_vec;
+        const unsigned grid = grid_for<T>(n_elem, &n_vec);
+        swiglu_bwd_kernel<T><<<dim3(grid), dim3(kBlock), 0, (hipStream_t)stream>>>((const T*)a, (const T*)gate, (const T*)dout,
+                                                                                  (T*)da, (T*)dgate, n_vec, n_elem);
+    });
+    return mi_check_launch("swiglu_bwd");
+}
+
+}  // extern "C"

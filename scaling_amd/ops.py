@@ -1,0 +1,314 @@
+"""Tensor-level entry points of the HIP kernels (through the C ABI) and their autograd wrappers.
+
+Every function here launches a hand-written gfx950 kernel on the current stream.  None of them falls
+back to PyTorch arithmetic: tensors must live on the GPU, and shapes or dtypes a kernel does not
+support raise.  Autograd functions keep tensors with ``ctx.save_for_backward`` only, so they work
+under saved-tensor hooks (activation checkpointing) and are deterministic under recomputation.
+"""
+
+import ctypes
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import MiAttnArgs, MiAttnBwdArgs, MiDecodeArgs, check, dtype_code, ptr, stream_ptr
+
+__all__ = [
+    "rms_norm", "swiglu", "rotary_embedding", "attention", "attention_forward", "attention_backward",
+    "decode_attention", "rms_norm_forward", "rms_norm_backward", "swiglu_forward", "swiglu_backward",
+]
+
+
+def _need_cuda(*tensors):
+    _lib.require_device()
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("scaling_amd ops take GPU tensors only (got a CPU tensor); there is no CPU path")
+
+
+# ------------------------------------------------------------------------------------------------
+# RMSNorm
+# ------------------------------------------------------------------------------------------------
+def rms_norm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    _need_cuda(x, weight)
+    assert x.shape[-1] == weight.shape[0] and weight.dtype == x.dtype
+    x2 = x.contiguous().view(-1, x.shape[-1])
+    w = weight.contiguous()
+    y = torch.empty_like(x2)
+    check(_lib.load().mi_rmsnorm_fwd(ptr(x2), ptr(w), ptr(y), None, x2.shape[0], x2.shape[1], float(eps),
+                                     dtype_code(x.dtype), stream_ptr()), "mi_rmsnorm_fwd")
+    return y.view(x.shape)
+
+
+def rms_norm_backward(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor, eps: float):
+    _need_cuda(x, weight, dy)
+    lib = _lib.load()
+    x2 = x.contiguous().view(-1, x.shape[-1])
+    dy2 = dy.contiguous().view(-1, x.shape[-1])
+    w = weight.contiguous()
+    dx = torch.empty_like(x2)
+    dw = torch.empty_like(w)
+    nbytes = lib.mi_rmsnorm_bwd_workspace_bytes(x2.shape[0], x2.shape[1])
+    ws = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
+    check(lib.mi_rmsnorm_bwd(ptr(x2), ptr(w), ptr(dy2), ptr(dx), ptr(dw), ptr(ws), nbytes, x2.shape[0], x2.shape[1],
+                             float(eps), dtype_code(x.dtype), stream_ptr()), "mi_rmsnorm_bwd")
+    return dx.view(x.shape), dw
+
+
+class _RMSNorm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        ctx.save_for_backward(x, weight)
+        ctx.eps = eps
+        return rms_norm_forward(x, weight, eps)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        dx, dw = rms_norm_backward(x, weight, dy, ctx.eps)
+        return dx, dw, None
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """y = x * rsqrt(mean(x^2, -1) + eps) * weight (fp32 math, one rounding)."""
+    return _RMSNorm.apply(x, weight, eps)
+
+
+# ------------------------------------------------------------------------------------------------
+# SwiGLU
+# ------------------------------------------------------------------------------------------------
+def swiglu_forward(a: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    _need_cuda(a, gate)
+    assert a.shape == gate.shape and a.dtype == gate.dtype
+    a, gate = a.contiguous(), gate.contiguous()
+    out = torch.empty_like(a)
+    check(_lib.load().mi_swiglu_fwd(ptr(a), ptr(gate), ptr(out), a.numel(), dtype_code(a.dtype), stream_ptr()),
+          "mi_swiglu_fwd")
+    return out
+
+
+def swiglu_backward(a: torch.Tensor, gate: torch.Tensor, dout: torch.Tensor):
+    _need_cuda(a, gate, dout)
+    a, gate, dout = a.contiguous(), gate.contiguous(), dout.contiguous()
+    da, dg = torch.empty_like(a), torch.empty_like(gate)
+    check(_lib.load().mi_swiglu_bwd(ptr(a), ptr(gate), ptr(dout), ptr(da), ptr(dg), a.numel(), dtype_code(a.dtype),
+                                    stream_ptr()), "mi_swiglu_bwd")
+    return da, dg
+
+
+class _SwiGLU(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, gate):
+        ctx.save_for_backward(a, gate)
+        return swiglu_forward(a, gate)
+
+    @staticmethod
+    def backward(ctx, dout):
+        a, gate = ctx.saved_tensors
+        return swiglu_backward(a, gate, dout)
+
+
+def swiglu(a: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """silu(a) * gate."""
+    return _SwiGLU.apply(a, gate)
+
+
+# ------------------------------------------------------------------------------------------------
+# rotary (stand-alone kernel)
+# ------------------------------------------------------------------------------------------------
+def _rotary_launch(x, cos, sin, position_ids, seq_len_for_null_ids, inverse, out=None):
+    """x: [tokens, heads, head_dim] view whose last dim is contiguous; cos/sin: [rows, rot_dim]."""
+    _need_cuda(x, cos, sin, position_ids)
+    assert x.dim() == 3 and x.stride(2) == 1
+    assert cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape and cos.dim() == 2
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if position_ids is not None:
+        position_ids = position_ids.contiguous()
+        assert position_ids.dtype == torch.int64 and position_ids.numel() == x.shape[0]
+    check(_lib.load().mi_rotary(ptr(x), ptr(out), ptr(cos), ptr(sin), ptr(position_ids), x.shape[0], x.shape[1],
+                                x.shape[2], cos.shape[1], x.stride(0), x.stride(1), out.stride(0), out.stride(1),
+                                cos.shape[0], int(seq_len_for_null_ids), int(bool(inverse)), dtype_code(x.dtype),
+                                dtype_code(cos.dtype), stream_ptr()), "mi_rotary")
+    return out
+
+
+class _Rotary(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, cos, sin, position_ids, seq_len_for_null_ids):
+        ctx.save_for_backward(cos, sin, position_ids if position_ids is not None else torch.empty(0, device=x.device))
+        ctx.has_ids = position_ids is not None
+        ctx.seq_len = seq_len_for_null_ids
+        return _rotary_launch(x, cos, sin, position_ids, seq_len_for_null_ids, False)
+
+    @staticmethod
+    def backward(ctx, dout):
+        cos, sin, ids = ctx.saved_tensors
+        if dout.stride(-1) != 1:
+            dout = dout.contiguous()
+        dx = _rotary_launch(dout, cos, sin, ids if ctx.has_ids else None, ctx.seq_len, True)
+        return dx, None, None, None, None
+
+
+def rotary_embedding(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                     position_ids: Optional[torch.Tensor] = None, seq_len_for_null_ids: int = 0) -> torch.Tensor:
+    """Rotate-half rotary on x [tokens, heads, head_dim]; position_ids int64 [tokens] (flattened (b s))."""
+    return _Rotary.apply(x, cos, sin, position_ids, seq_len_for_null_ids)
+
+
+# ------------------------------------------------------------------------------------------------
+# attention core
+# ------------------------------------------------------------------------------------------------
+def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None) -> MiAttnArgs:
+    a = MiAttnArgs()
+    a.q, a.k, a.v, a.o, a.lse = ptr(q), ptr(k), ptr(v), ptr(o), ptr(lse)
+    a.cu_seqlens_q, a.cu_seqlens_k = ptr(cu_q), ptr(cu_k)
+    a.n_docs = cu_q.numel() - 1
+    a.causal = int(bool(causal))
+    a.total_q, a.total_k = q.shape[0], k.shape[0]
+    a.n_q_heads, a.n_kv_heads, a.head_dim = q.shape[1], k.shape[1], q.shape[2]
+    a.dtype = dtype_code(q.dtype)
+    a.q_stride_token, a.q_stride_head = q.stride(0), q.stride(1)
+    a.k_stride_token, a.k_stride_head = k.stride(0), k.stride(1)
+    a.v_stride_token, a.v_stride_head = v.stride(0), v.stride(1)
+    a.o_stride_token, a.o_stride_head = o.stride(0), o.stride(1)
+    a.softmax_scale = float(scale)
+    if rotary is not None:
+        cos, sin, pos_q, pos_k = rotary
+        a.rotary_cos, a.rotary_sin = ptr(cos), ptr(sin)
+        a.position_ids_q, a.position_ids_k = ptr(pos_q), ptr(pos_k)
+        a.rotary_table_rows = cos.shape[0]
+    a.stream = stream_ptr()
+    return a
+
+
+def _check_qkv(q, k, v, cu_q, cu_k):
+    _need_cuda(q, k, v, cu_q, cu_k)
+    for t in (q, k, v):
+        assert t.dim() == 3 and t.stride(2) == 1, "q/k/v must be [tokens, heads, head_dim] with contiguous features"
+    assert k.shape == v.shape and q.shape[2] == k.shape[2]
+    assert cu_q.dtype == torch.int32 and cu_q.is_contiguous()
+    if cu_k is not None:
+        assert cu_k.dtype == torch.int32 and cu_k.is_contiguous() and cu_k.numel() == cu_q.numel()
+
+
+def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None, rotary=None):
+    """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens])."""
+    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(q.shape[2])
+    if rotary is not None:
+        cos, sin, pos_q, pos_k = rotary
+        assert cos.dtype == q.dtype and cos.is_contiguous() and sin.is_contiguous() and cos.shape[1] == q.shape[2]
+        assert pos_q.dtype == torch.int64 and pos_q.is_contiguous() and pos_q.numel() == q.shape[0]
+        assert pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0]
+    o = torch.empty((q.shape[0], q.shape[1], q.shape[2]), dtype=q.dtype, device=q.device)
+    lse = torch.empty((q.shape[1], q.shape[0]), dtype=torch.float32, device=q.device)
+    a = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary)
+    check(_lib.load().mi_attn_fwd(ctypes.byref(a)), "mi_attn_fwd")
+    return o, lse
+
+
+def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None):
+    """Returns (dq, dk, dv) for already rotated q/k."""
+    _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    lib = _lib.load()
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(q.shape[2])
+    if do.stride() != o.stride():
+        do = do.contiguous()
+        assert do.stride() == o.stride()
+    dq = torch.empty_like(q)
+    if dq.stride() != q.stride():
+        dq = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+    nbytes = lib.mi_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], q.shape[2])
+    ws = torch.empty(max(nbytes // 4, 4), dtype=torch.float32, device=q.device)
+    b = MiAttnBwdArgs()
+    b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale)
+    b.d_o, b.dq, b.dk, b.dv = ptr(do), ptr(dq), ptr(dk), ptr(dv)
+    b.dk_stride_token, b.dk_stride_head = dk.stride(0), dk.stride(1)
+    b.dv_stride_token, b.dv_stride_head = dv.stride(0), dv.stride(1)
+    b.workspace, b.workspace_bytes = ptr(ws), ws.numel() * 4
+    check(lib.mi_attn_bwd(ctypes.byref(b)), "mi_attn_bwd")
+    return dq, dk, dv
+
+
+class _Attention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, cu_q, cu_k, causal, scale):
+        o, lse = attention_forward(q, k, v, cu_q, cu_k, causal, scale)
+        ctx.save_for_backward(q, k, v, o, lse, cu_q, cu_k if cu_k is not None else cu_q)
+        ctx.causal, ctx.scale = causal, scale
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, lse, cu_q, cu_k = ctx.saved_tensors
+        dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale)
+        return dq, dk, dv, None, None, None, None
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
+              cu_seqlens_k: Optional[torch.Tensor] = None, causal: bool = True,
+              softmax_scale: Optional[float] = None) -> torch.Tensor:
+    """Differentiable attention core on q [tokens, n_q, d], k/v [tokens_k, n_kv, d] (bf16).
+
+    Tokens are the flattened (batch seq) axis; cu_seqlens are int32 offsets on it.  Returns
+    o [tokens, n_q, d].
+    """
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(q.shape[2])
+    return _Attention.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, float(softmax_scale))
+
+
+# ------------------------------------------------------------------------------------------------
+# decode attention over a pre-allocated KV cache
+# ------------------------------------------------------------------------------------------------
+def decode_workspace(batch: int, n_q_heads: int, head_dim: int, max_ctx: int, device) -> torch.Tensor:
+    nbytes = _lib.load().mi_attn_decode_workspace_bytes(batch, n_q_heads, head_dim, max_ctx)
+    return torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+
+
+def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx_len: torch.Tensor,
+                     k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
+                     rotary: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None,
+                     softmax_scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
+                     n_splits: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One decode step.  q [B, n_q, d]; caches [B, max_ctx, n_kv, d]; ctx_len int32 [B] counts the valid
+    keys INCLUDING the token appended by this call (k_new/v_new [B, n_kv, d], written at ctx_len-1).
+    rotary = (cos, sin, position_ids[B]) rotates q and k_new inside the kernels."""
+    _need_cuda(q, k_cache, v_cache, ctx_len)
+    B, nq, d = q.shape
+    assert q.is_contiguous() and k_cache.dim() == 4 and k_cache.shape == v_cache.shape
+    assert k_cache.stride() == v_cache.stride() and k_cache.stride(3) == 1
+    assert ctx_len.dtype == torch.int32 and ctx_len.numel() == B
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if workspace is None:
+        workspace = decode_workspace(B, nq, d, k_cache.shape[1], q.device)
+    if out is None:
+        out = torch.empty_like(q)
+    a = MiDecodeArgs()
+    a.q, a.k_cache, a.v_cache, a.o, a.ctx_len = ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), ptr(ctx_len)
+    if k_new is not None:
+        assert k_new.is_contiguous() and v_new.is_contiguous() and k_new.shape == (B, k_cache.shape[2], d)
+        a.k_new, a.v_new = ptr(k_new), ptr(v_new)
+    if rotary is not None:
+        cos, sin, pos = rotary
+        assert cos.dtype == q.dtype and cos.is_contiguous() and sin.is_contiguous() and cos.shape[1] == d
+        assert pos.dtype == torch.int64 and pos.numel() == B and pos.is_contiguous()
+        a.rotary_cos, a.rotary_sin, a.position_ids = ptr(cos), ptr(sin), ptr(pos)
+        a.rotary_table_rows = cos.shape[0]
+    a.batch, a.max_ctx, a.n_q_heads, a.n_kv_heads, a.head_dim = B, k_cache.shape[1], nq, k_cache.shape[2], d
+    a.dtype = dtype_code(q.dtype)
+    a.cache_stride_batch, a.cache_stride_token, a.cache_stride_head = k_cache.stride(0), k_cache.stride(1), k_cache.stride(2)
+    a.softmax_scale = float(softmax_scale)
+    a.n_splits = int(n_splits)
+    a.workspace, a.workspace_bytes = ptr(workspace), workspace.numel() * 4
+    a.stream = stream_ptr()
+    check(_lib.load().mi_attn_decode(ctypes.byref(a)), "mi_attn_decode")
+    return out

@@ -1,0 +1,76 @@
+"""Helpers shared by the attention GPU tests: seeded inputs, layout conversion, oracle evaluation."""
+
+import math
+
+import torch
+
+import oracle
+
+
+def make_cu(b, s, cuts=()):
+    """int32 cumulative lengths containing every multiple of s plus the given extra cut points."""
+    return torch.tensor(sorted(set(i * s for i in range(b + 1)) | set(cuts)), dtype=torch.int32)
+
+
+def random_docs_cu(total, lo, hi, seed):
+    """Document lengths uniform in [lo, hi], last one truncated so the lengths sum to `total`."""
+    g = torch.Generator().manual_seed(seed)
+    cu = [0]
+    while cu[-1] < total:
+        n = int(torch.randint(lo, hi + 1, (1,), generator=g))
+        cu.append(min(total, cu[-1] + n))
+    return torch.tensor(cu, dtype=torch.int32)
+
+
+def position_ids_from_cu(cu, total):
+    pos = torch.zeros(total, dtype=torch.int64)
+    for a, b in zip(cu[:-1].tolist(), cu[1:].tolist()):
+        pos[a:b] = torch.arange(b - a)
+    return pos
+
+
+def make_qkv(b, s, nq, nkv, d, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b * s, nq, d, generator=g).to(dtype)
+    k = torch.randn(b * s, nkv, d, generator=g).to(dtype)
+    v = torch.randn(b * s, nkv, d, generator=g).to(dtype)
+    do = torch.randn(b * s, nq, d, generator=g).to(dtype)
+    return q, k, v, do
+
+
+def to_sbnd(x, b, s):
+    return x.view(b, s, x.shape[1], x.shape[2]).permute(1, 0, 2, 3)
+
+
+def from_bn_s_d(o, b, n):
+    # [(b n), s, d] -> [(b s), n, d]
+    s, d = o.shape[1], o.shape[2]
+    return o.view(b, n, s, d).permute(0, 2, 1, 3).reshape(b * s, n, d)
+
+
+def oracle_attention(q, k, v, cu, b, s, causal, scale, dtype=torch.float32, do=None, softmax_in_fp32=True):
+    """Runs the oracle on token-major tensors; returns o (and dq, dk, dv when `do` is given) in token layout."""
+    nq, nkv = q.shape[1], k.shape[1]
+    qq, kk, vv = (t.to(dtype).clone().requires_grad_(do is not None) for t in (q, k, v))
+    out = oracle.multi_head_attention(
+        to_sbnd(qq, b, s), oracle.repeat_kv(to_sbnd(kk, b, s), nq // nkv), oracle.repeat_kv(to_sbnd(vv, b, s), nq // nkv),
+        cu, causal, scale, softmax_in_fp32=softmax_in_fp32)
+    o = from_bn_s_d(out, b, nq)
+    if do is None:
+        return o.detach()
+    o.backward(do.to(dtype))
+    return o.detach(), qq.grad, kk.grad, vv.grad
+
+
+def rows_reference(q, k, v, lo_hi, rows, head, kv_head, scale):
+    """fp64 attention of selected query rows of one head against keys [lo, hi) per row (size-independent check)."""
+    outs = []
+    for r in rows:
+        lo, hi = lo_hi(r)
+        sc = (k[lo:hi, kv_head].double() @ q[r, head].double()) * scale
+        p = torch.softmax(sc, 0)
+        outs.append(p @ v[lo:hi, kv_head].double())
+    return torch.stack(outs)
+
+
+DEFAULT_SCALE = lambda d: 1.0 / math.sqrt(d)  # noqa: E731

@@ -1,0 +1,161 @@
+"""GPU parity of the attention core (forward, backward, masks, GQA, fused rotary) against the CPU
+oracle, called through the C ABI."""
+
+import math
+
+import pytest
+import torch
+
+import oracle
+from scaling_amd import ops
+from tests import attn_utils as U
+from tests.golden import known_answers as KA
+from tests.parity import check
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+# (batch, seq, n_q, n_kv, head_dim, causal, extra cut points)
+CASES = [
+    (2, 64, 4, 4, 32, True, (32,)),            # the reference's flash-vs-torch test shape (cu = [0,32,64,128])
+    (2, 64, 4, 2, 32, False, (32,)),           # ... its GQA variant, bidirectional
+    (2, 128, 4, 4, 64, True, ()),              # config 1 attention shape
+    (1, 200, 2, 1, 64, True, (3, 77, 78, 150)),  # ragged: seq not a multiple of any tile, tiny documents
+    (2, 256, 8, 2, 128, True, (100, 300, 301)),
+    (1, 512, 4, 4, 128, False, (130,)),
+    (1, 384, 6, 3, 96, True, (129,)),
+    (3, 1, 2, 2, 64, True, ()),                # one token per sequence
+]
+
+
+@pytest.mark.parametrize("b,s,nq,nkv,d,causal,cuts", CASES)
+def test_attention_fwd_bwd_parity(b, s, nq, nkv, d, causal, cuts):
+    print(f"case attn b={b} s={s} nq={nq} nkv={nkv} d={d} causal={causal} cuts={cuts}", flush=True)
+    q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=b * 1000 + s + d)
+    cu = U.make_cu(b, s, cuts)
+    scale = 1.0 / math.sqrt(d)
+    ref = U.oracle_attention(q, k, v, cu, b, s, causal, scale, torch.float32, do)
+    ref_o = U.oracle_attention(q, k, v, cu, b, s, causal, scale, torch.bfloat16, do)
+
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o = ops.attention(qg, kg, vg, cu.to(DEV), None, causal, scale)
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    check("attn.o", o, ref[0], ref_o[0])
+    check("attn.dq", qg.grad, ref[1], ref_o[1])
+    check("attn.dk", kg.grad, ref[2], ref_o[2])
+    check("attn.dv", vg.grad, ref[3], ref_o[3])
+
+
+def test_attention_mask_is_bit_exact_on_reference_known_answers():
+    """q = k = 0 makes the softmax uniform over the allowed keys; with one-hot values the output row is
+    1/count on exactly the allowed key positions, which exposes the kernel's mask predicate."""
+    s, b = KA.MASK_SEQ_LEN, 3
+    cu = torch.tensor(KA.MASK_CU_SEQLENS, dtype=torch.int32)
+    d = 32
+    q = torch.zeros(b * s, 1, d, dtype=torch.bfloat16)
+    v = torch.zeros(b * s, 1, d, dtype=torch.bfloat16)
+    for t in range(b * s):
+        v[t, 0, t % s] = 1.0
+    for causal, allowed in ((True, KA.MASK_ALLOWED_CAUSAL), (False, KA.MASK_ALLOWED_BIDIRECTIONAL)):
+        o, _ = ops.attention_forward(q.to(DEV), q.to(DEV), v.to(DEV), cu.to(DEV), None, causal, 1.0)
+        got = (o.float().cpu().view(b, s, d)[:, :, :s] > 0)
+        assert torch.equal(got, torch.tensor(allowed, dtype=torch.bool))
+        assert torch.equal(~got.unsqueeze(1), oracle.cumulative_seq_lengths_to_dense_attention_mask(cu, s, causal))
+        assert not bool((o.float().cpu().view(b, s, d)[:, :, s:] != 0).any())
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_attention_mask_random_documents_bit_exact(seed):
+    g = torch.Generator().manual_seed(seed)
+    b, s, d = 2, 96, 96
+    cuts = sorted(set(int(x) for x in torch.randint(1, b * s, (7,), generator=g)))
+    cu = U.make_cu(b, s, cuts)
+    q = torch.zeros(b * s, 2, d, dtype=torch.bfloat16)
+    v = torch.zeros(b * s, 2, d, dtype=torch.bfloat16)
+    for t in range(b * s):
+        v[t, :, t % s] = 1.0
+    for causal in (True, False):
+        o, _ = ops.attention_forward(q.to(DEV), q.to(DEV), v.to(DEV), cu.to(DEV), None, causal, 1.0)
+        got = o.float().cpu().view(b, s, 2, d) > 0
+        want = ~oracle.cumulative_seq_lengths_to_dense_attention_mask(cu, s, causal)   # [b,1,s,s]
+        assert torch.equal(got[:, :, 0, :], want[:, 0]) and torch.equal(got[:, :, 1, :], want[:, 0])
+
+
+def test_attention_fused_rotary_matches_separate_rotary():
+    b, s, nq, nkv, d = 2, 192, 4, 2, 128
+    q, k, v, _ = U.make_qkv(b, s, nq, nkv, d, seed=5)
+    cu = U.make_cu(b, s, (50, 250))
+    pos = U.position_ids_from_cu(cu, b * s)
+    tabs = oracle.rotary_tables(d, s, 500000, torch.bfloat16)
+    cos, sin = tabs.cos.to(DEV), tabs.sin.to(DEV)
+    qd, kd, vd, cud, posd = q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), pos.to(DEV)
+    # oracle: rotary (table values as stored, fp32 arithmetic) then attention, everything fp32
+    hi = oracle.RotaryTables(tabs.cos.float(), tabs.sin.float(), d)
+    ids = pos.view(b, s).transpose(0, 1)
+    qr, kr = oracle.apply_rotary(U.to_sbnd(q.float(), b, s), U.to_sbnd(k.float(), b, s), hi, ids, ids)
+    ref = U.from_bn_s_d(oracle.multi_head_attention(qr, oracle.repeat_kv(kr, 2), oracle.repeat_kv(U.to_sbnd(v.float(), b, s), 2),
+                                                    cu, True, 1 / math.sqrt(d), softmax_in_fp32=True), b, nq)
+    qo, ko = oracle.apply_rotary(U.to_sbnd(q, b, s), U.to_sbnd(k, b, s), tabs, ids, ids)
+    ref_o = U.from_bn_s_d(oracle.multi_head_attention(qo, oracle.repeat_kv(ko, 2), oracle.repeat_kv(U.to_sbnd(v, b, s), 2),
+                                                      cu, True, 1 / math.sqrt(d), softmax_in_fp32=True), b, nq)
+    fused, _ = ops.attention_forward(qd, kd, vd, cud, None, True, None, rotary=(cos, sin, posd, posd))
+    q2 = ops.rotary_embedding(qd, cos, sin, posd)
+    k2 = ops.rotary_embedding(kd, cos, sin, posd)
+    sep, _ = ops.attention_forward(q2, k2, vd, cud, None, True, None)
+    torch.cuda.synchronize()
+    check("attn.fused_rotary", fused, ref, ref_o)
+    check("attn.separate_rotary", sep, ref, ref_o)
+    # same rounding points (rotate in fp32, round once to bf16); only fma contraction may differ
+    diff = (fused.float() - sep.float()).abs()
+    assert float(diff.max()) <= 2e-2 and float((diff > 0).float().mean()) < 0.02
+
+
+def test_attention_is_bit_reproducible_and_gqa_equals_repeated_heads():
+    b, s, nq, nkv, d = 1, 320, 8, 2, 128
+    q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=9)
+    cu = U.make_cu(b, s, (100,)).to(DEV)
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    o1, lse1 = ops.attention_forward(qd, kd, vd, cu)
+    o2, lse2 = ops.attention_forward(qd, kd, vd, cu)
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2)
+    g1 = ops.attention_backward(dod, qd, kd, vd, o1, lse1, cu)
+    g2 = ops.attention_backward(dod, qd, kd, vd, o1, lse1, cu)
+    assert all(torch.equal(a, c) for a, c in zip(g1, g2))
+    # explicit repeat_interleave of the kv heads gives the same output bits
+    kr = torch.repeat_interleave(kd, 4, dim=1)
+    vr = torch.repeat_interleave(vd, 4, dim=1)
+    o3, _ = ops.attention_forward(qd, kr, vr, cu)
+    assert torch.equal(o1, o3)
+    # log-sum-exp against the closed form on a few rows
+    lse_ref = []
+    for t in (0, 99, 100, 319):
+        lo = 0 if t < 100 else 100
+        sc = (k[lo:t + 1, 0].double() @ q[t, 1].double()) / math.sqrt(d)
+        lse_ref.append(torch.logsumexp(sc, 0))
+    got = lse1[1, [0, 99, 100, 319]].double().cpu()
+    assert torch.allclose(got, torch.stack(lse_ref), atol=2e-3)
+
+
+def test_attention_strided_views_of_fused_qkv():
+    """q, k, v as per-head slices of one fused projection output ([tokens, heads, 3*d]), as the
+    reference's qkv_in_one layout produces them."""
+    b, s, n, d = 2, 96, 4, 64
+    g = torch.Generator().manual_seed(13)
+    qkv = torch.randn(b * s, n, 3 * d, generator=g).bfloat16()
+    cu = U.make_cu(b, s)
+    ref = U.oracle_attention(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], cu, b, s, True, 1 / math.sqrt(d))
+    ref_o = U.oracle_attention(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], cu, b, s, True, 1 / math.sqrt(d), torch.bfloat16)
+    qd = qkv.to(DEV)
+    o, _ = ops.attention_forward(qd[..., :d], qd[..., d:2 * d], qd[..., 2 * d:], cu.to(DEV))
+    check("attn.o(strided)", o, ref, ref_o)
+
+
+def test_attention_rejects_unsupported_input():
+    q = torch.zeros(8, 2, 80, dtype=torch.bfloat16, device=DEV)
+    cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        ops.attention_forward(q, q, q, cu)
+    qf = torch.zeros(8, 2, 64, dtype=torch.float32, device=DEV)
+    with pytest.raises(RuntimeError, match="bf16"):
+        ops.attention_forward(qf, qf, qf, cu)

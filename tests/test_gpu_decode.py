@@ -1,0 +1,107 @@
+"""GPU parity of the KV-cache decode kernel against the CPU oracle (per-sequence batch-1 reference
+semantics: the step output equals the last row of full causal attention over the cached positions)."""
+
+import math
+
+import pytest
+import torch
+
+import oracle
+from scaling_amd import ops
+from tests.parity import check
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _oracle_decode(q, kc, vc, ctx, scale, dtype):
+    """q [B,nq,d], caches [B,max,nkv,d] (already containing the new token); one reference call per sequence."""
+    B, nq, d = q.shape
+    nkv = kc.shape[2]
+    outs = []
+    for b in range(B):
+        n = int(ctx[b])
+        qq = q[b].to(dtype).view(1, 1, nq, d)                                   # [s_q=1, b=1, n, d]
+        kk = oracle.repeat_kv(kc[b, :n].to(dtype).unsqueeze(1), nq // nkv)      # [s_k, 1, nq, d]
+        vv = oracle.repeat_kv(vc[b, :n].to(dtype).unsqueeze(1), nq // nkv)
+        o = oracle.multi_head_attention(qq, kk, vv, torch.tensor([0, 1], dtype=torch.int32), True, scale,
+                                        softmax_in_fp32=True)                   # [(1 nq), 1, d]
+        outs.append(o.view(nq, d))
+    return torch.stack(outs)
+
+
+@pytest.mark.parametrize("B,nq,nkv,d,max_ctx,lens", [
+    (3, 8, 2, 128, 300, [1, 137, 300]),
+    (2, 4, 4, 64, 128, [128, 5]),
+    (4, 32, 8, 128, 1100, [1024, 1025, 33, 1100]),
+    (1, 16, 1, 128, 64, [64]),
+])
+@pytest.mark.parametrize("n_splits", [0, 1, 3])
+def test_decode_parity(B, nq, nkv, d, max_ctx, lens, n_splits):
+    print(f"case decode B={B} nq={nq} nkv={nkv} d={d} max_ctx={max_ctx} lens={lens} splits={n_splits}", flush=True)
+    g = torch.Generator().manual_seed(B * 31 + d)
+    q = torch.randn(B, nq, d, generator=g).bfloat16()
+    kc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16()
+    vc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16()
+    ctx = torch.tensor(lens, dtype=torch.int32)
+    scale = 1 / math.sqrt(d)
+    ref = _oracle_decode(q, kc, vc, ctx, scale, torch.float32)
+    ref_o = _oracle_decode(q, kc, vc, ctx, scale, torch.bfloat16)
+    out = ops.decode_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), ctx.to(DEV), softmax_scale=scale, n_splits=n_splits)
+    torch.cuda.synchronize()
+    check("decode.o", out, ref, ref_o)
+
+
+def test_decode_append_and_fused_rotary():
+    B, nq, nkv, d, max_ctx = 3, 8, 2, 128, 96
+    g = torch.Generator().manual_seed(77)
+    lens = [10, 96, 1]                       # lengths INCLUDING the appended token
+    q = torch.randn(B, nq, d, generator=g).bfloat16()
+    k_new = torch.randn(B, nkv, d, generator=g).bfloat16()
+    v_new = torch.randn(B, nkv, d, generator=g).bfloat16()
+    kc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16()
+    vc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16()
+    ctx = torch.tensor(lens, dtype=torch.int32)
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int64)
+    tabs = oracle.rotary_tables(d, max_ctx, 500000, torch.bfloat16)
+    hi = oracle.RotaryTables(tabs.cos.float(), tabs.sin.float(), d)
+    # reference: rotate the new q/k at their positions, append, attend
+    qr, kr = oracle.apply_rotary(q.float().unsqueeze(0), k_new.float().unsqueeze(0), hi, pos.view(1, B), pos.view(1, B))
+    qr, kr = qr[0].bfloat16(), kr[0].bfloat16()     # what is stored / consumed after one rounding
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    for b in range(B):
+        kc_ref[b, lens[b] - 1] = kr[b]
+        vc_ref[b, lens[b] - 1] = v_new[b]
+    scale = 1 / math.sqrt(d)
+    ref = _oracle_decode(qr, kc_ref, vc_ref, ctx, scale, torch.float32)
+    ref_o = _oracle_decode(qr, kc_ref, vc_ref, ctx, scale, torch.bfloat16)
+    kcd, vcd = kc.to(DEV), vc.to(DEV)
+    out = ops.decode_attention(q.to(DEV), kcd, vcd, ctx.to(DEV), k_new.to(DEV), v_new.to(DEV),
+                               rotary=(tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV)), softmax_scale=scale)
+    torch.cuda.synchronize()
+    check("decode.o(append+rotary)", out, ref, ref_o)
+    # the cache was updated in place: only the appended rows changed, and they hold the rotated key
+    for b in range(B):
+        kd = (kcd[b, lens[b] - 1].float().cpu() - kr[b].float()).abs()
+        assert float(kd.max()) <= 2e-2 and float((kd > 0).float().mean()) < 0.02
+        assert torch.equal(vcd[b, lens[b] - 1].cpu(), v_new[b])
+    mask = torch.ones(B, max_ctx, dtype=torch.bool)
+    for b in range(B):
+        mask[b, lens[b] - 1] = False
+    assert torch.equal(kcd.cpu()[mask], kc[mask]) and torch.equal(vcd.cpu()[mask], vc[mask])
+
+
+def test_decode_equals_last_row_of_prefill_kernel():
+    """Cached == uncached: the decode kernel agrees with the last query row of the forward kernel."""
+    nq, nkv, d, n = 8, 2, 128, 333
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(n, nq, d, generator=g).bfloat16().to(DEV)
+    k = torch.randn(n, nkv, d, generator=g).bfloat16().to(DEV)
+    v = torch.randn(n, nkv, d, generator=g).bfloat16().to(DEV)
+    cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
+    full, _ = ops.attention_forward(q, k, v, cu)
+    out = ops.decode_attention(q[n - 1:n].contiguous(), k.unsqueeze(0), v.unsqueeze(0),
+                               torch.tensor([n], dtype=torch.int32, device=DEV))
+    torch.cuda.synchronize()
+    diff = (out[0].float() - full[n - 1].float()).abs()
+    assert float(diff.max()) <= 1.6e-2

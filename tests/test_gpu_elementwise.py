@@ -1,0 +1,132 @@
+"""GPU parity of the bandwidth-bound kernels (RMSNorm, SwiGLU, rotary) against the CPU oracle,
+called through the C ABI."""
+
+import pytest
+import torch
+
+import oracle
+from scaling_amd import ops
+from tests.parity import check
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _rand(gen, *shape, dtype=torch.bfloat16, scale=1.0):
+    return (torch.randn(*shape, generator=gen) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("rows,hidden", [(2 * 128, 256), (37, 128), (1024, 4096), (19, 8192), (5, 1000 * 8), (64, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_parity(rows, hidden, dtype):
+    print(f"case rmsnorm rows={rows} hidden={hidden} dtype={dtype}", flush=True)
+    g = torch.Generator().manual_seed(rows * 7 + hidden)
+    x = _rand(g, rows, hidden, dtype=dtype)
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    dy = _rand(g, rows, hidden, dtype=dtype)
+    xr = x.float().requires_grad_()
+    wr = w.float().requires_grad_()
+    ref = oracle.rms_norm(xr, wr, 1e-5)
+    ref.backward(dy.float())
+    xo = x.clone().requires_grad_()
+    wo = w.clone().requires_grad_()
+    ref_o = oracle.rms_norm(xo, wo, 1e-5)          # the reference's own operation order in `dtype`
+    ref_o.backward(dy)
+
+    xg = x.to(DEV).requires_grad_()
+    wg = w.to(DEV).requires_grad_()
+    y = ops.rms_norm(xg, wg, 1e-5)
+    y.backward(dy.to(DEV))
+    torch.cuda.synchronize()
+    tol = dict(max_abs_tol=2e-2, mean_rel_tol=1e-3) if dtype == torch.bfloat16 else dict(max_abs_tol=1e-4, mean_rel_tol=1e-5)
+    check("rmsnorm.y", y, ref, ref_o, **tol)
+    check("rmsnorm.dx", xg.grad, xr.grad, xo.grad, **tol)
+    check("rmsnorm.dw", wg.grad, wr.grad, wo.grad, **tol)
+
+
+def test_rmsnorm_bwd_is_bit_reproducible():
+    g = torch.Generator().manual_seed(3)
+    x, w, dy = _rand(g, 3000, 4096).to(DEV), torch.ones(4096, dtype=torch.bfloat16, device=DEV), _rand(g, 3000, 4096).to(DEV)
+    a = ops.rms_norm_backward(x, w, dy, 1e-5)
+    b = ops.rms_norm_backward(x, w, dy, 1e-5)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+@pytest.mark.parametrize("shape", [(2, 128, 688), (3, 7, 5), (4, 1000, 14336), (1, 1, 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_swiglu_parity(shape, dtype):
+    print(f"case swiglu shape={shape} dtype={dtype}", flush=True)
+    g = torch.Generator().manual_seed(sum(shape))
+    a, gate, do = (_rand(g, *shape, dtype=dtype) for _ in range(3))
+    ar, gr = a.float().requires_grad_(), gate.float().requires_grad_()
+    ref = oracle.swiglu(ar, gr)
+    ref.backward(do.float())
+    ao, go = a.clone().requires_grad_(), gate.clone().requires_grad_()
+    ref_o = oracle.swiglu(ao, go)
+    ref_o.backward(do)
+    ag, gg = a.to(DEV).requires_grad_(), gate.to(DEV).requires_grad_()
+    out = ops.swiglu(ag, gg)
+    out.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    tol = dict(max_abs_tol=1e-4, mean_rel_tol=1e-5) if dtype == torch.float32 else {}
+    check("swiglu.out", out, ref, ref_o, **tol)
+    check("swiglu.da", ag.grad, ar.grad, ao.grad, **tol)
+    check("swiglu.dgate", gg.grad, gr.grad, go.grad, **tol)
+    # closed-form gradient of the oracle agrees with what the kernel returns
+    da_cf, dg_cf = oracle.swiglu_grad(a.float(), gate.float(), do.float())
+    check("swiglu.da(closed form)", ag.grad, da_cf, ao.grad, **tol)
+
+
+@pytest.mark.parametrize("seq,batch,heads,dim,rot", [(17, 2, 4, 16, 16), (10, 7, 1, 2, 2), (10, 2, 2, 8, 8),
+                                                      (64, 2, 8, 128, 128), (33, 1, 3, 64, 32), (16, 2, 2, 128, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("with_ids", [True, False])
+def test_rotary_parity(seq, batch, heads, dim, rot, dtype, with_ids):
+    print(f"case rotary s={seq} b={batch} n={heads} d={dim} rot={rot} {dtype} ids={with_ids}", flush=True)
+    g = torch.Generator().manual_seed(seq + dim)
+    tabs = oracle.rotary_tables(rot, seq, 10000, dtype)
+    q = _rand(g, seq, batch, heads, dim, dtype=dtype)
+    if with_ids:
+        ids = torch.randint(0, seq, (seq, batch), generator=g)
+    else:
+        ids = None
+    hi = oracle.RotaryTables(tabs.cos.float(), tabs.sin.float(), rot)   # same (rounded) table values, fp32 arithmetic
+    ref, _ = oracle.apply_rotary(q.float(), q.float(), hi, ids, ids)
+    ref_o, _ = oracle.apply_rotary(q, q, tabs, ids, ids)
+    # kernel layout: tokens = (b s)
+    x = q.permute(1, 0, 2, 3).reshape(batch * seq, heads, dim).contiguous().to(DEV)
+    pid = None if ids is None else ids.transpose(0, 1).reshape(-1).contiguous().to(DEV)
+    out = ops.rotary_embedding(x, tabs.cos.to(DEV), tabs.sin.to(DEV), pid, seq_len_for_null_ids=seq)
+    torch.cuda.synchronize()
+    got = out.view(batch, seq, heads, dim).permute(1, 0, 2, 3)
+    tol = dict(max_abs_tol=1e-5, mean_rel_tol=1e-6) if dtype == torch.float32 else {}
+    check("rotary.out", got, ref, ref_o, **tol)
+    if rot < dim:
+        assert torch.equal(got[..., rot:].cpu(), q[..., rot:])
+
+
+def test_rotary_reference_invariants_and_backward():
+    g = torch.Generator().manual_seed(11)
+    seq, batch, heads, dim = 17, 2, 4, 16
+    tabs = oracle.rotary_tables(dim, seq, 10000, torch.bfloat16)
+    cos, sin = tabs.cos.to(DEV), tabs.sin.to(DEV)
+    x = _rand(g, batch * seq, heads, dim).to(DEV)
+    ids = torch.arange(seq).repeat(batch).to(DEV)
+    a = ops.rotary_embedding(x, cos, sin, None, seq_len_for_null_ids=seq)
+    b = ops.rotary_embedding(x, cos, sin, ids)
+    assert torch.equal(a, b)                       # arange ids == no ids
+    xs = x.view(batch, seq, heads, dim)[:, 1:].reshape(-1, heads, dim)
+    ids_s = ids.view(batch, seq)[:, 1:].reshape(-1).contiguous()
+    c = ops.rotary_embedding(xs, cos, sin, ids_s)
+    assert torch.equal(c.view(batch, seq - 1, heads, dim), a.view(batch, seq, heads, dim)[:, 1:])
+    # backward == rotation by the negative angle == autograd of the oracle
+    xr = x.float().cpu().view(batch, seq, heads, dim).permute(1, 0, 2, 3).clone().requires_grad_()
+    hi = oracle.RotaryTables(tabs.cos.float(), tabs.sin.float(), dim)
+    out_r, _ = oracle.apply_rotary(xr, xr.detach(), hi)
+    go = _rand(g, seq, batch, heads, dim)
+    out_r.backward(go.float())
+    xg = x.clone().requires_grad_()
+    out = ops.rotary_embedding(xg, cos, sin, ids)
+    out.backward(go.permute(1, 0, 2, 3).reshape(batch * seq, heads, dim).contiguous().to(DEV))
+    torch.cuda.synchronize()
+    check("rotary.dx", xg.grad.view(batch, seq, heads, dim).permute(1, 0, 2, 3), xr.grad)
