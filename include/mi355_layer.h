@@ -118,6 +118,9 @@ int mi_rotary(const void* x, void* out, const void* cos, const void* sin, const 
  * Algorithmic work: 4 * head_dim * n_q_heads * P flop forward, 10 * head_dim * n_q_heads * P backward,
  * P = number of allowed (query, key) pairs per head.
  * ------------------------------------------------------------------------------------------ */
+#define MI_ATTN_QG1 1   /* forward: one group of 32 queries per wavefront (128 per workgroup) */
+#define MI_ATTN_QG2 2   /* forward: two groups of 32 queries per wavefront (256 per workgroup) */
+
 typedef struct mi_attn_args {
     const void* q;
     const void* k;
@@ -139,7 +142,7 @@ typedef struct mi_attn_args {
     int64_t v_stride_token, v_stride_head;
     int64_t o_stride_token, o_stride_head;
     float softmax_scale;
-    int32_t reserved0;
+    int32_t flags;                 /* 0 = library chooses; MI_ATTN_QG1 / MI_ATTN_QG2 pin the forward tiling */
     /* optional fused rotary */
     const void* rotary_cos;
     const void* rotary_sin;

@@ -36,7 +36,7 @@ class MiAttnArgs(Structure):
         ("k_stride_token", c_int64), ("k_stride_head", c_int64),
         ("v_stride_token", c_int64), ("v_stride_head", c_int64),
         ("o_stride_token", c_int64), ("o_stride_head", c_int64),
-        ("softmax_scale", c_float), ("reserved0", c_int32),
+        ("softmax_scale", c_float), ("flags", c_int32),
         ("rotary_cos", c_void_p), ("rotary_sin", c_void_p),
         ("position_ids_q", c_void_p), ("position_ids_k", c_void_p),
         ("rotary_table_rows", c_int64),

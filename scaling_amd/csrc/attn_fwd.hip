@@ -342,7 +342,9 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     // two query groups per wavefront halve the LDS traffic per MFMA; worth it once the grid still
     // fills the chip
     const int64_t blocks_qg2 = (((int64_t)p.total_q + 255) / 256) * p.nq;
-    const int qg = blocks_qg2 >= 512 ? 2 : 1;
+    int qg = blocks_qg2 >= 512 ? 2 : 1;
+    if (a->flags & MI_ATTN_QG1) qg = 1;
+    if (a->flags & MI_ATTN_QG2) qg = 2;
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
         case 32: return launch_d<32>(p, rot, qg, st);

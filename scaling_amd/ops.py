@@ -161,8 +161,9 @@ def rotary_embedding(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
 # ------------------------------------------------------------------------------------------------
 # attention core
 # ------------------------------------------------------------------------------------------------
-def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None) -> MiAttnArgs:
+def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, flags=0) -> MiAttnArgs:
     a = MiAttnArgs()
+    a.flags = int(flags)
     a.q, a.k, a.v, a.o, a.lse = ptr(q), ptr(k), ptr(v), ptr(o), ptr(lse)
     a.cu_seqlens_q, a.cu_seqlens_k = ptr(cu_q), ptr(cu_k)
     a.n_docs = cu_q.numel() - 1
@@ -194,8 +195,10 @@ def _check_qkv(q, k, v, cu_q, cu_k):
         assert cu_k.dtype == torch.int32 and cu_k.is_contiguous() and cu_k.numel() == cu_q.numel()
 
 
-def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None, rotary=None):
-    """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens])."""
+def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None, rotary=None, flags=0):
+    """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens]).
+
+    flags: 0 lets the library pick the tiling; 1 / 2 pin one / two query groups per wavefront."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
@@ -206,7 +209,7 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
         assert pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0]
     o = torch.empty((q.shape[0], q.shape[1], q.shape[2]), dtype=q.dtype, device=q.device)
     lse = torch.empty((q.shape[1], q.shape[0]), dtype=torch.float32, device=q.device)
-    a = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary)
+    a = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary, flags)
     check(_lib.load().mi_attn_fwd(ctypes.byref(a)), "mi_attn_fwd")
     return o, lse
 

@@ -159,3 +159,78 @@ def test_attention_rejects_unsupported_input():
     qf = torch.zeros(8, 2, 64, dtype=torch.float32, device=DEV)
     with pytest.raises(RuntimeError, match="bf16"):
         ops.attention_forward(qf, qf, qf, cu)
+
+
+@pytest.mark.parametrize("flags", [1, 2])
+@pytest.mark.parametrize("rot", [False, True])
+def test_attention_forward_tilings_agree_with_oracle(flags, rot):
+    """Both forward tilings (one / two query groups per wavefront), with and without fused rotary."""
+    b, s, nq, nkv, d = 1, 700, 4, 2, 128
+    q, k, v, _ = U.make_qkv(b, s, nq, nkv, d, seed=21)
+    cu = U.make_cu(b, s, (130, 131, 555))
+    pos = U.position_ids_from_cu(cu, b * s)
+    tabs = oracle.rotary_tables(d, s, 500000, torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    if rot:
+        ids = pos.view(b, s).transpose(0, 1)
+        hi = oracle.RotaryTables(tabs.cos.float(), tabs.sin.float(), d)
+        qr, kr = oracle.apply_rotary(U.to_sbnd(q.float(), b, s), U.to_sbnd(k.float(), b, s), hi, ids, ids)
+        qr = qr.permute(1, 0, 2, 3).reshape(b * s, nq, d).bfloat16()
+        kr = kr.permute(1, 0, 2, 3).reshape(b * s, nkv, d).bfloat16()
+    else:
+        qr, kr = q, k
+    ref = U.oracle_attention(qr, kr, v, cu, b, s, True, scale)
+    ref_o = U.oracle_attention(qr, kr, v, cu, b, s, True, scale, torch.bfloat16)
+    rotary = (tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV), pos.to(DEV)) if rot else None
+    o, _ = ops.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), None, True, scale, rotary=rotary, flags=flags)
+    torch.cuda.synchronize()
+    check(f"attn.o(flags={flags},rot={rot})", o, ref, ref_o)
+
+
+def test_attention_medium_multi_tile_backward():
+    """Several query / key blocks per head and a GQA group of 4: exercises every loop of the backward."""
+    b, s, nq, nkv, d = 1, 1024, 8, 2, 128
+    q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=33)
+    cu = U.make_cu(b, s, (300, 700))
+    scale = 1 / math.sqrt(d)
+    ref = U.oracle_attention(q, k, v, cu, b, s, True, scale, torch.float32, do)
+    ref_o = U.oracle_attention(q, k, v, cu, b, s, True, scale, torch.bfloat16, do)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale)
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    check("attn1k.o", o, ref[0], ref_o[0])
+    check("attn1k.dq", qg.grad, ref[1], ref_o[1])
+    check("attn1k.dk", kg.grad, ref[2], ref_o[2])
+    check("attn1k.dv", vg.grad, ref[3], ref_o[3])
+
+
+@pytest.mark.parametrize("name,b,s,nq,nkv,docs", [("config2", 4, 2048, 32, 32, False), ("config3", 1, 8192, 32, 8, True)])
+def test_attention_full_size_properties(name, b, s, nq, nkv, docs):
+    """At the benchmark sizes the dense oracle does not fit; check size-independent properties:
+    sampled rows against an fp64 row-wise evaluation, V = ones -> O = ones, and GQA head sharing."""
+    d = 128
+    g = torch.Generator().manual_seed(100 + s)
+    q = torch.randn(b * s, nq, d, generator=g).bfloat16()
+    k = torch.randn(b * s, nkv, d, generator=g).bfloat16()
+    v = torch.randn(b * s, nkv, d, generator=g).bfloat16()
+    cu = U.random_docs_cu(b * s, 256, 2048, seed=7) if docs else U.make_cu(b, s)
+    scale = 1 / math.sqrt(d)
+    qd, kd, vd, cud = q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV)
+    o, lse = ops.attention_forward(qd, kd, vd, cud, None, True, scale)
+    torch.cuda.synchronize()
+    starts = cu.tolist()
+
+    def lo_hi(r):
+        j = max(i for i, c in enumerate(starts) if c <= r)
+        return starts[j], r + 1
+
+    rows = sorted(set([0, 1, 127, 128, 255, 256, b * s - 1] + [int(x) for x in torch.randint(0, b * s, (40,), generator=g)]))
+    for head in (0, nq // 2 + 1, nq - 1):
+        kvh = head // (nq // nkv)
+        ref = U.rows_reference(q, k, v, lo_hi, rows, head, kvh, scale)
+        check(f"{name}.rows.head{head}", o[rows, head], ref.float())
+    ones = torch.ones_like(vd)
+    o1, _ = ops.attention_forward(qd, kd, ones, cud, None, True, scale)
+    assert float((o1.float() - 1).abs().max()) <= 2 ** -7
+    assert bool(torch.isfinite(lse).all())

@@ -24,8 +24,8 @@ def test_rmsnorm_parity(rows, hidden, dtype):
     x = _rand(g, rows, hidden, dtype=dtype)
     w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
     dy = _rand(g, rows, hidden, dtype=dtype)
-    xr = x.float().requires_grad_()
-    wr = w.float().requires_grad_()
+    xr = x.float().clone().requires_grad_()
+    wr = w.float().clone().requires_grad_()
     ref = oracle.rms_norm(xr, wr, 1e-5)
     ref.backward(dy.float())
     xo = x.clone().requires_grad_()
@@ -33,8 +33,8 @@ def test_rmsnorm_parity(rows, hidden, dtype):
     ref_o = oracle.rms_norm(xo, wo, 1e-5)          # the reference's own operation order in `dtype`
     ref_o.backward(dy)
 
-    xg = x.to(DEV).requires_grad_()
-    wg = w.to(DEV).requires_grad_()
+    xg = x.to(DEV).detach().requires_grad_()
+    wg = w.to(DEV).detach().requires_grad_()
     y = ops.rms_norm(xg, wg, 1e-5)
     y.backward(dy.to(DEV))
     torch.cuda.synchronize()
@@ -58,13 +58,13 @@ def test_swiglu_parity(shape, dtype):
     print(f"case swiglu shape={shape} dtype={dtype}", flush=True)
     g = torch.Generator().manual_seed(sum(shape))
     a, gate, do = (_rand(g, *shape, dtype=dtype) for _ in range(3))
-    ar, gr = a.float().requires_grad_(), gate.float().requires_grad_()
+    ar, gr = a.float().clone().requires_grad_(), gate.float().clone().requires_grad_()
     ref = oracle.swiglu(ar, gr)
     ref.backward(do.float())
     ao, go = a.clone().requires_grad_(), gate.clone().requires_grad_()
     ref_o = oracle.swiglu(ao, go)
     ref_o.backward(do)
-    ag, gg = a.to(DEV).requires_grad_(), gate.to(DEV).requires_grad_()
+    ag, gg = a.to(DEV).detach().requires_grad_(), gate.to(DEV).detach().requires_grad_()
     out = ops.swiglu(ag, gg)
     out.backward(do.to(DEV))
     torch.cuda.synchronize()
