@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the transformer-layer hot path on one MI355X.
+
+Headline workload (`config.workload`): attention core forward + backward, GQA 32 query / 8 KV heads,
+head_dim 128, one sequence of 8192 tokens, causal, bf16, fp32 softmax.  One step = one forward and
+one backward pass over synthetic N(0,1) inputs already resident in HBM.  `value` is
+14 * d * n_q * P / time (P = allowed (query, key) pairs per head), i.e. the algorithmic TFLOP/s.
+
+The JSON line also carries
+  roofline      the dominant kernel of the step, timed live with HIP events on the launch stream
+  cpu_baseline  the reference's operation order (CPU oracle, plain torch) timed on the host cores
+                on a bounded sample of the same workload
+  extra         the other quantities of the metric: per-kernel attention times, config-2 / config-3
+                attention, RMSNorm / SwiGLU / rotary GB/s at the config-4 sizes, decode-attention GB/s
+                at the config-5 per-layer shape.
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, vendor figure
+
+
+def causal_pairs(cu):
+    return sum((b - a) * (b - a + 1) // 2 for a, b in zip(cu[:-1], cu[1:]))
+
+
+def time_gpu(fn, steps, warmup):
+    """Average milliseconds per call, measured with events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=False):
+    """Times forward, backward stages and the whole step for one attention workload."""
+    import torch
+    from scaling_amd import ops
+    dev = "cuda"
+    g = torch.Generator().manual_seed(seed)
+    T = b * s
+    q = torch.randn(T, nq, d, generator=g).bfloat16().to(dev)
+    k = torch.randn(T, nkv, d, generator=g).bfloat16().to(dev)
+    v = torch.randn(T, nkv, d, generator=g).bfloat16().to(dev)
+    do = torch.randn(T, nq, d, generator=g).bfloat16().to(dev)
+    cu = torch.tensor(cu_list, dtype=torch.int32, device=dev)
+    scale = 1.0 / math.sqrt(d)
+    pairs = causal_pairs(cu_list)
+    rot = None
+    if rotary:
+        import oracle  # table construction only (not timed)
+        tabs = oracle.rotary_tables(d, s, 500000, torch.bfloat16)
+        pos = torch.zeros(T, dtype=torch.int64)
+        for a_, b_ in zip(cu_list[:-1], cu_list[1:]):
+            pos[a_:b_] = torch.arange(b_ - a_)
+        pos = pos.to(dev)
+        rot = (tabs.cos.to(dev), tabs.sin.to(dev), pos, pos)
+
+    o, lse = ops.attention_forward(q, k, v, cu, None, True, scale)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    ws = torch.empty(nq * T, dtype=torch.float32, device=dev)
+    bufs = (dq, dk, dv, ws)
+
+    def fwd():
+        ops.attention_forward(q, k, v, cu, None, True, scale)
+
+    def fwd_rot():
+        ops.attention_forward(q, k, v, cu, None, True, scale, rotary=rot)
+
+    def bwd(flags=0):
+        ops.attention_backward(do, q, k, v, o, lse, cu, None, True, scale, flags=flags, buffers=bufs)
+
+    def step():
+        fwd()
+        bwd()
+
+    res = {"pairs_per_head": pairs}
+    res["ms_step"] = time_gpu(step, steps, warmup)
+    res["ms_fwd"] = time_gpu(fwd, steps, warmup)
+    res["ms_bwd_delta"] = time_gpu(lambda: bwd(16), steps, 1)
+    res["ms_bwd_dkdv"] = time_gpu(lambda: bwd(32), steps, 1)
+    res["ms_bwd_dq"] = time_gpu(lambda: bwd(64), steps, 1)
+    if rot is not None:
+        res["ms_fwd_fused_rotary"] = time_gpu(fwd_rot, steps, warmup)
+    flops_unit = d * nq * pairs
+    res["tflops_fwd"] = 4 * flops_unit / (res["ms_fwd"] * 1e-3) / 1e12
+    res["tflops_step"] = 14 * flops_unit / (res["ms_step"] * 1e-3) / 1e12
+    res["frac_of_bf16_peak_step"] = res["tflops_step"] / PEAK_BF16_TFLOPS
+    return res
+
+
+def bandwidth_cases(steps, warmup):
+    """RMSNorm / SwiGLU / rotary at the config-4 sizes and decode attention at the config-5 layer shape."""
+    import torch
+    import oracle  # rotary table construction only (not timed)
+    from scaling_amd import ops
+    dev = "cuda"
+    out = {}
+    g = torch.Generator().manual_seed(1)
+    N, H, I = 8192, 4096, 14336
+    x = torch.randn(N, H, generator=g).bfloat16().to(dev)
+    w = torch.ones(H, dtype=torch.bfloat16, device=dev)
+    dy = torch.randn(N, H, generator=g).bfloat16().to(dev)
+    ms = time_gpu(lambda: ops.rms_norm_forward(x, w, 1e-5), steps, warmup)
+    out["rmsnorm_fwd"] = {"ms": ms, "GBs": 2 * N * H * 2 / ms / 1e6}
+    ms = time_gpu(lambda: ops.rms_norm_backward(x, w, dy, 1e-5), steps, warmup)
+    out["rmsnorm_bwd"] = {"ms": ms, "GBs": 3 * N * H * 2 / ms / 1e6}
+    a = torch.randn(N, I, generator=g).bfloat16().to(dev)
+    gate = torch.randn(N, I, generator=g).bfloat16().to(dev)
+    dout = torch.randn(N, I, generator=g).bfloat16().to(dev)
+    ms = time_gpu(lambda: ops.swiglu_forward(a, gate), steps, warmup)
+    out["swiglu_fwd"] = {"ms": ms, "GBs": 3 * N * I * 2 / ms / 1e6}
+    ms = time_gpu(lambda: ops.swiglu_backward(a, gate, dout), steps, warmup)
+    out["swiglu_bwd"] = {"ms": ms, "GBs": 5 * N * I * 2 / ms / 1e6}
+    del a, gate, dout
+    nq, nkv, d = 32, 8, 128
+    qk = torch.randn(N, nq + nkv, d, generator=g).bfloat16().to(dev)
+    tabs = oracle.rotary_tables(d, 8192, 500000, torch.bfloat16)
+    cos, sin = tabs.cos.to(dev), tabs.sin.to(dev)
+    pos = torch.arange(N, dtype=torch.int64, device=dev) % 4096
+    ms = time_gpu(lambda: ops.rotary_embedding(qk, cos, sin, pos), steps, warmup)
+    out["rotary"] = {"ms": ms, "GBs": (2 * N * (nq + nkv) * d * 2 + 8 * N) / ms / 1e6}
+    del qk
+    B, ctx, max_ctx = 32, 4096, 4352
+    kc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16().to(dev)
+    vc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16().to(dev)
+    q1 = torch.randn(B, nq, d, generator=g).bfloat16().to(dev)
+    ctx_len = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    wsd = ops.decode_workspace(B, nq, d, max_ctx, dev)
+    od = torch.empty_like(q1)
+    ms = time_gpu(lambda: ops.decode_attention(q1, kc, vc, ctx_len, workspace=wsd, out=od), steps, warmup)
+    out["decode_attention"] = {"ms": ms, "GBs": 2 * B * ctx * nkv * d * 2 / ms / 1e6, "batch": B, "ctx": ctx}
+    for v_ in out.values():
+        v_["frac_of_hbm_peak"] = v_["GBs"] / PEAK_HBM_GBS
+    return out
+
+
+def cpu_baseline(seconds_budget=25.0):
+    """The reference's operation order (CPU oracle) on a bounded sample of the headline workload:
+    same head_dim / GQA ratio / causal mask / bf16 with fp32 softmax, fewer heads and a shorter sequence."""
+    import torch
+    import oracle
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    s, nq, nkv, d = 2048, 4, 1, 128
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(s, 1, nq, d, generator=g).bfloat16().requires_grad_()
+    k = torch.randn(s, 1, nkv, d, generator=g).bfloat16().requires_grad_()
+    v = torch.randn(s, 1, nkv, d, generator=g).bfloat16().requires_grad_()
+    do = torch.randn(nq, s, d, generator=g).bfloat16()
+    cu = torch.tensor([0, s], dtype=torch.int32)
+
+    def step():
+        out = oracle.multi_head_attention(q, oracle.repeat_kv(k, nq // nkv), oracle.repeat_kv(v, nq // nkv), cu, True,
+                                          1 / math.sqrt(d), softmax_in_fp32=True)
+        out.backward(do)
+        q.grad = k.grad = v.grad = None
+
+    step()
+    times = []
+    t_all = time.time()
+    while len(times) < 3 or (time.time() - t_all < seconds_budget / 2 and len(times) < 10):
+        t0 = time.time()
+        step()
+        times.append(time.time() - t0)
+    med = sorted(times)[len(times) // 2]
+    flops = 14 * d * nq * (s * (s + 1) // 2)
+    return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"oracle (reference op order, bf16 + fp32 softmax) attention fwd+bwd, b1 s{s} {nq}q/{nkv}kv d{d} causal, "
+                      f"median of {len(times)} runs = {med * 1e3:.1f} ms"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the path; this build uses no collectives, so --gpus must be 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from scaling_amd import _lib
+    _lib.require_device()
+    torch.cuda.set_device(0)
+
+    b, s, nq, nkv, d = 1, 8192, 32, 8, 128
+    main_res = attention_case(b, s, nq, nkv, d, [0, s], args.steps, args.warmup)
+    flops_unit = d * nq * main_res["pairs_per_head"]
+    # dominant kernel of the step and the algorithmic flops it is credited with:
+    #   forward 4 (QK^T, PV), dK/dV kernel 8 (S, dP, dV, dK), dQ kernel 2 (dQ; its S / dP are recomputation)
+    kernels = {"attn_fwd_kernel": (main_res["ms_fwd"], 4), "attn_bwd_dkdv_kernel": (main_res["ms_bwd_dkdv"], 8),
+               "attn_bwd_dq_kernel": (main_res["ms_bwd_dq"], 2)}
+    dom = max(kernels, key=lambda n: kernels[n][0])
+    dom_ms, dom_mult = kernels[dom]
+    achieved = dom_mult * flops_unit / (dom_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "avg_launch_ms": dom_ms}
+
+    extra = {"headline": main_res}
+    if not args.no_extra:
+        from tests.attn_utils import random_docs_cu
+        extra["config2_mha_b4_s2048"] = attention_case(4, 2048, 32, 32, 128, [i * 2048 for i in range(5)], args.steps, args.warmup, seed=2)
+        cu3 = random_docs_cu(8192, 256, 2048, seed=0).tolist()
+        extra["config3_gqa_packed_rotary_s8192"] = attention_case(1, 8192, 32, 8, 128, cu3, args.steps, args.warmup, seed=3, rotary=True)
+        extra["config3_gqa_packed_rotary_s8192"]["n_docs"] = len(cu3) - 1
+        extra.update(bandwidth_cases(args.steps, args.warmup))
+
+    line = {
+        "metric": "attn fwd+bwd TFLOP/s (% bf16 MFMA peak); decode tok/s; norm GB/s (% HBM)",
+        "value": main_res["tflops_step"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "attention core fwd+bwd, GQA 32q/8kv, head_dim 128, batch 1 x seq 8192, causal, bf16, fp32 softmax",
+                   "pairs_per_head": main_res["pairs_per_head"], "flop_formula": "14*d*n_q*P"},
+        "frac_of_bf16_peak": main_res["tflops_step"] / PEAK_BF16_TFLOPS,
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    line["extra"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

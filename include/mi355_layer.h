@@ -120,6 +120,10 @@ int mi_rotary(const void* x, void* out, const void* cos, const void* sin, const 
  * ------------------------------------------------------------------------------------------ */
 #define MI_ATTN_QG1 1   /* forward: one group of 32 queries per wavefront (128 per workgroup) */
 #define MI_ATTN_QG2 2   /* forward: two groups of 32 queries per wavefront (256 per workgroup) */
+/* backward: run only the named kernels (for per-kernel timing; all three when none of the bits is set) */
+#define MI_ATTN_BWD_DELTA 16
+#define MI_ATTN_BWD_DKDV 32
+#define MI_ATTN_BWD_DQ 64
 
 typedef struct mi_attn_args {
     const void* q;
@@ -142,7 +146,7 @@ typedef struct mi_attn_args {
     int64_t v_stride_token, v_stride_head;
     int64_t o_stride_token, o_stride_head;
     float softmax_scale;
-    int32_t flags;                 /* 0 = library chooses; MI_ATTN_QG1 / MI_ATTN_QG2 pin the forward tiling */
+    int32_t flags;                 /* 0 = library chooses; MI_ATTN_* bits above */
     /* optional fused rotary */
     const void* rotary_cos;
     const void* rotary_sin;

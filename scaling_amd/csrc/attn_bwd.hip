@@ -406,8 +406,10 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnParams 
     }
 }
 
-template <int D> int launch_bwd(const AttnParams& p, hipStream_t st) {
-    {
+template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) {
+    const int stages = flags & (MI_ATTN_BWD_DELTA | MI_ATTN_BWD_DKDV | MI_ATTN_BWD_DQ);
+    const bool all = stages == 0;
+    if (all || (stages & MI_ATTN_BWD_DELTA)) {
         const int64_t rows = (int64_t)p.total_q * p.nq;
         const int64_t blocks = (rows * 16 + kThreads - 1) / kThreads;
         if (blocks > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_bwd: grid too large");
@@ -415,17 +417,18 @@ template <int D> int launch_bwd(const AttnParams& p, hipStream_t st) {
         int rc = mi_check_launch("attn_bwd_delta");
         if (rc != MI_OK) return rc;
     }
-    {
+    if (all || (stages & MI_ATTN_BWD_DKDV)) {
         const int64_t grid = (((int64_t)p.total_k + 127) / 128) * p.nkv;
         attn_bwd_dkdv_kernel<D><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
         int rc = mi_check_launch("attn_bwd_dkdv");
         if (rc != MI_OK) return rc;
     }
-    {
+    if (all || (stages & MI_ATTN_BWD_DQ)) {
         const int64_t grid = (((int64_t)p.total_q + 127) / 128) * p.nq;
         attn_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
         return mi_check_launch("attn_bwd_dq");
     }
+    return MI_OK;
 }
 
 }  // namespace
@@ -464,10 +467,10 @@ extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
     p.delta = (float*)b->workspace;
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
-        case 32: return launch_bwd<32>(p, st);
-        case 64: return launch_bwd<64>(p, st);
-        case 96: return launch_bwd<96>(p, st);
-        case 128: return launch_bwd<128>(p, st);
+        case 32: return launch_bwd<32>(p, a->flags, st);
+        case 64: return launch_bwd<64>(p, a->flags, st);
+        case 96: return launch_bwd<96>(p, a->flags, st);
+        case 128: return launch_bwd<128>(p, a->flags, st);
         default: return mi_fail(MI_E_SHAPE, "attn_bwd: head_dim %d unsupported", a->head_dim);
     }
 }

@@ -214,8 +214,12 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
     return o, lse
 
 
-def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None):
-    """Returns (dq, dk, dv) for already rotated q/k."""
+def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None,
+                       flags=0, buffers=None):
+    """Returns (dq, dk, dv) for already rotated q/k.
+
+    flags: 0 runs the whole backward; 16 / 32 / 64 run only the delta / dK-dV / dQ kernel (timing aid).
+    buffers: optional (dq, dk, dv, workspace) to reuse across calls."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
     lib = _lib.load()
     if softmax_scale is None:
@@ -223,15 +227,19 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
     if do.stride() != o.stride():
         do = do.contiguous()
         assert do.stride() == o.stride()
-    dq = torch.empty_like(q)
-    if dq.stride() != q.stride():
-        dq = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
-    dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
-    dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
-    nbytes = lib.mi_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], q.shape[2])
-    ws = torch.empty(max(nbytes // 4, 4), dtype=torch.float32, device=q.device)
+    if buffers is not None:
+        dq, dk, dv, ws = buffers
+        assert dq.stride() == q.stride()
+    else:
+        dq = torch.empty_like(q)
+        if dq.stride() != q.stride():
+            dq = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+        dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+        dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+        nbytes = lib.mi_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], q.shape[2])
+        ws = torch.empty(max(nbytes // 4, 4), dtype=torch.float32, device=q.device)
     b = MiAttnBwdArgs()
-    b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale)
+    b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, None, flags)
     b.d_o, b.dq, b.dk, b.dv = ptr(do), ptr(dq), ptr(dk), ptr(dv)
     b.dk_stride_token, b.dk_stride_head = dk.stride(0), dk.stride(1)
     b.dv_stride_token, b.dv_stride_head = dv.stride(0), dv.stride(1)

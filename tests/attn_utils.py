@@ -62,14 +62,23 @@ def oracle_attention(q, k, v, cu, b, s, causal, scale, dtype=torch.float32, do=N
     return o.detach(), qq.grad, kk.grad, vv.grad
 
 
-def rows_reference(q, k, v, lo_hi, rows, head, kv_head, scale):
-    """fp64 attention of selected query rows of one head against keys [lo, hi) per row (size-independent check)."""
+def rows_reference(q, k, v, lo_hi, rows, head, kv_head, scale, reference_bf16_order=False):
+    """Attention of selected query rows of one head against keys [lo, hi) per row (size-independent check).
+
+    Default: fp64 truth.  reference_bf16_order=True reproduces the reference's rounding points for
+    bf16 tensors instead (scores rounded to bf16, fp32 softmax, probabilities rounded to bf16, output bf16).
+    """
     outs = []
     for r in rows:
         lo, hi = lo_hi(r)
-        sc = (k[lo:hi, kv_head].double() @ q[r, head].double()) * scale
-        p = torch.softmax(sc, 0)
-        outs.append(p @ v[lo:hi, kv_head].double())
+        if reference_bf16_order:
+            sc = ((k[lo:hi, kv_head].float() @ q[r, head].float()) * scale).bfloat16().float()
+            p = torch.softmax(sc, 0).bfloat16().float()
+            outs.append((p @ v[lo:hi, kv_head].float()).bfloat16().float())
+        else:
+            sc = (k[lo:hi, kv_head].double() @ q[r, head].double()) * scale
+            p = torch.softmax(sc, 0)
+            outs.append((p @ v[lo:hi, kv_head].double()).float())
     return torch.stack(outs)
 
 

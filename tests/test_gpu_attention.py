@@ -229,7 +229,8 @@ def test_attention_full_size_properties(name, b, s, nq, nkv, docs):
     for head in (0, nq // 2 + 1, nq - 1):
         kvh = head // (nq // nkv)
         ref = U.rows_reference(q, k, v, lo_hi, rows, head, kvh, scale)
-        check(f"{name}.rows.head{head}", o[rows, head], ref.float())
+        ref_o = U.rows_reference(q, k, v, lo_hi, rows, head, kvh, scale, reference_bf16_order=True)
+        check(f"{name}.rows.head{head}", o[rows, head], ref, ref_o)
     ones = torch.ones_like(vd)
     o1, _ = ops.attention_forward(qd, kd, ones, cud, None, True, scale)
     assert float((o1.float() - 1).abs().max()) <= 2 ** -7
