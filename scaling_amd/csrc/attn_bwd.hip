@@ -64,22 +64,9 @@ __device__ __forceinline__ void store_rows(const uint4 (&raw)[4], uint16_t* rm, 
 }
 
 __device__ __forceinline__ void store_transposed(const uint4 (&raw)[4], char* tr, int quad, int dg) {
-    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&raw[0]);
-    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&raw[1]);
-    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&raw[2]);
-    const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&raw[3]);
 #pragma unroll
-    for (int dd = 0; dd < 8; ++dd) {
-        uint32_t lo, hi;
-        if (dd & 1) {
-            lo = (w0[dd >> 1] >> 16) | (w1[dd >> 1] & 0xffff0000u);
-            hi = (w2[dd >> 1] >> 16) | (w3[dd >> 1] & 0xffff0000u);
-        } else {
-            lo = (w0[dd >> 1] & 0xffffu) | (w1[dd >> 1] << 16);
-            hi = (w2[dd >> 1] & 0xffffu) | (w3[dd >> 1] << 16);
-        }
-        *reinterpret_cast<uint2*>(tr + chunk_quad_offset<64>(8 * dg + dd, quad)) = make_uint2(lo, hi);
-    }
+    for (int dd = 0; dd < 8; ++dd)
+        *reinterpret_cast<uint2*>(tr + chunk_quad_offset<64>(8 * dg + dd, quad)) = transpose_quad(raw, dd);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -76,11 +76,12 @@ __device__ __forceinline__ void query_range(const AttnParams& p, int u, int& qlo
 }
 
 // ---- "chunk order" LDS layout for operands whose contraction index is the row index of a C tile ----
-// A [R rows][N contraction] matrix (N multiple of 16) is stored row-major with 16-byte units XOR-
-// swizzled per row; inside each 16-wide chunk the contraction indices are permuted so that lane
-// group g finds its 8 k-slots contiguous:  unit (2*m + g) of row r holds indices
-// 16*m + {4g..4g+3, 8+4g..8+4g+3}.
-__device__ __forceinline__ int swz(int row) { return ((row >> 1) + (row >> 4)) & 7; }
+// A [R rows][64 contraction] matrix is stored row-major (128 bytes per row) with the 16-byte units of a
+// row XOR-swizzled; inside each 16-wide chunk the contraction indices are permuted so that lane group
+// g finds its 8 k-slots contiguous: unit (2*m + g) of row r holds indices 16*m + {4g..4g+3, 8+4g..8+4g+3}.
+// The swizzle depends on (row & 31) only, so the address of (row + 32*dt) is the address of row plus
+// an immediate, and 16 consecutive rows read by one lane group hit 16 different bank quads.
+__device__ __forceinline__ int swz(int row) { return ((row >> 1) & 7) ^ ((row >> 3) & 3); }
 
 // byte offset of the 8-byte group holding contraction indices 4*quad .. 4*quad+3 (quad = index / 4)
 template <int N> __device__ __forceinline__ int chunk_quad_offset(int row, int quad) {
@@ -94,6 +95,17 @@ template <int N> __device__ __forceinline__ int chunk_quad_offset(int row, int q
 template <int N> __device__ __forceinline__ int chunk_unit_offset(int row, int m, int g) {
     static_assert(N == 64, "one row = 8 swizzled units of 16 bytes");
     return row * (N * 2) + (((2 * m + g) ^ swz(row)) << 4);
+}
+
+// 4 tokens x 8 features held as 4 row vectors -> for feature dd the 4 token values as one 8-byte group
+__device__ __forceinline__ uint2 transpose_quad(const uint4 (&raw)[4], int dd) {
+    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&raw[0]);
+    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&raw[1]);
+    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&raw[2]);
+    const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&raw[3]);
+    const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of the two words
+    return make_uint2(__builtin_amdgcn_perm(w1[dd >> 1], w0[dd >> 1], sel),
+                      __builtin_amdgcn_perm(w3[dd >> 1], w2[dd >> 1], sel));
 }
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {

@@ -1,11 +1,14 @@
 // Attention forward for gfx950 (bf16 MFMA, fp32 online softmax, causal / packed-document masks, GQA).
 //
-// Workgroup = 4 wavefronts; wavefront w owns QG groups of 32 consecutive query tokens of one head.
+// Workgroup = NW wavefronts (4 or 8); every wavefront owns 32 consecutive query tokens of one head and
+// two wavefronts share a SIMD, so one can issue MFMAs while the other runs its softmax on the VALU.
 // Keys/values stream through LDS in tiles of 64 tokens (double buffered, one barrier per tile).
-// Per tile and query group:
+// Per tile:
 //     S^T = K * Q^T            A = K tile rows from LDS, B = Q fragment held in registers
-//     online softmax           each lane owns ONE query (C column), so the row max / sum are in-lane
-//                              reductions plus a single exchange with lane ^ 32
+//     online softmax           each lane owns ONE query (C column): the row max / sum are in-lane
+//                              reductions plus a single exchange with lane ^ 32.  The running max is
+//                              only raised (and O rescaled) when it grows by more than 2^8, so the
+//                              rescale of the 64 accumulator registers is skipped on most tiles.
 //     O^T += V^T * P^T         B = P^T taken straight from the S^T accumulators (no LDS round trip),
 //                              A = V^T read from a transposed, chunk-ordered LDS copy of the V tile
 // The mask is a per-lane key interval [klo, khi) derived from the cumulative sequence lengths; tiles
@@ -14,22 +17,23 @@
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int BN = 64;  // keys per tile
+constexpr int BN = 64;               // keys per tile
+constexpr float kRescaleGap = 8.0f;  // log2 units by which a row max may lag before O is rescaled
 
-template <int D, int QG, bool ROT>
-__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnParams p) {
-    constexpr int BM = 128 * QG;
+template <int D, int NW, bool ROT>
+__global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p) {
+    constexpr int BM = 32 * NW;
     constexpr int KSTR = D + 8;           // padded K row (elements): conflict-free 128-bit row reads
     constexpr int KS = D / 16;            // contraction steps of Q K^T
     constexpr int DT = D / 32;            // 32-row tiles of O^T
-    constexpr int KV_VECS = D / 32;       // 128-bit K vectors per thread and tile
+    constexpr int KV_VECS = D / 32;       // 128-bit K vectors per loader thread and tile
     constexpr int V_ITEMS = 16 * (D / 8); // (key quad, 8-column group) items of a V tile
     static_assert(D % 32 == 0 && D <= 128, "head_dim must be 32, 64, 96 or 128");
+    static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts");
 
     __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KSTR];
     __shared__ __attribute__((aligned(16))) uint16_t vt_lds[2][D * BN];
-    __shared__ int range_lds[8];
+    __shared__ int range_lds[2 * NW];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -41,21 +45,15 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnParams p) 
     const int qb = nqb - 1 - (work / p.n_rep) % nqb;   // long (late) query blocks first
     const int kvh = work / (p.n_rep * nqb);
     const int head = kvh * p.n_rep + rep;
-    const int q0 = qb * BM + wave * (32 * QG);
 
-    // ---- per-lane query, mask interval, Q fragments ------------------------------------------
-    int tq[QG], klo[QG], khi[QG];
-    bf16x8_t qf[QG][KS];
-    int wmin = 0x7fffffff, wmax = 0;
-#pragma unroll
-    for (int i = 0; i < QG; ++i) {
-        tq[i] = q0 + 32 * i + l32;
-        key_range(p, tq[i], klo[i], khi[i]);
-        if (khi[i] > klo[i]) {
-            wmin = min(wmin, klo[i]);
-            wmax = max(wmax, khi[i]);
-        }
-        const int tl = tq[i] < p.total_q ? tq[i] : p.total_q - 1;
+    // ---- per-lane query, mask interval, Q fragment ---------------------------------------------
+    const int tq = qb * BM + wave * 32 + l32;
+    int klo, khi;
+    key_range(p, tq, klo, khi);
+    int wmin = khi > klo ? klo : 0x7fffffff, wmax = khi > klo ? khi : 0;
+    bf16x8_t qf[KS];
+    {
+        const int tl = tq < p.total_q ? tq : p.total_q - 1;
         const __bf16* qrow = p.q + (int64_t)tl * p.q_st + (int64_t)head * p.q_sh + 8 * g;
         uint4 raw[KS];
 #pragma unroll
@@ -73,116 +71,103 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnParams p) 
             }
         }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[i][ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
     }
-    // wave and block key ranges
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         wmin = min(wmin, __shfl_xor(wmin, off, 64));
         wmax = max(wmax, __shfl_xor(wmax, off, 64));
     }
-    if (lane == 0) { range_lds[wave] = wmin; range_lds[4 + wave] = wmax; }
+    if (lane == 0) { range_lds[wave] = wmin; range_lds[NW + wave] = wmax; }
     __syncthreads();
-    int bmin = min(min(range_lds[0], range_lds[1]), min(range_lds[2], range_lds[3]));
-    int bmax = max(max(range_lds[4], range_lds[5]), max(range_lds[6], range_lds[7]));
+    int bmin = 0x7fffffff, bmax = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) { bmin = min(bmin, range_lds[w]); bmax = max(bmax, range_lds[NW + w]); }
     if (bmax <= bmin) { bmin = 0; bmax = 0; }
     const int kt0 = bmin & ~(BN - 1);
     const int n_tiles = (bmax - kt0 + BN - 1) / BN;
 
     // ---- accumulators ----------------------------------------------------------------------
-    f32x16_t o_acc[QG][DT];
-    float m_i[QG], l_i[QG];
+    f32x16_t o_acc[DT];
 #pragma unroll
-    for (int i = 0; i < QG; ++i) {
-        m_i[i] = -INFINITY;
-        l_i[i] = 0.f;
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o_acc[i][dt][r] = 0.f;
-    }
+        for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
+    float m_i = -INFINITY, l_i = 0.f;
 
-    // ---- tile loaders ----------------------------------------------------------------------
+    // ---- tile loaders: with 8 wavefronts the first four stage V, the last four stage K ----------
+    const bool v_role = (NW == 4) || (tid < 256);
+    const bool k_role = (NW == 4) || (tid >= 256);
+    const int ltid = (NW == 4) ? tid : (tid & 255);
     uint4 kraw[KV_VECS];
     uint4 vraw[4];
     uint4 craw[ROT ? KV_VECS / 2 : 1], sraw[ROT ? KV_VECS / 2 : 1];  // rotary table rows of the K tile
     const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
     const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
-    const int v_kg = tid / (D / 8), v_dg = tid % (D / 8);
+    const int v_kg = ltid / (D / 8), v_dg = ltid % (D / 8);
+    const int last_k = p.total_k - 1;
 
     auto load_tile = [&](int kt) {
-        if constexpr (!ROT) {
+        if (k_role) {
+            if constexpr (!ROT) {
 #pragma unroll
-            for (int j = 0; j < KV_VECS; ++j) {
-                const int idx = tid + kThreads * j;
-                const int row = idx / (D / 8), c = idx % (D / 8);
-                int tok = kt + row;
-                tok = tok < p.total_k ? tok : p.total_k - 1;
-                kraw[j] = *reinterpret_cast<const uint4*>(kbase + (int64_t)tok * p.k_st + 8 * c);
-            }
-        } else {
+                for (int j = 0; j < KV_VECS; ++j) {
+                    const int idx = ltid + 256 * j;
+                    const int row = idx / (D / 8), c = idx % (D / 8);
+                    const int tok = min(kt + row, last_k);
+                    kraw[j] = *reinterpret_cast<const uint4*>(kbase + (int64_t)tok * p.k_st + 8 * c);
+                }
+            } else {
 #pragma unroll
-            for (int j = 0; j < KV_VECS / 2; ++j) {
-                const int idx = tid + kThreads * j;
-                const int row = idx / (D / 16), c = idx % (D / 16);
-                int tok = kt + row;
-                tok = tok < p.total_k ? tok : p.total_k - 1;
-                const __bf16* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
-                kraw[2 * j] = *reinterpret_cast<const uint4*>(kr);
-                kraw[2 * j + 1] = *reinterpret_cast<const uint4*>(kr + D / 2);
-                int64_t pos = p.pos_k[tok];
-                pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
-                craw[j] = *reinterpret_cast<const uint4*>(p.cos + pos * D + 8 * c);
-                sraw[j] = *reinterpret_cast<const uint4*>(p.sin + pos * D + 8 * c);
+                for (int j = 0; j < KV_VECS / 2; ++j) {
+                    const int idx = ltid + 256 * j;
+                    const int row = idx / (D / 16), c = idx % (D / 16);
+                    const int tok = min(kt + row, last_k);
+                    const __bf16* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
+                    kraw[2 * j] = *reinterpret_cast<const uint4*>(kr);
+                    kraw[2 * j + 1] = *reinterpret_cast<const uint4*>(kr + D / 2);
+                    int64_t pos = p.pos_k[tok];
+                    pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+                    craw[j] = *reinterpret_cast<const uint4*>(p.cos + pos * D + 8 * c);
+                    sraw[j] = *reinterpret_cast<const uint4*>(p.sin + pos * D + 8 * c);
+                }
             }
         }
-        if (tid < V_ITEMS) {
+        if (v_role && ltid < V_ITEMS) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                int tok = kt + 4 * v_kg + j;
-                tok = tok < p.total_k ? tok : p.total_k - 1;
+                const int tok = min(kt + 4 * v_kg + j, last_k);
                 vraw[j] = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.v_st + 8 * v_dg);
             }
         }
     };
 
     auto store_tile = [&](int buf) {
-        uint16_t* ks = k_lds[buf];
-        if constexpr (!ROT) {
+        if (k_role) {
+            uint16_t* ks = k_lds[buf];
+            if constexpr (!ROT) {
 #pragma unroll
-            for (int j = 0; j < KV_VECS; ++j) {
-                const int idx = tid + kThreads * j;
-                const int row = idx / (D / 8), c = idx % (D / 8);
-                *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[j];
-            }
-        } else {
+                for (int j = 0; j < KV_VECS; ++j) {
+                    const int idx = ltid + 256 * j;
+                    const int row = idx / (D / 8), c = idx % (D / 8);
+                    *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[j];
+                }
+            } else {
 #pragma unroll
-            for (int j = 0; j < KV_VECS / 2; ++j) {
-                const int idx = tid + kThreads * j;
-                const int row = idx / (D / 16), c = idx % (D / 16);
-                rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);  // rotate after the MFMA section
-                *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[2 * j];
-                *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c + D / 2) = kraw[2 * j + 1];
+                for (int j = 0; j < KV_VECS / 2; ++j) {
+                    const int idx = ltid + 256 * j;
+                    const int row = idx / (D / 16), c = idx % (D / 16);
+                    rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);  // after the MFMA section
+                    *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[2 * j];
+                    *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c + D / 2) = kraw[2 * j + 1];
+                }
             }
         }
-        if (tid < V_ITEMS) {
+        if (v_role && ltid < V_ITEMS) {
             char* vt = reinterpret_cast<char*>(vt_lds[buf]);
-            const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&vraw[0]);
-            const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&vraw[1]);
-            const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&vraw[2]);
-            const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&vraw[3]);
 #pragma unroll
-            for (int dd = 0; dd < 8; ++dd) {
-                uint32_t lo, hi;
-                if (dd & 1) {
-                    lo = (w0[dd >> 1] >> 16) | (w1[dd >> 1] & 0xffff0000u);
-                    hi = (w2[dd >> 1] >> 16) | (w3[dd >> 1] & 0xffff0000u);
-                } else {
-                    lo = (w0[dd >> 1] & 0xffffu) | (w1[dd >> 1] << 16);
-                    hi = (w2[dd >> 1] & 0xffffu) | (w3[dd >> 1] << 16);
-                }
-                *reinterpret_cast<uint2*>(vt + chunk_quad_offset<BN>(8 * v_dg + dd, v_kg)) = make_uint2(lo, hi);
-            }
+            for (int dd = 0; dd < 8; ++dd)
+                *reinterpret_cast<uint2*>(vt + chunk_quad_offset<BN>(8 * v_dg + dd, v_kg)) = transpose_quad(vraw, dd);
         }
     };
 
@@ -193,6 +178,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnParams p) 
     }
     __syncthreads();
 
+    const float c2 = p.scale_log2;
     for (int it = 0; it < n_tiles; ++it) {
         const int kt = kt0 + it * BN;
         const int buf = it & 1;
@@ -200,79 +186,77 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnParams p) 
 
         const bool wave_active = (kt < wmax) && (kt + BN > wmin);
         if (wave_active) {
-            const uint16_t* ks = k_lds[buf];
+            const uint16_t* ks = k_lds[buf] + l32 * KSTR + 8 * g;
             const char* vt = reinterpret_cast<const char*>(vt_lds[buf]);
 
-            f32x16_t s_acc[QG][2];
+            f32x16_t s_acc[2];
 #pragma unroll
-            for (int i = 0; i < QG; ++i)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) s_acc[i][t][r] = 0.f;
-
+                for (int r = 0; r < 16; ++r) s_acc[t][r] = 0.f;
 #pragma unroll
             for (int ksi = 0; ksi < KS; ++ksi) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks + (32 * t + l32) * KSTR + 16 * ksi + 8 * g);
-#pragma unroll
-                    for (int i = 0; i < QG; ++i) s_acc[i][t] = mfma_32x32x16(a, qf[i][ksi], s_acc[i][t]);
+                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks + 32 * t * KSTR + 16 * ksi);
+                    s_acc[t] = mfma_32x32x16(a, qf[ksi], s_acc[t]);
                 }
             }
 
-            bf16x8_t pf[QG][4];
-#pragma unroll
-            for (int i = 0; i < QG; ++i) {
-                const bool need_mask = __any((kt < klo[i]) || (kt + BN > khi[i]));
-                if (need_mask) {
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int key = kt + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
-                            if (key < klo[i] || key >= khi[i]) s_acc[i][t][r] = -INFINITY;
-                        }
-                }
-                float mx = -INFINITY;
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[i][t][r]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m_i[i], mx * p.scale_log2);
-                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                const float alpha = fast_exp2(m_i[i] - m_use);
-                m_i[i] = m_new;
-                float rs = 0.f;
+            // tiles that cross an interval boundary of some lane get the compare; the others skip it
+            if (__any((kt < klo) || (kt + BN > khi))) {
+                int rel0 = kt + 4 * g - klo;
+                asm volatile("" : "+v"(rel0));   // opaque: keeps the 32 compares inside this branch
+                const unsigned len = (unsigned)(khi - klo);
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const float e = fast_exp2(s_acc[i][t][r] * p.scale_log2 - m_use);
-                        s_acc[i][t][r] = e;
-                        rs += e;
+                        const unsigned rel = (unsigned)(rel0 + 32 * t + 8 * (r >> 2) + (r & 3));
+                        if (rel >= len) s_acc[t][r] = -INFINITY;
                     }
-                l_i[i] = l_i[i] * alpha + rs;
+            }
+            float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s_acc[0][r], s_acc[1][r]));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_cand = mx * c2;
+            if (__any(m_cand > m_i + kRescaleGap)) {
+                const float m_new = fmaxf(m_i, m_cand);
+                float alpha = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_i - m_new);
+                // opaque to the optimiser: keeps the 64 multiplies below inside this rarely taken
+                // branch instead of being speculated onto every tile
+                asm volatile("" : "+v"(alpha));
+                m_i = m_new;
+                l_i *= alpha;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) o_acc[i][dt][r] *= alpha;
-#pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    const int t = m >> 1, r0 = 8 * (m & 1);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) pf[i][m][e] = (__bf16)s_acc[i][t][r0 + e];
-                }
+                    for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
             }
+            const float m_use = (m_i == -INFINITY) ? 0.f : m_i;
+            float rs0 = 0.f, rs1 = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e0 = fast_exp2(s_acc[0][r] * c2 - m_use);
+                const float e1 = fast_exp2(s_acc[1][r] * c2 - m_use);
+                s_acc[0][r] = e0;
+                s_acc[1][r] = e1;
+                rs0 += e0;
+                rs1 += e1;
+            }
+            l_i += rs0 + rs1;
 
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
+                const int t = m >> 1, r0 = 8 * (m & 1);
+                bf16x8_t pf;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s_acc[t][r0 + e];
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
                     const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(vt + chunk_unit_offset<BN>(32 * dt + l32, m, g));
-#pragma unroll
-                    for (int i = 0; i < QG; ++i) o_acc[i][dt] = mfma_32x32x16(a, pf[i][m], o_acc[i][dt]);
+                    o_acc[dt] = mfma_32x32x16(a, pf, o_acc[dt]);
                 }
             }
         }
@@ -282,46 +266,43 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(const AttnParams p) 
     }
 
     // ---- epilogue ------------------------------------------------------------------------------
+    const float l_tot = l_i + __shfl_xor(l_i, 32, 64);
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    if (tq < p.total_q) {
+        __bf16* orow = p.o + (int64_t)tq * p.o_st + (int64_t)head * p.o_sh + 4 * g;
 #pragma unroll
-    for (int i = 0; i < QG; ++i) {
-        const float l_tot = l_i[i] + __shfl_xor(l_i[i], 32, 64);
-        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-        if (tq[i] < p.total_q) {
-            __bf16* orow = p.o + (int64_t)tq[i] * p.o_st + (int64_t)head * p.o_sh + 4 * g;
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const uint32_t w0 = pack_bf16x2(o_acc[i][dt][4 * a] * inv, o_acc[i][dt][4 * a + 1] * inv);
-                    const uint32_t w1 = pack_bf16x2(o_acc[i][dt][4 * a + 2] * inv, o_acc[i][dt][4 * a + 3] * inv);
-                    *reinterpret_cast<uint2*>(orow + 32 * dt + 8 * a) = make_uint2(w0, w1);
-                }
-            if (g == 0 && p.lse != nullptr) {
-                const float lse = l_tot > 0.f ? (m_i[i] + __log2f(l_tot)) * 0.6931471805599453f : INFINITY;
-                p.lse[(int64_t)head * p.total_q + tq[i]] = lse;
+            for (int a = 0; a < 4; ++a) {
+                const uint32_t w0 = pack_bf16x2(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv);
+                const uint32_t w1 = pack_bf16x2(o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
+                *reinterpret_cast<uint2*>(orow + 32 * dt + 8 * a) = make_uint2(w0, w1);
             }
+        if (g == 0 && p.lse != nullptr) {
+            const float lse = l_tot > 0.f ? (m_i + __log2f(l_tot)) * 0.6931471805599453f : INFINITY;
+            p.lse[(int64_t)head * p.total_q + tq] = lse;
         }
     }
 }
 
-template <int D, int QG, bool ROT> int launch(const AttnParams& p, hipStream_t st) {
-    constexpr int BM = 128 * QG;
+template <int D, int NW, bool ROT> int launch(const AttnParams& p, hipStream_t st) {
+    constexpr int BM = 32 * NW;
     const int64_t nqb = ((int64_t)p.total_q + BM - 1) / BM;
     const int64_t grid = nqb * p.nq;
     if (grid > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_fwd: grid too large");
-    attn_fwd_kernel<D, QG, ROT><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
+    attn_fwd_kernel<D, NW, ROT><<<dim3((unsigned)grid), dim3(64 * NW), 0, st>>>(p);
     return mi_check_launch("attn_fwd");
 }
 
-template <int D> int launch_d(const AttnParams& p, bool rot, int qg, hipStream_t st) {
+template <int D> int launch_d(const AttnParams& p, bool rot, int nw, hipStream_t st) {
     if (rot) {
         if constexpr (D == 64 || D == 128) {
-            return qg == 2 ? launch<D, 2, true>(p, st) : launch<D, 1, true>(p, st);
+            return nw == 8 ? launch<D, 8, true>(p, st) : launch<D, 4, true>(p, st);
         } else {
             return mi_fail(MI_E_SHAPE, "attn_fwd: fused rotary needs head_dim 64 or 128");
         }
     }
-    return qg == 2 ? launch<D, 2, false>(p, st) : launch<D, 1, false>(p, st);
+    return nw == 8 ? launch<D, 8, false>(p, st) : launch<D, 4, false>(p, st);
 }
 
 }  // namespace
@@ -339,18 +320,18 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     AttnParams p;
     mi_attn_fill_params(a, &p);
     const bool rot = a->rotary_cos != nullptr;
-    // two query groups per wavefront halve the LDS traffic per MFMA; worth it once the grid still
-    // fills the chip
-    const int64_t blocks_qg2 = (((int64_t)p.total_q + 255) / 256) * p.nq;
-    int qg = blocks_qg2 >= 512 ? 2 : 1;
-    if (a->flags & MI_ATTN_QG1) qg = 1;
-    if (a->flags & MI_ATTN_QG2) qg = 2;
+    // 256-query workgroups halve the K/V staging work per query; worth it once the grid still fills
+    // the 256 compute units a few times over
+    const int64_t blocks_256 = (((int64_t)p.total_q + 255) / 256) * p.nq;
+    int nw = blocks_256 >= 512 ? 8 : 4;
+    if (a->flags & MI_ATTN_QG1) nw = 4;
+    if (a->flags & MI_ATTN_QG2) nw = 8;
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
-        case 32: return launch_d<32>(p, rot, qg, st);
-        case 64: return launch_d<64>(p, rot, qg, st);
-        case 96: return launch_d<96>(p, rot, qg, st);
-        case 128: return launch_d<128>(p, rot, qg, st);
+        case 32: return launch_d<32>(p, rot, nw, st);
+        case 64: return launch_d<64>(p, rot, nw, st);
+        case 96: return launch_d<96>(p, rot, nw, st);
+        case 128: return launch_d<128>(p, rot, nw, st);
         default: return mi_fail(MI_E_SHAPE, "attn_fwd: head_dim %d unsupported (32, 64, 96, 128)", a->head_dim);
     }
 }

@@ -15,9 +15,11 @@ LIB_NAME = "libmi355_layer.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = ["abi.hip", "rmsnorm.hip", "swiglu.hip", "rotary.hip", "attn_host.hip", "attn_fwd.hip", "attn_bwd.hip",
            "attn_decode.hip"]
-# packed fp32 VALU instructions stay disabled for every device translation unit
+# packed fp32 VALU instructions stay disabled for every device translation unit; the kernels never
+# produce NaNs on purpose (masked scores are -inf and every inf - inf is guarded), so NaN-preserving
+# canonicalisation of the MFMA results before max / min is switched off
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+         "-packed-fp32-ops", "-fno-honor-nans", "-Wno-unused-command-line-argument"]
 
 
 def _hipcc() -> str:
