@@ -2,11 +2,11 @@
 //
 // Three kernels, no atomics, fixed summation order (bit-reproducible):
 //   1. delta[h][t] = sum_d dO[t][h][d] * O[t][h][d]
-//   2. dK/dV: a workgroup owns 128 keys of one KV head (32 per wavefront, K and V fragments stay in
-//      registers), loops over the query heads of the group and over 64-query tiles staged in LDS:
+//   2. dK/dV: a workgroup owns 128 keys of one KV head (K and V rows stay in LDS), loops over the query
+//      heads of the group and over 64-query tiles staged in LDS:
 //          S = Q K^T,  P = exp2(S*c - lse),  dP = dO V^T,  dS = P * (dP - delta)
 //          dV^T += dO^T P        dK^T += Q^T dS         (P / dS feed the MFMA straight from registers)
-//   3. dQ: a workgroup owns 128 queries of one head (32 per wavefront, Q and dO fragments in registers),
+//   3. dQ: a workgroup owns 256 queries of one head (32 per wavefront, Q and dO fragments in registers),
 //      loops over 64-key tiles:  S^T = K Q^T, dP^T = V dO^T, dS^T, dQ^T += K^T dS^T.
 // Operands whose contraction index is a token index are kept in LDS transposed and "chunk ordered"
 // (see attn_common.h) so that score tiles can be consumed in their accumulator layout.
@@ -72,31 +72,46 @@ __device__ __forceinline__ void store_transposed(const uint4 (&raw)[4], char* tr
 // ---------------------------------------------------------------------------------------------
 // 2. dK / dV
 // ---------------------------------------------------------------------------------------------
+// 8 wavefronts, two per SIMD.  The workgroup owns 128 keys of one KV head whose K and V rows stay in
+// LDS for its lifetime; wavefront w works on key group (w & 3) (32 keys) and on query sub-tile (w >> 2)
+// (32 of the 64 queries staged per iteration), so the pair (w, w + 4) accumulates the same dK / dV
+// rows and is summed once at the end.  The first four wavefronts stage Q, the last four dO.
 template <int D>
-__global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(const AttnParams p) {
-    constexpr int BNK = 128;              // keys per workgroup (32 per wavefront)
+__global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
+    constexpr int NT = 512;
+    constexpr int BNK = 128;              // keys per workgroup
     constexpr int BQ = 64;                // queries per tile
     constexpr int STR = D + 8;
     constexpr int KS = D / 16;
     constexpr int DT = D / 32;
     constexpr int ITEMS = 16 * (D / 8);
+    constexpr int KV_BYTES = BNK * STR * 2;
+    constexpr int QROW_BYTES = BQ * STR * 2;
+    constexpr int QTR_BYTES = D * BQ * 2;
+    constexpr int STAGE_BYTES = 2 * KV_BYTES + 2 * QROW_BYTES + 2 * QTR_BYTES;
+    constexpr int RED_BYTES = 4 * 16 * DT * 64 * 4;   // one accumulator set of four wavefronts
+    constexpr int SMEM_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
 
-    __shared__ __attribute__((aligned(16))) uint16_t q_rm[BQ * STR];
-    __shared__ __attribute__((aligned(16))) uint16_t do_rm[BQ * STR];
-    __shared__ __attribute__((aligned(16))) uint16_t q_tr[D * BQ];
-    __shared__ __attribute__((aligned(16))) uint16_t do_tr[D * BQ];
+    __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
     __shared__ __attribute__((aligned(16))) float lse_lds[BQ];
     __shared__ __attribute__((aligned(16))) float delta_lds[BQ];
-    __shared__ int range_lds[8];
+    __shared__ int range_lds[16];
+    uint16_t* k_rm = reinterpret_cast<uint16_t*>(smem);
+    uint16_t* v_rm = reinterpret_cast<uint16_t*>(smem + KV_BYTES);
+    uint16_t* q_rm = reinterpret_cast<uint16_t*>(smem + 2 * KV_BYTES);
+    uint16_t* do_rm = reinterpret_cast<uint16_t*>(smem + 2 * KV_BYTES + QROW_BYTES);
+    char* q_tr = smem + 2 * KV_BYTES + 2 * QROW_BYTES;
+    char* do_tr = q_tr + QTR_BYTES;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int kgp = wave & 3, sub = wave >> 2;
 
     const int nkb = (p.total_k + BNK - 1) / BNK;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
     const int kb = work % nkb;            // early key blocks (most queries under a causal mask) first
     const int kvh = work / nkb;
-    const int key = kb * BNK + wave * 32 + l32;
+    const int key = kb * BNK + kgp * 32 + l32;
 
     int qlo, qhi;
     query_range(p, key, qlo, qhi);
@@ -106,23 +121,25 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(const AttnParam
         wmin = min(wmin, __shfl_xor(wmin, off, 64));
         wmax = max(wmax, __shfl_xor(wmax, off, 64));
     }
-    if (lane == 0) { range_lds[wave] = wmin; range_lds[4 + wave] = wmax; }
+    if (lane == 0) { range_lds[wave] = wmin; range_lds[8 + wave] = wmax; }
 
-    // K and V fragments (B operands: column = key, contraction = feature)
-    bf16x8_t kf[KS], vf[KS];
+    // stage the K / V rows of this key block (row-major, padded rows)
     {
-        const int kl = key < p.total_k ? key : p.total_k - 1;
-        const __bf16* kr = p.k + (int64_t)kl * p.k_st + (int64_t)kvh * p.k_sh + 8 * g;
-        const __bf16* vr = p.v + (int64_t)kl * p.v_st + (int64_t)kvh * p.v_sh + 8 * g;
+        const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
+        const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            kf[ks] = *reinterpret_cast<const bf16x8_t*>(kr + 16 * ks);
-            vf[ks] = *reinterpret_cast<const bf16x8_t*>(vr + 16 * ks);
+        for (int j = 0; j < (BNK * (D / 8)) / NT; ++j) {
+            const int idx = tid + NT * j;
+            const int row = idx / (D / 8), c = idx % (D / 8);
+            const int tok = min(kb * BNK + row, p.total_k - 1);
+            *reinterpret_cast<uint4*>(k_rm + row * STR + 8 * c) = *reinterpret_cast<const uint4*>(kbase + (int64_t)tok * p.k_st + 8 * c);
+            *reinterpret_cast<uint4*>(v_rm + row * STR + 8 * c) = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.v_st + 8 * c);
         }
     }
     __syncthreads();
-    int bmin = min(min(range_lds[0], range_lds[1]), min(range_lds[2], range_lds[3]));
-    int bmax = max(max(range_lds[4], range_lds[5]), max(range_lds[6], range_lds[7]));
+    int bmin = 0x7fffffff, bmax = 0;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) { bmin = min(bmin, range_lds[w]); bmax = max(bmax, range_lds[8 + w]); }
     if (bmax <= bmin) { bmin = 0; bmax = 0; }
     const int qt0 = bmin & ~(BQ - 1);
     const int n_tiles = (bmax - qt0 + BQ - 1) / BQ;
@@ -133,32 +150,31 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(const AttnParam
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk_acc[dt][r] = 0.f; dv_acc[dt][r] = 0.f; }
 
-    const int quad = tid / (D / 8), dg = tid % (D / 8);
-    uint4 qraw[4], doraw[4];
+    const bool q_role = tid < 256;
+    const int ltid = tid & 255;
+    const int quad = ltid / (D / 8), dg = ltid % (D / 8);
+    uint4 raw[4];
     float stat = 0.f;
 
     const int total_iters = n_tiles * p.n_rep;
     auto load_tile = [&](int iter) {
         const int rep = iter / n_tiles, qt = qt0 + (iter % n_tiles) * BQ;
         const int head = kvh * p.n_rep + rep;
-        if (tid < ITEMS) {
-            load_quad<D>(qraw, p.q + (int64_t)head * p.q_sh, p.q_st, qt, p.total_q, quad, dg);
-            load_quad<D>(doraw, p.d_o + (int64_t)head * p.o_sh, p.o_st, qt, p.total_q, quad, dg);
+        if (ltid < ITEMS) {
+            if (q_role) load_quad<D>(raw, p.q + (int64_t)head * p.q_sh, p.q_st, qt, p.total_q, quad, dg);
+            else load_quad<D>(raw, p.d_o + (int64_t)head * p.o_sh, p.o_st, qt, p.total_q, quad, dg);
         }
         if (tid < 2 * BQ) {
-            int tok = qt + (tid & (BQ - 1));
-            tok = tok < p.total_q ? tok : p.total_q - 1;
+            const int tok = min(qt + (tid & (BQ - 1)), p.total_q - 1);
             const float* src = (tid < BQ) ? p.lse : p.delta;
             stat = src[(int64_t)head * p.total_q + tok];
             if (tid < BQ) stat *= 1.4426950408889634f;  // log-sum-exp in the exp2 domain
         }
     };
     auto store_tile = [&]() {
-        if (tid < ITEMS) {
-            store_rows<STR>(qraw, q_rm, quad, dg);
-            store_rows<STR>(doraw, do_rm, quad, dg);
-            store_transposed(qraw, reinterpret_cast<char*>(q_tr), quad, dg);
-            store_transposed(doraw, reinterpret_cast<char*>(do_tr), quad, dg);
+        if (ltid < ITEMS) {
+            store_rows<STR>(raw, q_role ? q_rm : do_rm, quad, dg);
+            store_transposed(raw, q_role ? q_tr : do_tr, quad, dg);
         }
         if (tid < BQ) lse_lds[tid] = stat;
         else if (tid < 2 * BQ) delta_lds[tid - BQ] = stat;
@@ -170,54 +186,62 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(const AttnParam
     }
     __syncthreads();
 
+    const uint16_t* a_q = q_rm + (32 * sub + l32) * STR + 8 * g;
+    const uint16_t* a_do = do_rm + (32 * sub + l32) * STR + 8 * g;
+    const uint16_t* b_k = k_rm + (32 * kgp + l32) * STR + 8 * g;
+    const uint16_t* b_v = v_rm + (32 * kgp + l32) * STR + 8 * g;
+    const float c2 = p.scale_log2;
+
     for (int iter = 0; iter < total_iters; ++iter) {
-        const int qt = qt0 + (iter % n_tiles) * BQ;
+        const int qs = qt0 + (iter % n_tiles) * BQ + 32 * sub;
         if (iter + 1 < total_iters) load_tile(iter + 1);
 
-        const bool wave_active = (qt < wmax) && (qt + BQ > wmin);
-        if (wave_active) {
+        if ((qs < wmax) && (qs + 32 > wmin)) {
+            f32x16_t s_acc, dp_acc;
 #pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                const int qs = qt + 32 * sub;
-                if (!((qs < wmax) && (qs + 32 > wmin))) continue;
-                f32x16_t s_acc, dp_acc;
+            for (int r = 0; r < 16; ++r) { s_acc[r] = 0.f; dp_acc[r] = 0.f; }
 #pragma unroll
-                for (int r = 0; r < 16; ++r) { s_acc[r] = 0.f; dp_acc[r] = 0.f; }
+            for (int ks = 0; ks < KS; ++ks) {
+                const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(a_q + 16 * ks);
+                const bf16x8_t bk = *reinterpret_cast<const bf16x8_t*>(b_k + 16 * ks);
+                s_acc = mfma_32x32x16(aq, bk, s_acc);
+                const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(a_do + 16 * ks);
+                const bf16x8_t bv = *reinterpret_cast<const bf16x8_t*>(b_v + 16 * ks);
+                dp_acc = mfma_32x32x16(ad, bv, dp_acc);
+            }
+            // rows of the accumulators are queries qs + 8a + 4g + c, the column is this lane's key
+            if (__any((qs < qlo) || (qs + 32 > qhi))) {
+                int rel0 = qs + 4 * g - qlo;
+                asm volatile("" : "+v"(rel0));   // opaque: keeps the compares inside this branch
+                const unsigned len = (unsigned)(qhi - qlo);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(q_rm + (32 * sub + l32) * STR + 16 * ks + 8 * g);
-                    const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(do_rm + (32 * sub + l32) * STR + 16 * ks + 8 * g);
-                    s_acc = mfma_32x32x16(aq, kf[ks], s_acc);
-                    dp_acc = mfma_32x32x16(ad, vf[ks], dp_acc);
+                for (int r = 0; r < 16; ++r) {
+                    const unsigned rel = (unsigned)(rel0 + 8 * (r >> 2) + (r & 3));
+                    if (rel >= len) s_acc[r] = -INFINITY;
                 }
-                // rows of the accumulators are queries qs + 8a + 4g + c, the column is this lane's key
-                bf16x8_t pf[2], dsf[2];
+            }
+            bf16x8_t pf[2], dsf[2];
 #pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(lse_lds + 32 * sub + 8 * a + 4 * g);
-                    const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(delta_lds + 32 * sub + 8 * a + 4 * g);
+            for (int a = 0; a < 4; ++a) {
+                const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(lse_lds + 32 * sub + 8 * a + 4 * g);
+                const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(delta_lds + 32 * sub + 8 * a + 4 * g);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const int r = 4 * a + c;
-                        const int qi = qs + 8 * a + 4 * g + c;
-                        float pv = fast_exp2(s_acc[r] * p.scale_log2 - l4[c]);
-                        if (qi < qlo || qi >= qhi) pv = 0.f;
-                        const float ds = pv * (dp_acc[r] - d4[c]);
-                        pf[a >> 1][4 * (a & 1) + c] = (__bf16)pv;
-                        dsf[a >> 1][4 * (a & 1) + c] = (__bf16)ds;
-                    }
+                for (int c = 0; c < 4; ++c) {
+                    const int r = 4 * a + c;
+                    const float pv = fast_exp2(s_acc[r] * c2 - l4[c]);
+                    const float ds = pv * (dp_acc[r] - d4[c]);
+                    pf[a >> 1][4 * (a & 1) + c] = (__bf16)pv;
+                    dsf[a >> 1][4 * (a & 1) + c] = (__bf16)ds;
                 }
+            }
 #pragma unroll
-                for (int m = 0; m < 2; ++m) {
+            for (int m = 0; m < 2; ++m) {
 #pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        const bf16x8_t adt = *reinterpret_cast<const bf16x8_t*>(
-                            reinterpret_cast<const char*>(do_tr) + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
-                        const bf16x8_t aqt = *reinterpret_cast<const bf16x8_t*>(
-                            reinterpret_cast<const char*>(q_tr) + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
-                        dv_acc[dt] = mfma_32x32x16(adt, pf[m], dv_acc[dt]);
-                        dk_acc[dt] = mfma_32x32x16(aqt, dsf[m], dk_acc[dt]);
-                    }
+                for (int dt = 0; dt < DT; ++dt) {
+                    const bf16x8_t adt = *reinterpret_cast<const bf16x8_t*>(do_tr + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
+                    const bf16x8_t aqt = *reinterpret_cast<const bf16x8_t*>(q_tr + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
+                    dv_acc[dt] = mfma_32x32x16(adt, pf[m], dv_acc[dt]);
+                    dk_acc[dt] = mfma_32x32x16(aqt, dsf[m], dk_acc[dt]);
                 }
             }
         }
@@ -226,7 +250,28 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(const AttnParam
         __syncthreads();
     }
 
-    if (key < p.total_k) {
+    // ---- sum the two wavefronts of each key group (fixed order), then store -------------------------
+    float* red = reinterpret_cast<float*>(smem) + (size_t)kgp * (16 * DT * 64) + lane;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        f32x16_t* acc = which == 0 ? dk_acc : dv_acc;
+        if (sub == 1) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) red[(dt * 16 + r) * 64] = acc[dt][r];
+        }
+        __syncthreads();
+        if (sub == 0) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[dt][r] += red[(dt * 16 + r) * 64];
+        }
+        __syncthreads();
+    }
+
+    if (sub == 0 && key < p.total_k) {
         __bf16* dkr = p.dk + (int64_t)key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * g;
         __bf16* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
 #pragma unroll
@@ -246,19 +291,21 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(const AttnParam
 // ---------------------------------------------------------------------------------------------
 // 3. dQ
 // ---------------------------------------------------------------------------------------------
+// 8 wavefronts, two per SIMD, 32 queries each (256 per workgroup); the first four stage K (rows and the
+// transposed copy), the last four stage V.  Double-buffered LDS, one barrier per 64-key tile.
 template <int D>
-__global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnParams p) {
-    constexpr int BM = 128;
+__global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p) {
+    constexpr int BM = 256;
     constexpr int BN = 64;
     constexpr int STR = D + 8;
     constexpr int KS = D / 16;
     constexpr int DT = D / 32;
     constexpr int ITEMS = 16 * (D / 8);
 
-    __shared__ __attribute__((aligned(16))) uint16_t k_rm[BN * STR];
-    __shared__ __attribute__((aligned(16))) uint16_t v_rm[BN * STR];
-    __shared__ __attribute__((aligned(16))) uint16_t k_tr[D * BN];
-    __shared__ int range_lds[8];
+    __shared__ __attribute__((aligned(16))) uint16_t k_rm[2][BN * STR];
+    __shared__ __attribute__((aligned(16))) uint16_t v_rm[2][BN * STR];
+    __shared__ __attribute__((aligned(16))) uint16_t k_tr[2][D * BN];
+    __shared__ int range_lds[16];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -279,7 +326,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnParams 
         wmin = min(wmin, __shfl_xor(wmin, off, 64));
         wmax = max(wmax, __shfl_xor(wmax, off, 64));
     }
-    if (lane == 0) { range_lds[wave] = wmin; range_lds[4 + wave] = wmax; }
+    if (lane == 0) { range_lds[wave] = wmin; range_lds[8 + wave] = wmax; }
 
     const int tl = tq < p.total_q ? tq : p.total_q - 1;
     bf16x8_t qf[KS], dof[KS];
@@ -296,8 +343,9 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnParams 
     const float delta = p.delta[(int64_t)head * p.total_q + tl];
 
     __syncthreads();
-    int bmin = min(min(range_lds[0], range_lds[1]), min(range_lds[2], range_lds[3]));
-    int bmax = max(max(range_lds[4], range_lds[5]), max(range_lds[6], range_lds[7]));
+    int bmin = 0x7fffffff, bmax = 0;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) { bmin = min(bmin, range_lds[w]); bmax = max(bmax, range_lds[8 + w]); }
     if (bmax <= bmin) { bmin = 0; bmax = 0; }
     const int kt0 = bmin & ~(BN - 1);
     const int n_tiles = (bmax - kt0 + BN - 1) / BN;
@@ -308,37 +356,46 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnParams 
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq_acc[dt][r] = 0.f;
 
-    const int quad = tid / (D / 8), dg = tid % (D / 8);
-    uint4 kraw[4], vraw[4];
+    const bool k_role = tid < 256;
+    const int ltid = tid & 255;
+    const int quad = ltid / (D / 8), dg = ltid % (D / 8);
+    uint4 raw[4];
     const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
     const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
 
     auto load_tile = [&](int kt) {
-        if (tid < ITEMS) {
-            load_quad<D>(kraw, kbase, p.k_st, kt, p.total_k, quad, dg);
-            load_quad<D>(vraw, vbase, p.v_st, kt, p.total_k, quad, dg);
+        if (ltid < ITEMS) {
+            if (k_role) load_quad<D>(raw, kbase, p.k_st, kt, p.total_k, quad, dg);
+            else load_quad<D>(raw, vbase, p.v_st, kt, p.total_k, quad, dg);
         }
     };
-    auto store_tile = [&]() {
-        if (tid < ITEMS) {
-            store_rows<STR>(kraw, k_rm, quad, dg);
-            store_rows<STR>(vraw, v_rm, quad, dg);
-            store_transposed(kraw, reinterpret_cast<char*>(k_tr), quad, dg);
+    auto store_tile = [&](int buf) {
+        if (ltid < ITEMS) {
+            if (k_role) {
+                store_rows<STR>(raw, k_rm[buf], quad, dg);
+                store_transposed(raw, reinterpret_cast<char*>(k_tr[buf]), quad, dg);
+            } else {
+                store_rows<STR>(raw, v_rm[buf], quad, dg);
+            }
         }
     };
 
     if (n_tiles > 0) {
         load_tile(kt0);
-        store_tile();
+        store_tile(0);
     }
     __syncthreads();
 
+    const float c2 = p.scale_log2;
     for (int it = 0; it < n_tiles; ++it) {
         const int kt = kt0 + it * BN;
+        const int buf = it & 1;
         if (it + 1 < n_tiles) load_tile(kt + BN);
 
-        const bool wave_active = (kt < wmax) && (kt + BN > wmin);
-        if (wave_active) {
+        if ((kt < wmax) && (kt + BN > wmin)) {
+            const uint16_t* a_k = k_rm[buf] + l32 * STR + 8 * g;
+            const uint16_t* a_v = v_rm[buf] + l32 * STR + 8 * g;
+            const char* a_kt = reinterpret_cast<const char*>(k_tr[buf]);
             f32x16_t s_acc[2], dp_acc[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
@@ -348,35 +405,41 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(const AttnParams 
             for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(k_rm + (32 * t + l32) * STR + 16 * ks + 8 * g);
-                    const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(v_rm + (32 * t + l32) * STR + 16 * ks + 8 * g);
+                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(a_k + 32 * t * STR + 16 * ks);
                     s_acc[t] = mfma_32x32x16(ak, qf[ks], s_acc[t]);
+                    const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(a_v + 32 * t * STR + 16 * ks);
                     dp_acc[t] = mfma_32x32x16(av, dof[ks], dp_acc[t]);
                 }
             }
-            bf16x8_t dsf[4];
+            if (__any((kt < klo) || (kt + BN > khi))) {
+                int rel0 = kt + 4 * g - klo;
+                asm volatile("" : "+v"(rel0));   // opaque: keeps the compares inside this branch
+                const unsigned len = (unsigned)(khi - klo);
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kj = kt + 32 * t + 8 * (r >> 2) + 4 * g + (r & 3);
-                    float pv = fast_exp2(s_acc[t][r] * p.scale_log2 - lse2);
-                    if (kj < klo || kj >= khi) pv = 0.f;
-                    const float ds = pv * (dp_acc[t][r] - delta);
-                    dsf[2 * t + (r >> 3)][r & 7] = (__bf16)ds;
-                }
+                    for (int r = 0; r < 16; ++r) {
+                        const unsigned rel = (unsigned)(rel0 + 32 * t + 8 * (r >> 2) + (r & 3));
+                        if (rel >= len) s_acc[t][r] = -INFINITY;
+                    }
+            }
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
+                const int t = m >> 1, r0 = 8 * (m & 1);
+                bf16x8_t dsf;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float pv = fast_exp2(s_acc[t][r0 + e] * c2 - lse2);
+                    dsf[e] = (__bf16)(pv * (dp_acc[t][r0 + e] - delta));
+                }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t akt = *reinterpret_cast<const bf16x8_t*>(
-                        reinterpret_cast<const char*>(k_tr) + chunk_unit_offset<64>(32 * dt + l32, m, g));
-                    dq_acc[dt] = mfma_32x32x16(akt, dsf[m], dq_acc[dt]);
+                    const bf16x8_t akt = *reinterpret_cast<const bf16x8_t*>(a_kt + chunk_unit_offset<64>(32 * dt + l32, m, g));
+                    dq_acc[dt] = mfma_32x32x16(akt, dsf, dq_acc[dt]);
                 }
             }
         }
-        __syncthreads();
-        if (it + 1 < n_tiles) store_tile();
+        if (it + 1 < n_tiles) store_tile(buf ^ 1);
         __syncthreads();
     }
 
@@ -406,13 +469,13 @@ template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) 
     }
     if (all || (stages & MI_ATTN_BWD_DKDV)) {
         const int64_t grid = (((int64_t)p.total_k + 127) / 128) * p.nkv;
-        attn_bwd_dkdv_kernel<D><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
+        attn_bwd_dkdv_kernel<D><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         int rc = mi_check_launch("attn_bwd_dkdv");
         if (rc != MI_OK) return rc;
     }
     if (all || (stages & MI_ATTN_BWD_DQ)) {
-        const int64_t grid = (((int64_t)p.total_q + 127) / 128) * p.nq;
-        attn_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(p);
+        const int64_t grid = (((int64_t)p.total_q + 255) / 256) * p.nq;
+        attn_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         return mi_check_launch("attn_bwd_dq");
     }
     return MI_OK;
