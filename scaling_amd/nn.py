@@ -1,0 +1,336 @@
+"""Drop-in layer modules at tensor-parallel size 1 backed by the gfx950 kernels.
+
+Constructor arguments, forward signatures, sub-module names and parameter names follow the
+reference's modules (see each class), so state dicts and the per-layer checkpoint files of the
+reference load unchanged.  Linear projections stay on PyTorch-ROCm matmul.  Everything else on the
+path (norm, rotary, attention core, SwiGLU) runs the HIP kernels of this package; options the kernels
+do not cover raise `NotImplementedError` instead of silently taking another path.
+"""
+
+import math
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from . import ops
+from .config import (LayerNormConfig, MaskedSoftmaxConfig, MaskedSoftmaxKernel, NormType,
+                     RelativePositionEmbeddingType, RotaryConfig)
+
+InitMethod = Callable[[torch.Tensor], torch.Tensor]
+
+
+def _default_device(device, topology=None) -> torch.device:
+    if topology is not None:
+        raise NotImplementedError("scaling_amd modules cover tensor-parallel size 1 only; pass topology=None")
+    if device is not None:
+        return torch.device(device)
+    return torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() else torch.device("cpu")
+
+
+class _Linear(torch.nn.Module):
+    """weight [out, in] (+ bias [out]): the parameter layout of the reference's Column/RowParallelLinear
+    at model-parallel size 1 (core/nn/linear/column_parallel_linear.py:109-116, row_parallel_linear.py:117-124)."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool, device, dtype, init_method: InitMethod):
+        super().__init__()
+        self.weight = torch.nn.Parameter(torch.empty(out_features, in_features, device=device, dtype=dtype))
+        init_method(self.weight)
+        if bias:
+            self.bias = torch.nn.Parameter(torch.zeros(out_features, device=device, dtype=dtype))
+        else:
+            self.register_parameter("bias", None)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(x, self.weight, self.bias)
+
+
+class RMSNorm(torch.nn.Module):
+    """Mirror of core/nn/norm/rms_norm.py:19-106 (u-muP and sequence-parallel branches excluded)."""
+
+    def __init__(self, dimensions: int, device: Optional[torch.device] = None, config: Optional[LayerNormConfig] = None,
+                 dtype: torch.dtype = torch.float32, topology=None, umup_on_residual: Optional[bool] = None) -> None:
+        super().__init__()
+        device = _default_device(device, topology)
+        self.config = config if config is not None else LayerNormConfig()
+        self.eps = self.config.layernorm_epsilon
+        self.topology = None
+        self.weight = torch.nn.Parameter(torch.ones(dimensions, dtype=dtype, device=device))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.rms_norm(x, self.weight, self.eps)
+
+
+def get_norm(norm_type: NormType, layernorm_config: Optional[LayerNormConfig], dimensions: int,
+             device: Optional[torch.device], dtype: torch.dtype, bitfit_bias_name: Optional[str] = None,
+             topology=None, umup_on_residual: Optional[bool] = None) -> RMSNorm:
+    """Mirror of core/nn/norm/get_norm.py:17-49; only the RMS branch has a kernel in this package."""
+    if norm_type == NormType.RMS:
+        return RMSNorm(dimensions=dimensions, device=device, config=layernorm_config, dtype=dtype, topology=topology)
+    raise NotImplementedError(f"norm_type {norm_type} has no HIP kernel in this package (supported: rms)")
+
+
+class RotaryEmbedding(torch.nn.Module):
+    """Mirror of core/nn/rotary.py:142-213: fp32 table construction, tables cast to the module dtype and
+    kept as non-persistent buffers `cos` / `sin` of shape [max_seq, 1, 1, dim]."""
+
+    def __init__(self, config: RotaryConfig, device: torch.device, dtype: torch.dtype = torch.float32) -> None:
+        super().__init__()
+        assert config.dimensions > 1, "RotaryEmbedding cannot use `dim` == 1"
+        dim, n = config.dimensions, config.max_seq_length
+        self.inv_freq = 1.0 / (config.base ** (torch.arange(0, dim, 2).float() / dim))
+        ang = torch.outer(torch.arange(n).float(), self.inv_freq)
+        ang = torch.cat((ang, ang), dim=-1).to(device).float()
+        self.register_buffer("cos", ang.cos().reshape(n, 1, 1, dim).to(dtype), persistent=False)
+        self.register_buffer("sin", ang.sin().reshape(n, 1, 1, dim).to(dtype), persistent=False)
+        self.dimensions = dim
+        self.max_seq_length = n
+
+    def tables(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        return self.cos.view(self.max_seq_length, self.dimensions), self.sin.view(self.max_seq_length, self.dimensions)
+
+    def rotate_tokens(self, x: torch.Tensor, position_ids: Optional[torch.Tensor], seq_len: int) -> torch.Tensor:
+        """x [tokens, heads, head_dim] (tokens = flattened (b s)); position_ids int64 [tokens] or None."""
+        cos, sin = self.tables()
+        return ops.rotary_embedding(x, cos, sin, position_ids, seq_len_for_null_ids=seq_len)
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, query_position_ids: Optional[torch.Tensor] = None,
+                key_position_ids: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        """query [s_q, b, n_q, d], key [s_k, b, n_kv, d], ids [s, b] as in the reference."""
+        def one(x, ids):
+            s, b, n, d = x.shape
+            tok = x.permute(1, 0, 2, 3).reshape(b * s, n, d)
+            flat = None if ids is None else ids.transpose(0, 1).reshape(-1).contiguous()
+            return self.rotate_tokens(tok, flat, s).view(b, s, n, d).permute(1, 0, 2, 3)
+        return one(query, query_position_ids), one(key, key_position_ids)
+
+
+class ParallelSwiGLUMLP(torch.nn.Module):
+    """Mirror of core/nn/mlp.py:149-282: dense_out(silu(dense_in(x)) * siglu_weight(x))."""
+
+    def __init__(self, io_features: int, intermediate_feature_factor: float, bias: bool = True,
+                 device: Optional[torch.device] = None, dtype: torch.dtype = torch.float32, topology=None,
+                 init_method: InitMethod = torch.nn.init.xavier_normal_, bitfit_bias_name: Optional[str] = None,
+                 umup_mult: Optional[float] = None, umup_is_first_layer: Optional[bool] = None,
+                 umup_is_last_layer: Optional[bool] = None, umup_on_residual: Optional[bool] = None,
+                 fp8_config=None, fp8_config_dense_out=None) -> None:
+        super().__init__()
+        device = _default_device(device, topology)
+        if fp8_config is not None or fp8_config_dense_out is not None or bitfit_bias_name is not None:
+            raise NotImplementedError("fp8 / bitfit options are outside the layer hot path of this package")
+        assert float(int(io_features * intermediate_feature_factor)) == io_features * intermediate_feature_factor, \
+            "io_features * intermediate_feature_factor does not result in a natural number for feature dimensions"
+        inter = int(io_features * intermediate_feature_factor)
+        self.topology = None
+        self.dense_in = _Linear(io_features, inter, bias, device, dtype, init_method)
+        self.siglu_weight = _Linear(io_features, inter, bias, device, dtype, init_method)
+        self.dense_out = _Linear(inter, io_features, bias, device, dtype, init_method)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.dense_out(ops.swiglu(self.dense_in(x), self.siglu_weight(x)))
+
+
+class KVCache:
+    """Pre-allocated cache of post-rotary K and un-repeated V, [batch, max_ctx, n_kv, d], replacing the
+    reference's per-step torch.cat (core/nn/attention/attention.py:862-869)."""
+
+    def __init__(self, batch: int, max_ctx: int, n_kv: int, head_dim: int, dtype, device) -> None:
+        self.k = torch.zeros(batch, max_ctx, n_kv, head_dim, dtype=dtype, device=device)
+        self.v = torch.zeros(batch, max_ctx, n_kv, head_dim, dtype=dtype, device=device)
+        self.ctx_len = torch.zeros(batch, dtype=torch.int32, device=device)
+        self.length = 0          # host copy of the (uniform) context length
+        self.max_ctx = max_ctx
+        self.workspace: Optional[torch.Tensor] = None
+
+
+class ParallelSelfAttention(torch.nn.Module):
+    """Mirror of core/nn/attention/attention.py:509-969 for `masked_softmax.kernel = hip`.
+
+    Same constructor arguments and forward signature.  Differences, all documented errors rather than
+    silent fall-backs: attention-probability dropout, attention-score manipulation, LoRA, local
+    attention windows, u-muP, fp8, `rotary_complex` and LayerNorm query/key norm are not available;
+    the dtype must be bfloat16.  The KV cache is pre-allocated (see `KVCache`), supports batches of
+    single-document rows and is filled/extended in place.
+    """
+
+    def __init__(self, hidden_size: int, num_attention_heads: int, masked_softmax_config: MaskedSoftmaxConfig,
+                 causal: bool = True, num_local_attention_heads: int = 0,
+                 local_attention_window_size: Optional[int] = None, dropout_attention_probs: float = 0.0,
+                 rotary_config: Optional[RotaryConfig] = None,
+                 relative_position_embedding_type: RelativePositionEmbeddingType = RelativePositionEmbeddingType.ROTARY,
+                 bias: bool = True, device: Optional[torch.device] = None, dtype: torch.dtype = torch.float32,
+                 topology=None, init_method: InitMethod = torch.nn.init.xavier_normal_,
+                 bitfit_bias_name: Optional[str] = None, lora_config=None, norm_type: NormType = NormType.LAYERNORM,
+                 key_query_norm: bool = False, layernorm_config: Optional[LayerNormConfig] = None,
+                 qkv_in_one: bool = True, num_kv_heads: Optional[int] = None, use_matmul: bool = False,
+                 umup_mult: Optional[float] = None, umup_is_first_layer: Optional[bool] = None,
+                 umup_is_last_layer: Optional[bool] = None, umup_on_residual: Optional[bool] = None,
+                 fp8_config=None, fp8_config_dense_out=None, max_cache_length: Optional[int] = None) -> None:
+        super().__init__()
+        self._device = _default_device(device, topology)
+        assert hidden_size % num_attention_heads == 0, \
+            f"hidden size ({hidden_size}) must be divisible by num_attention_heads ({num_attention_heads})"
+        if masked_softmax_config.kernel != MaskedSoftmaxKernel.HIP:
+            raise NotImplementedError(
+                f"this module implements masked_softmax.kernel = 'hip' only (got '{masked_softmax_config.kernel.value}'); "
+                "the other kernels live in the reference implementation")
+        if dropout_attention_probs != 0.0:
+            raise NotImplementedError("dropout on attention probabilities is not available with the hip kernel")
+        if num_local_attention_heads > 0 or lora_config is not None or fp8_config is not None or \
+                fp8_config_dense_out is not None or bitfit_bias_name is not None:
+            raise NotImplementedError("local attention, LoRA, fp8 and bitfit are outside the hip kernel's scope")
+        if relative_position_embedding_type == RelativePositionEmbeddingType.ROTARY_COMPLEX:
+            raise NotImplementedError("rotary_complex has no HIP kernel yet (supported: none, rotary)")
+        if dtype != torch.bfloat16:
+            raise NotImplementedError("the hip attention kernels compute in bfloat16; set precision: bfloat16")
+
+        self.hidden_size_per_attention_head = hidden_size // num_attention_heads
+        self.num_attention_heads = num_attention_heads
+        self.num_attention_heads_per_partition = num_attention_heads
+        self.causal = causal
+        self.masked_softmax_config = masked_softmax_config
+        self.use_flash_attention = False
+        self.dtype = dtype
+        self.lora_config = None
+        self.topology = None
+        self.qkv_in_one = qkv_in_one
+        self.num_kv_heads = num_kv_heads
+        if num_kv_heads:
+            assert not qkv_in_one, "for a differing number of kv heads, qkv cannot be stored in one"
+            assert num_attention_heads % num_kv_heads == 0
+            self.num_kv_heads_per_partition = num_kv_heads
+        else:
+            self.num_kv_heads_per_partition = num_attention_heads
+        self.num_repeat_kv = num_attention_heads // self.num_kv_heads_per_partition
+        d = self.hidden_size_per_attention_head
+        if d not in (32, 64, 96, 128):
+            raise NotImplementedError(f"head_dim {d} is not supported by the hip attention kernels (32, 64, 96, 128)")
+
+        if qkv_in_one:
+            self.query_key_value = _Linear(hidden_size, 3 * hidden_size, bias, self._device, dtype, init_method)
+        else:
+            self.query = _Linear(hidden_size, hidden_size, bias, self._device, dtype, init_method)
+            self.key = _Linear(hidden_size, hidden_size // self.num_repeat_kv, bias, self._device, dtype, init_method)
+            self.value = _Linear(hidden_size, hidden_size // self.num_repeat_kv, bias, self._device, dtype, init_method)
+
+        self.rotary_embedding: Optional[RotaryEmbedding] = None
+        if relative_position_embedding_type == RelativePositionEmbeddingType.ROTARY:
+            assert rotary_config is not None
+            self.rotary_embedding = RotaryEmbedding(config=rotary_config, device=self._device, dtype=dtype)
+
+        self.key_query_norm = key_query_norm
+        self.norm_query = self.norm_key = None
+        if key_query_norm:
+            self.norm_query = get_norm(norm_type, layernorm_config, d, self._device, dtype)
+            self.norm_key = get_norm(norm_type, layernorm_config, d, self._device, dtype)
+
+        # softmax_fn scale: alpha * masked_softmax.scale (attention.py:297 with masked_softmax.py:21-22)
+        self.query_key_scaling_factor = 1.0 / math.sqrt(d)
+        self.softmax_scale = self.query_key_scaling_factor * masked_softmax_config.scale
+        self.dense = _Linear(hidden_size, hidden_size, bias, self._device, dtype, init_method)
+        self.cache: Dict[int, Optional[KVCache]] = dict()
+        self.max_cache_length = max_cache_length
+
+    # ---- reference API that callers of every ParallelSelfAttention instance use ---------------------
+    def merge_lora_weights(self) -> None:  # core/trainer/trainer.py:87-92 calls this unconditionally
+        return None
+
+    # ---- helpers --------------------------------------------------------------------------------
+    def _project(self, x: torch.Tensor):
+        b, s, _ = x.shape
+        nq, nkv, d = self.num_attention_heads, self.num_kv_heads_per_partition, self.hidden_size_per_attention_head
+        if self.qkv_in_one:
+            qkv = self.query_key_value(x).view(b * s, nq, 3 * d)       # per head: q then k then v (attention.py:790-796)
+            return qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:]
+        q = self.query(x).view(b * s, nq, d)
+        k = self.key(x).view(b * s, nkv, d)
+        v = self.value(x).view(b * s, nkv, d)
+        return q, k, v
+
+    @staticmethod
+    def _rows_are_single_documents(cu: torch.Tensor, b: int, s: int) -> bool:
+        return cu.numel() == b + 1 and bool(torch.equal(cu.cpu(), torch.arange(0, b * s + 1, s, dtype=cu.dtype)))
+
+    def forward(self, x: torch.Tensor, cumulative_seq_lengths: torch.Tensor, position_ids: Optional[torch.Tensor],
+                cumulative_seq_lengths_key: Optional[torch.Tensor] = None, use_cache: bool = False,
+                reset_cache: bool = False, cache_index: int = 0, attention_scores_manipulation=None,
+                attentions_score_manipulation_log_additive=True) -> torch.Tensor:
+        if attention_scores_manipulation is not None:
+            raise NotImplementedError("attention_scores_manipulation is not available with the hip kernel")
+        b, s, hidden = x.shape
+        nq, nkv, d = self.num_attention_heads, self.num_kv_heads_per_partition, self.hidden_size_per_attention_head
+        q, k, v = self._project(x)
+        if self.key_query_norm:
+            q = self.norm_query(q)
+            k = self.norm_key(k)
+        pos = None if position_ids is None else position_ids.reshape(-1).contiguous()
+        cu = cumulative_seq_lengths.to(torch.int32)
+
+        if use_cache:
+            if not self.causal:
+                raise ValueError("KV caching is only supported for causal attention.")
+            assert self._rows_are_single_documents(cu, b, s), "sequence packing is not supported with cache"
+            if not reset_cache:
+                return self.dense(self._decode_step(q, k, v, pos, b, s, cache_index).view(b, s, nq * d))
+        elif reset_cache:
+            self.cache[cache_index] = None
+
+        if (self.rotary_embedding is not None and not use_cache and not torch.is_grad_enabled() and pos is not None
+                and self.rotary_embedding.dimensions == d and d in (64, 128)):
+            # inference without cache: rotary is applied while the kernel loads Q and K
+            cos, sin = self.rotary_embedding.tables()
+            cu_k = None if cumulative_seq_lengths_key is None else cumulative_seq_lengths_key.to(torch.int32)
+            ctx, _ = ops.attention_forward(q, k, v, cu, cu_k, self.causal, self.softmax_scale, rotary=(cos, sin, pos, pos))
+            return self.dense(ctx.view(b, s, nq * d))
+        if self.rotary_embedding is not None:
+            q = self.rotary_embedding.rotate_tokens(q, pos, s)
+            k = self.rotary_embedding.rotate_tokens(k, pos, s)
+        if use_cache:  # prefill: keep post-rotary K and V (attention.py:861-862)
+            self._fill_cache(k, v, b, s, cache_index)
+        ctx = ops.attention(q, k, v, cu, None if cumulative_seq_lengths_key is None else cumulative_seq_lengths_key.to(torch.int32),
+                            self.causal, self.softmax_scale)
+        return self.dense(ctx.view(b, s, nq * d))
+
+    # ---- KV cache ----------------------------------------------------------------------------------
+    def _cache_capacity(self) -> int:
+        if self.max_cache_length is not None:
+            return self.max_cache_length
+        if self.rotary_embedding is not None:
+            return self.rotary_embedding.max_seq_length
+        raise ValueError("set max_cache_length when the module has no rotary table to size the cache from")
+
+    def _fill_cache(self, k: torch.Tensor, v: torch.Tensor, b: int, s: int, cache_index: int) -> None:
+        nkv, d = self.num_kv_heads_per_partition, self.hidden_size_per_attention_head
+        cap = max(self._cache_capacity(), s)
+        cache = self.cache.get(cache_index)
+        if cache is None or cache.k.shape[0] != b or cache.max_ctx < cap:
+            cache = KVCache(b, cap, nkv, d, k.dtype, k.device)
+            self.cache[cache_index] = cache
+        cache.k[:, :s].copy_(k.detach().view(b, s, nkv, d))
+        cache.v[:, :s].copy_(v.detach().view(b, s, nkv, d))
+        cache.length = s
+        cache.ctx_len.fill_(s)
+
+    def _decode_step(self, q, k, v, pos, b: int, s: int, cache_index: int) -> torch.Tensor:
+        cache = self.cache.get(cache_index)
+        assert cache is not None, "decode step without a prefilled cache"
+        if s != 1:
+            raise NotImplementedError("cached attention extends the context one token per sequence and step")
+        assert cache.k.shape[0] == b and cache.length + 1 <= cache.max_ctx, "KV cache too small or batch changed"
+        nq, nkv, d = self.num_attention_heads, self.num_kv_heads_per_partition, self.hidden_size_per_attention_head
+        cache.length += 1
+        cache.ctx_len.add_(1)
+        rotary = None
+        if self.rotary_embedding is not None:
+            if pos is None:
+                pos = torch.full((b,), cache.length - 1, dtype=torch.int64, device=q.device)
+            cos, sin = self.rotary_embedding.tables()
+            if self.rotary_embedding.dimensions == d and d in (64, 128):
+                rotary = (cos, sin, pos)
+            else:  # partial rotary: stand-alone kernel, then a plain append
+                q = self.rotary_embedding.rotate_tokens(q, pos, 1)
+                k = self.rotary_embedding.rotate_tokens(k, pos, 1)
+        if cache.workspace is None:
+            cache.workspace = ops.decode_workspace(b, nq, d, cache.max_ctx, q.device)
+        return ops.decode_attention(q.contiguous(), cache.k, cache.v, cache.ctx_len, k.contiguous(), v.contiguous(),
+                                    rotary=rotary, softmax_scale=self.softmax_scale, workspace=cache.workspace)

@@ -1,0 +1,150 @@
+"""GPU parity of the drop-in modules (norm -> attention -> residual -> norm -> SwiGLU MLP -> residual)
+and of the cached decode loop against the CPU oracle."""
+
+import pytest
+import torch
+
+import oracle
+from scaling_amd import config as C
+from scaling_amd import data as D
+from scaling_amd.inference import TransformerInferenceModule
+from scaling_amd.layer import TransformerLayer, TransformerLayerIO
+from tests.parity import check, metrics
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _arch(**kw):
+    d = dict(vocab_size=96, hidden_size=256, num_layers=2, num_attention_heads=4, attention_qkv_in_one=False,
+             norm_type="rms", mlp_type="swiglu", mlp_factor=2.6875, attention_bias=False, mlp_bias=False,
+             precision="bfloat16", sequence_length=128, rotary_embedding_base=10000,
+             masked_softmax={"kernel": "hip", "softmax_in_fp32": True}, weight_tying=False)
+    d.update(kw)
+    return C.TransformerArchitectureConfig.from_dict(d)
+
+
+def _spec(cfg, dtype):
+    return oracle.LayerSpec(hidden_size=cfg.hidden_size, num_attention_heads=cfg.num_attention_heads,
+                            num_kv_heads=cfg.attention_num_kv_heads, qkv_in_one=cfg.attention_qkv_in_one, norm_type="rms",
+                            mlp_type="swiglu", layernorm_epsilon=cfg.layernorm.layernorm_epsilon,
+                            rotary_base=cfg.rotary_embedding_base, sequence_length=cfg.sequence_length, causal=cfg.causal,
+                            softmax_in_fp32=True, dtype=dtype)
+
+
+def _seeded_layer(cfg, seed):
+    g = torch.Generator().manual_seed(seed)
+
+    def init(w):
+        w.data.copy_((torch.randn(w.shape, generator=g) * 0.02).to(w.dtype))
+        return w
+
+    layer = TransformerLayer(cfg, layer_index=0, init_method=init, device=DEV)
+    with torch.no_grad():   # perturb the norm weights so their gradient path is exercised non-trivially
+        for n in (layer.input_layernorm, layer.post_attention_layernorm):
+            n.weight.copy_((1 + 0.02 * torch.randn(n.weight.shape, generator=g)).to(n.weight.dtype))
+    return layer
+
+
+def _oracle_layer(cfg, weights, x, cu, pos, dy, dtype):
+    """Runs the oracle layer in `dtype` on the (bf16-rounded) weights and inputs; returns y, dx, dweights."""
+    spec = _spec(cfg, dtype)
+    w = {k: v.detach().cpu().to(dtype).clone().requires_grad_() for k, v in weights.items()}
+    xx = x.to(dtype).clone().requires_grad_()
+    # the module keeps its rotary tables in bf16 (reference behaviour); the oracle uses the same values
+    t = oracle.rotary_tables(spec.rotary_dim, spec.sequence_length, spec.rotary_base, torch.bfloat16)
+    tables = oracle.RotaryTables(t.cos.to(dtype), t.sin.to(dtype), t.dim)
+    y = oracle.transformer_layer(spec, w, xx, cu, pos, tables=tables)
+    y.backward(dy.to(dtype))
+    return y.detach(), xx.grad, {k: v.grad for k, v in w.items()}
+
+
+@pytest.mark.parametrize("name,kw,b,s,cuts", [
+    ("config1_mha", dict(), 2, 128, ()),                                                    # config 1 shape, bf16 on the GPU
+    ("gqa_packed", dict(hidden_size=512, num_attention_heads=8, attention_num_kv_heads=2, mlp_factor=2.5), 2, 96, (40, 130)),
+    ("fused_qkv_bias", dict(attention_qkv_in_one=True, attention_bias=True, mlp_bias=True), 1, 64, ()),
+])
+def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
+    print(f"case layer {name}", flush=True)
+    cfg = _arch(**kw)
+    layer = _seeded_layer(cfg, seed=0)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(b, s, cfg.hidden_size, generator=g).bfloat16()
+    dy = torch.randn(b, s, cfg.hidden_size, generator=g).bfloat16()
+    cu = torch.tensor(sorted(set(i * s for i in range(b + 1)) | set(cuts)), dtype=torch.int32)
+    pos = torch.zeros(b * s, dtype=torch.int64)
+    for a_, b_ in zip(cu[:-1].tolist(), cu[1:].tolist()):
+        pos[a_:b_] = torch.arange(b_ - a_)
+    pos = pos.view(b, s)
+    weights = {k: v for k, v in layer.state_dict().items()}
+    ref = _oracle_layer(cfg, weights, x, cu, pos, dy, torch.float32)
+    ref_o = _oracle_layer(cfg, weights, x, cu, pos, dy, torch.bfloat16)
+
+    xg = x.to(DEV).requires_grad_()
+    out = layer(TransformerLayerIO(activations=xg, position_ids=pos.to(DEV), cumulative_seq_lengths=cu.to(DEV)))
+    out.activations.backward(dy.to(DEV))
+    torch.cuda.synchronize()
+    check(f"{name}.y", out.activations, ref[0], ref_o[0])
+    check(f"{name}.dx", xg.grad, ref[1], ref_o[1])
+    for k, p in layer.named_parameters():
+        # parameter gradients sum over all tokens: compare against the reference's own bf16 error, with 25 % slack
+        m = metrics(p.grad, ref[2][k])
+        f = metrics(ref_o[2][k], ref[2][k], torch.bfloat16)
+        print(f"[parity] {name}.d{k}: mean_rel={m['mean_rel']:.3e} (reference bf16 order {f['mean_rel']:.3e})", flush=True)
+        assert m["finite"] and m["mean_rel"] <= max(1e-3, 1.25 * f["mean_rel"]), (k, m, f)
+
+
+def test_cached_generation_matches_uncached_and_oracle():
+    cfg = _arch(attention_num_kv_heads=2)
+    model = TransformerInferenceModule(cfg, device=DEV, init_std=0.2, seed=3)
+    prompt = [5, 17, 3, 90, 41, 8, 63]
+    tok_c, log_c = model.generate(6, prompt, use_cache=True)
+    tok_u, log_u = model.generate(6, prompt, use_cache=False)
+    assert tok_c == tok_u                                                    # the reference's own invariant
+    assert torch.allclose(log_c.float(), log_u.float(), rtol=1e-2, atol=1e-2)
+    # oracle: same weights with the reference's key names, teacher-forced on the GPU's own tokens; once in
+    # fp32 (the target) and once in the reference's bf16 operation order (the floor)
+    def oracle_logits(dtype):
+        sd = {k: v.detach().cpu().to(dtype) for k, v in model.state_dict().items()}
+        layers = [{k[len(f"_layers.{i + 1}."):]: v for k, v in sd.items() if k.startswith(f"_layers.{i + 1}.")} for i in range(2)]
+        om = {"embedding.weight": sd["_layers.0.embedding.weight"], "layers": layers,
+              "final": {"norm.weight": sd["_layers.3.norm.weight"]}, "lm_head.weight": sd["_layers.4.linear.weight"]}
+        spec = _spec(cfg, dtype)
+        full = torch.tensor([prompt + tok_c[0][:-1]])
+        cu = oracle.get_cumulative_seq_lengths(full)
+        with torch.no_grad():
+            out = oracle.layer._logits(spec, om, full, oracle.get_position_ids(full), cu, None, False, False)
+        return out[0, len(prompt) - 1:]
+
+    ref, ref_o = oracle_logits(torch.float32), oracle_logits(torch.bfloat16)
+    m, f = metrics(log_c[0], ref), metrics(ref_o, ref, torch.bfloat16)
+    print(f"[parity] generate.logits: max_abs={m['max_abs']:.3e} mean_rel={m['mean_rel']:.3e} | reference bf16 order: "
+          f"max_abs={f['max_abs']:.3e} mean_rel={f['mean_rel']:.3e}", flush=True)
+    assert m["mean_rel"] <= max(1e-3, 1.25 * f["mean_rel"])
+
+
+def test_batched_cached_decode_equals_single_sequences(tmp_path):
+    cfg = _arch(attention_num_kv_heads=1, hidden_size=512, num_attention_heads=4)   # head_dim 128, MQA
+    model = TransformerInferenceModule(cfg, device=DEV, init_std=0.1, seed=4)
+    g = torch.Generator().manual_seed(5)
+    prompts = torch.randint(1, cfg.vocab_size, (3, 19), generator=g)
+    toks, logits = model.generate(5, prompts)
+    for i in range(3):
+        t1, l1 = model.generate(5, prompts[i].tolist())
+        assert t1[0] == toks[i]
+        assert torch.allclose(l1[0].float(), logits[i].float(), rtol=1e-2, atol=1e-2)
+    # checkpoint round trip through the reference's per-layer file layout
+    model.save_checkpoint(tmp_path)
+    assert sorted(p.name for p in tmp_path.iterdir())[:3] == ["model_state_layer_0_EmbeddingInput.pt",
+                                                             "model_state_layer_1_TransformerLayer.pt",
+                                                             "model_state_layer_2_TransformerLayer.pt"]
+    other = TransformerInferenceModule(cfg, device=DEV, seed=99)
+    other.load_checkpoint(tmp_path)
+    t2, _ = other.generate(5, prompts)
+    assert t2 == toks
+
+
+def test_index_construction_on_device_is_bit_exact():
+    ids = torch.tensor([[1, 2, 3, 0, 1, 2], [1, 2, 3, 4, 5, 6], [1, 2, 3, 4, 5, 0]], device=DEV)
+    assert D.get_cumulative_seq_lengths(ids).tolist() == [0, 4, 6, 12, 18]
+    assert D.get_position_ids(ids).tolist() == [[0, 1, 2, 3, 0, 1], [0, 1, 2, 3, 4, 5], [0, 1, 2, 3, 4, 5]]

@@ -1,0 +1,150 @@
+"""CPU-only checks of the host-side mirror of the reference interface: config surface, index
+construction (bit-exact against the oracle and the reference's known answers), module / parameter
+names (checkpoint contract) and the documented error behaviour.  No kernel is launched."""
+
+import os
+
+import pytest
+import torch
+
+import oracle
+from scaling_amd import config as C
+from scaling_amd import data as D
+from scaling_amd.layer import LayerNormWrapper, TransformerLayer
+from scaling_amd.nn import ParallelSelfAttention, ParallelSwiGLUMLP, RMSNorm, RotaryEmbedding
+from tests.golden import known_answers as KA
+
+CPU = torch.device("cpu")
+
+
+def _arch(**kw):
+    d = dict(vocab_size=64, hidden_size=256, num_layers=2, num_attention_heads=4, attention_num_kv_heads=2,
+             attention_qkv_in_one=False, norm_type="rms", mlp_type="swiglu", mlp_factor=2.6875, attention_bias=False,
+             mlp_bias=False, precision="bfloat16", sequence_length=128, masked_softmax={"kernel": "hip"}, weight_tying=False)
+    d.update(kw)
+    return C.TransformerArchitectureConfig.from_dict(d)
+
+
+# ---- config surface ------------------------------------------------------------------------------------
+def test_masked_softmax_config_defaults_and_new_member():
+    c = C.MaskedSoftmaxConfig()
+    assert c.kernel == C.MaskedSoftmaxKernel.TORCH and c.softmax_in_fp32 is False and c.scale == 1.0
+    assert c.deterministic_flash_attn_bwd is False
+    assert [k.value for k in C.MaskedSoftmaxKernel] == ["torch", "flash_attention", "hip"]
+    assert C.MaskedSoftmaxConfig(kernel="hip").as_dict()["kernel"] == "hip"
+    with pytest.raises(Exception):
+        C.MaskedSoftmaxConfig(kernel="cuda")
+    with pytest.raises(Exception):
+        C.MaskedSoftmaxConfig(unknown_key=1)           # extra = forbid
+    with pytest.raises(Exception):
+        c.scale = 2.0                                  # frozen
+
+
+def test_architecture_config_round_trip_and_defaults():
+    a = C.TransformerArchitectureConfig()
+    assert a.norm_type == C.NormType.LAYERNORM and a.mlp_type == C.MLPType.DEFAULT and a.mlp_factor == 4.0
+    assert a.attention_qkv_in_one and a.attention_num_kv_heads is None and a.rotary_embedding_base == 10000
+    assert a.sequence_length == 2048 and a.causal and a.precision == C.Precision.FLOAT32
+    assert a.relative_position_embedding_type == C.RelativePositionEmbeddingType.ROTARY
+    assert C.RotaryConfig().max_seq_length == 2048 and C.LayerNormConfig().layernorm_epsilon == 1e-5
+    b = _arch()
+    assert C.TransformerArchitectureConfig.from_dict(b.as_dict()) == b
+    assert C.TransformerArchitectureConfig.from_str(b.as_str()) == b
+    assert b.rotary_config() == C.RotaryConfig(dimensions=64, max_seq_length=128, base=10000)
+    assert b.precision.dtype == torch.bfloat16
+
+
+def test_example_architecture_block_validates(tmp_path):
+    # the transformer_architecture block of the reference's example config (values restated as data)
+    block = {"weight_tying": False, "vocab_size": 128000, "hidden_size": 256, "num_layers": 4, "num_attention_heads": 2,
+             "rotary_embedding_base": 10000, "sequence_length": 64, "norm_type": "rms",
+             "relative_position_embedding_type": "rotary_complex", "attention_bias": False, "mlp_type": "swiglu",
+             "mlp_factor": 2.5, "mlp_bias": False, "masked_softmax": {"kernel": "flash_attention", "softmax_in_fp32": True,
+                                                                      "deterministic_flash_attn_bwd": False, "scale": 1.0},
+             "layernorm": {"optimization_type": "torch", "layernorm_epsilon": 1e-5}, "precision": "bfloat16",
+             "dropout_embedding": 0.1, "dropout_attention_probs": 0.1, "dropout_after_attention": 0.1,
+             "dropout_after_mlp": 0.1, "bitfit_bias_config": None, "softprompt_config": None, "adapter_config": None,
+             "lora_config": None, "image_encoder": False, "dropout_image_encoder": 0.0}
+    import yaml
+    f = tmp_path / "config.yml"
+    f.write_text(yaml.safe_dump({"transformer_architecture": block}))
+    a = C.architecture_from_config_file(f, kernel=None)
+    assert a.masked_softmax.kernel == C.MaskedSoftmaxKernel.FLASH_ATTENTION
+    assert C.architecture_from_config_file(f, kernel="hip").masked_softmax.kernel == C.MaskedSoftmaxKernel.HIP
+
+
+# ---- index construction -----------------------------------------------------------------------------------
+def test_data_utils_known_answers():
+    ids = torch.tensor(KA.TOKEN_IDS)
+    assert D.get_cumulative_seq_lengths(ids).tolist() == KA.CU_WITH_RESET
+    assert D.get_cumulative_seq_lengths(ids).dtype == torch.int32
+    assert D.get_cumulative_seq_lengths(ids, reset_attention_mask=False).tolist() == KA.CU_WITHOUT_RESET
+    assert D.get_position_ids(ids).tolist() == KA.POSITION_IDS_WITH_RESET
+    assert D.get_position_ids(ids, reset_position_ids=False).tolist() == KA.POSITION_IDS_WITHOUT_RESET
+    padded = D.add_cumulative_seq_lengths_padding(torch.tensor(KA.PADDING_INPUT), KA.PADDING_PAD_TO)
+    assert padded.tolist() == KA.PADDING_EXPECTED
+    assert D.remove_cumulative_seq_lengths_padding(padded).tolist() == KA.PADDING_INPUT
+
+
+def test_data_utils_bit_exact_against_oracle():
+    g = torch.Generator().manual_seed(0)
+    for _ in range(20):
+        b, s = int(torch.randint(1, 5, (1,), generator=g)), int(torch.randint(1, 40, (1,), generator=g))
+        ids = torch.randint(0, 4, (b, s), generator=g)
+        for reset in (True, False):
+            a, o = D.get_cumulative_seq_lengths(ids, reset), oracle.get_cumulative_seq_lengths(ids, reset)
+            assert a.dtype == o.dtype and torch.equal(a, o)
+            a, o = D.get_position_ids(ids, reset), oracle.get_position_ids(ids, reset)
+            assert a.dtype == o.dtype and torch.equal(a, o)
+
+
+# ---- module / checkpoint contract ---------------------------------------------------------------------------
+def test_layer_parameter_names_match_reference_checkpoint(golden_dir):
+    legacy = torch.load(os.path.join(golden_dir, "legacy_layer_state.pt"), weights_only=True)
+    layer = TransformerLayer(_arch(attention_qkv_in_one=True, attention_num_kv_heads=None), layer_index=0, device=CPU)
+    assert set(layer.state_dict().keys()) == set(legacy.keys())      # rotary tables are not persistent
+    names = [n for n, _ in layer.named_children()]
+    assert names == ["input_layernorm", "self_attention", "dropout_attention", "post_attention_layernorm", "mlp", "dropout_mlp"]
+    gqa = TransformerLayer(_arch(), layer_index=1, device=CPU).state_dict()
+    assert {"self_attention.query.weight", "self_attention.key.weight", "self_attention.value.weight",
+            "self_attention.dense.weight", "mlp.dense_in.weight", "mlp.siglu_weight.weight", "mlp.dense_out.weight",
+            "input_layernorm.weight", "post_attention_layernorm.weight"} == set(gqa.keys())
+    assert gqa["self_attention.key.weight"].shape == (128, 256) and gqa["mlp.dense_in.weight"].shape == (688, 256)
+    assert list(LayerNormWrapper(_arch(), layer_index=2, device=CPU).state_dict().keys()) == ["norm.weight"]
+    biased = ParallelSelfAttention(256, 4, C.MaskedSoftmaxConfig(kernel="hip"), rotary_config=C.RotaryConfig(dimensions=64),
+                                   dtype=torch.bfloat16, device=CPU)
+    assert "query_key_value.bias" in biased.state_dict() and "dense.bias" in biased.state_dict()
+    assert biased.state_dict()["query_key_value.weight"].shape == (768, 256)
+
+
+def test_rotary_tables_match_oracle_and_are_not_persistent():
+    r = RotaryEmbedding(C.RotaryConfig(dimensions=64, max_seq_length=128, base=500000), CPU, torch.bfloat16)
+    t = oracle.rotary_tables(64, 128, 500000, torch.bfloat16)
+    cos, sin = r.tables()
+    assert r.cos.shape == (128, 1, 1, 64) and torch.equal(cos, t.cos) and torch.equal(sin, t.sin)
+    assert len(r.state_dict()) == 0
+
+
+def test_unsupported_options_raise():
+    hip = C.MaskedSoftmaxConfig(kernel="hip")
+    with pytest.raises(NotImplementedError, match="hip"):
+        ParallelSelfAttention(256, 4, C.MaskedSoftmaxConfig(kernel="torch"), dtype=torch.bfloat16, device=CPU)
+    with pytest.raises(NotImplementedError, match="dropout"):
+        ParallelSelfAttention(256, 4, hip, dropout_attention_probs=0.1, dtype=torch.bfloat16, device=CPU)
+    with pytest.raises(NotImplementedError, match="bfloat16"):
+        ParallelSelfAttention(256, 4, hip, dtype=torch.float32, device=CPU)
+    with pytest.raises(NotImplementedError, match="rotary_complex"):
+        ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU,
+                              relative_position_embedding_type=C.RelativePositionEmbeddingType.ROTARY_COMPLEX)
+    with pytest.raises(AssertionError, match="kv heads"):
+        ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, num_kv_heads=2, qkv_in_one=True,
+                              rotary_config=C.RotaryConfig(dimensions=64))
+    with pytest.raises(AssertionError):
+        ParallelSwiGLUMLP(10, 0.33, device=CPU)
+    with pytest.raises(NotImplementedError, match="swiglu"):
+        TransformerLayer(_arch(mlp_type="default"), 0, device=CPU)
+    with pytest.raises(NotImplementedError, match="rms"):
+        TransformerLayer(_arch(norm_type="layernorm"), 0, device=CPU)
+    with pytest.raises(NotImplementedError):
+        TransformerLayer(_arch(umup={"enable": True}), 0, device=CPU)
+    assert RMSNorm(16, CPU).weight.tolist() == [1.0] * 16
