@@ -195,6 +195,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 1 GiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path; this build uses no collectives, so --gpus must be 1",
@@ -205,6 +207,14 @@ def main():
     from scaling_amd import _lib
     _lib.require_device()
     torch.cuda.set_device(0)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        ms = time_gpu(lambda: dst.copy_(src), args.steps, args.warmup)
+        print(json.dumps({"calibration": "device copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "ms": ms,
+                          "GBs": 2 * (1 << 30) / ms / 1e6}))
+        return
 
     b, s, nq, nkv, d = 1, 8192, 32, 8, 128
     main_res = attention_case(b, s, nq, nkv, d, [0, s], args.steps, args.warmup)

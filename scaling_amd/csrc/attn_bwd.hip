@@ -156,9 +156,12 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     uint4 raw[4];
     float stat = 0.f;
 
+    // Query tiles are visited from the last one downwards: under a causal mask every key block of a
+    // document needs the document's last queries, so the workgroups that share an XCD start on the same
+    // tile and keep streaming the same Q / dO rows through that XCD's L2.
     const int total_iters = n_tiles * p.n_rep;
     auto load_tile = [&](int iter) {
-        const int rep = iter / n_tiles, qt = qt0 + (iter % n_tiles) * BQ;
+        const int rep = iter / n_tiles, qt = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ;
         const int head = kvh * p.n_rep + rep;
         if (ltid < ITEMS) {
             if (q_role) load_quad<D>(raw, p.q + (int64_t)head * p.q_sh, p.q_st, qt, p.total_q, quad, dg);
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     const float c2 = p.scale_log2;
 
     for (int iter = 0; iter < total_iters; ++iter) {
-        const int qs = qt0 + (iter % n_tiles) * BQ + 32 * sub;
+        const int qs = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ + 32 * sub;
         if (iter + 1 < total_iters) load_tile(iter + 1);
 
         if ((qs < wmax) && (qs + 32 > wmin)) {
