@@ -169,6 +169,123 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
     for (int i = threadIdx.x; i < hidden; i += kBlock) out[i] = dw_lds[i];
 }
 
+// Backward for wide rows: 1024 threads per block, TPR (128 or 256) threads per row, so 8 or 4 rows are in
+// flight per block and the per-thread slices (raw row vectors, packed weight, fp32 dweight) are small
+// enough for 16 wavefronts per compute unit; the number of per-block dweight partial rows stays <= 512.
+// One barrier per row step (both row sums travel through a double-buffered LDS slot).
+constexpr int kWideBlock = 1024;
+
+template <typename T, int TPR, int CH>
+__global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                          const T* __restrict__ dy, T* __restrict__ dx,
+                                                                          float* __restrict__ dw_partial, int64_t n_rows,
+                                                                          int hidden, float eps) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int RPB = kWideBlock / TPR;
+    constexpr int WPR = TPR / 64;      // wavefronts per row
+    extern __shared__ float dw_lds[];  // [hidden] dweight combine buffer, then [hidden] fp32 copy of the weight
+    __shared__ float2 part[2][16];     // [parity][wavefront]
+    float* w_lds = dw_lds + hidden;
+    const int tr = threadIdx.x % TPR;
+    const int rg = threadIdx.x / TPR;
+    const int wave = threadIdx.x >> 6;
+    const int vecs = hidden / V;
+    const float inv_h = 1.0f / (float)hidden;
+
+    // the weight is read from LDS where it is used: keeping it in registers would cost as many registers
+    // as the dweight accumulator and halve the number of resident wavefronts
+    float acc[CH][V];
+    for (int i = threadIdx.x; i < hidden; i += kWideBlock) w_lds[i] = Elem<T>::load1(w + i);
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[c][i] = 0.f;
+    __syncthreads();
+    const int64_t row_step = (int64_t)gridDim.x * RPB;
+    const int64_t iters = (n_rows + row_step - 1) / row_step;
+    for (int64_t it = 0; it < iters; ++it) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
+        const uint4* gr = reinterpret_cast<const uint4*>(dy + (row_ok ? row : 0) * hidden);
+        uint4 xraw[CH], graw[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int v = c * TPR + tr;
+            const bool ok = row_ok && v < vecs;
+            xraw[c] = ok ? xr[v] : make_uint4(0, 0, 0, 0);
+            graw[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
+        }
+        float ss = 0.f, dot = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float xf[V], gf[V], wf[V];
+            Elem<T>::unpack(xraw[c], xf);
+            Elem<T>::unpack(graw[c], gf);
+            const int v0 = (c * TPR + tr < vecs ? c * TPR + tr : 0) * V;
+#pragma unroll
+            for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v0 + i);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                ss += xf[i] * xf[i];
+                dot += gf[i] * wf[i] * xf[i];
+            }
+        }
+        ss = group_sum<64>(ss);
+        dot = group_sum<64>(dot);
+        const int par = (int)(it & 1);
+        if ((threadIdx.x & 63) == 0) part[par][wave] = make_float2(ss, dot);
+        __syncthreads();
+        ss = 0.f;
+        dot = 0.f;
+#pragma unroll
+        for (int j = 0; j < WPR; ++j) {
+            const float2 pj = part[par][WPR * rg + j];
+            ss += pj.x;
+            dot += pj.y;
+        }
+        const float rstd = rsqrtf(ss * inv_h + eps);
+        const float coef = dot * inv_h * rstd * rstd * rstd;
+        if (row_ok) {
+            uint4* dxr = reinterpret_cast<uint4*>(dx + row * hidden);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+                    float xf[V], gf[V], wf[V], o[V];
+                    Elem<T>::unpack(xraw[c], xf);
+                    Elem<T>::unpack(graw[c], gf);
+#pragma unroll
+                    for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v * V + i);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        o[i] = rstd * (gf[i] * wf[i]) - xf[i] * coef;
+                        acc[c][i] += gf[i] * (xf[i] * rstd);
+                    }
+                    dxr[v] = Elem<T>::pack(o);
+                }
+            }
+        }
+    }
+    for (int i = threadIdx.x; i < hidden; i += kWideBlock) dw_lds[i] = 0.f;
+    __syncthreads();
+    for (int g = 0; g < RPB; ++g) {
+        if (rg == g) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) dw_lds[v * V + i] += acc[c][i];
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out = dw_partial + (int64_t)blockIdx.x * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kWideBlock) out[i] = dw_lds[i];
+}
+
 // dw[col] = sum_p partial[p][col]; 16 columns x 16 row groups per block, fixed summation order.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw,
@@ -177,8 +294,18 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* 
     const int cl = threadIdx.x % 16, pg = threadIdx.x / 16;
     const int col = blockIdx.x * 16 + cl;
     float s = 0.f;
-    if (col < hidden)
-        for (int p = pg; p < n_partial; p += 16) s += partial[(int64_t)p * hidden + col];
+    if (col < hidden) {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        int p = pg;
+        for (; p + 48 < n_partial; p += 64) {   // four independent loads in flight per thread
+            s0 += partial[(int64_t)p * hidden + col];
+            s1 += partial[(int64_t)(p + 16) * hidden + col];
+            s2 += partial[(int64_t)(p + 32) * hidden + col];
+            s3 += partial[(int64_t)(p + 48) * hidden + col];
+        }
+        for (; p < n_partial; p += 16) s0 += partial[(int64_t)p * hidden + col];
+        s = (s0 + s1) + (s2 + s3);
+    }
     lds[pg][cl] = s;
     __syncthreads();
     if (pg == 0 && col < hidden) {
@@ -251,10 +378,29 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
     Plan plan;
     if (!make_plan<T>(hidden, &plan))
         return mi_fail(MI_E_SHAPE, "rmsnorm: hidden=%lld unsupported", (long long)hidden);
-    const int blocks = bwd_blocks(n_rows, plan.tpr);
+    const int64_t vecs = hidden / Elem<T>::kVec;
+    const bool wide = vecs >= 256;
+    // wide rows: 128 threads per row up to 512 vectors (8 rows per block), 256 threads per row beyond
+    const int wide_tpr = vecs <= 512 ? 128 : 256;
+    // one 1024-thread block per compute unit: a single round of blocks, each amortising its epilogue over more rows
+    const int blocks = wide ? (bwd_blocks(n_rows, wide_tpr / 4) > 256 ? 256 : bwd_blocks(n_rows, wide_tpr / 4)) : bwd_blocks(n_rows, plan.tpr);
     if (ws == nullptr || ws_bytes < (size_t)blocks * hidden * sizeof(float))
         return mi_fail(MI_E_WORKSPACE, "rmsnorm_bwd: workspace needs %zu bytes, got %zu",
                        (size_t)blocks * hidden * sizeof(float), ws_bytes);
+    if (wide) {
+        const int ch = (int)((vecs + wide_tpr - 1) / wide_tpr);
+        const size_t lds = 2 * hidden * sizeof(float);
+#define RMS_WIDE(TPRV, CHV) rmsnorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kWideBlock), lds, st>>>( \
+            (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps)
+        if (wide_tpr == 128) { if (ch <= 2) RMS_WIDE(128, 2); else RMS_WIDE(128, 4); }
+        else { if (ch <= 4) RMS_WIDE(256, 4); else RMS_WIDE(256, 8); }
+#undef RMS_WIDE
+        int rcw = mi_check_launch("rmsnorm_bwd_wide");
+        if (rcw != MI_OK) return rcw;
+        rmsnorm_dw_reduce_kernel<T><<<dim3((unsigned)((hidden + 15) / 16)), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw,
+                                                                                                   blocks, (int)hidden);
+        return mi_check_launch("rmsnorm_dw_reduce");
+    }
     const bool launched = dispatch_plan(plan, [&](auto tag) {
         constexpr int TPR = decltype(tag)::TPR;
         constexpr int CH = decltype(tag)::CH;
@@ -294,7 +440,7 @@ int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, 
     if (n_rows <= 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "rmsnorm_bwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
     if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(dy) || !mi_aligned16(dx) || !mi_aligned16(workspace))
         return mi_fail(MI_E_ALIGN, "rmsnorm_bwd: pointers must be 16-byte aligned");
-    if (hidden * sizeof(float) > 160 * 1024 - 64) return mi_fail(MI_E_SHAPE, "rmsnorm_bwd: hidden too large for LDS");
+    if (2 * hidden * sizeof(float) > 160 * 1024 - 256) return mi_fail(MI_E_SHAPE, "rmsnorm_bwd: hidden too large for LDS");
     MI_DISPATCH_DTYPE(dtype, return launch_bwd<T>(x, weight, dy, dx, dweight, workspace, workspace_bytes, n_rows, hidden,
                                                   eps, (hipStream_t)stream));
     return MI_OK;
