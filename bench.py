@@ -152,6 +152,46 @@ def bandwidth_cases(steps, warmup):
     return out
 
 
+def decode_case(steps, layers=32, batch=32, prompt=4096):
+    """Config 5: random-init 8B-class decoder, batch of prompts prefilled, then greedy cached decoding.
+    Reports decode tokens/s (batch * steps / decode wall time) and the prefill time."""
+    import torch
+    from scaling_amd.config import TransformerArchitectureConfig
+    from scaling_amd.inference import TransformerInferenceModule
+    cfg = TransformerArchitectureConfig.from_dict(dict(
+        vocab_size=128256, hidden_size=4096, num_layers=layers, num_attention_heads=32, attention_num_kv_heads=8,
+        attention_qkv_in_one=False, norm_type="rms", mlp_type="swiglu", mlp_factor=3.5, attention_bias=False, mlp_bias=False,
+        precision="bfloat16", sequence_length=prompt + steps + 16, rotary_embedding_base=500000, weight_tying=False,
+        masked_softmax={"kernel": "hip", "softmax_in_fp32": True}))
+    torch.manual_seed(0)
+    model = TransformerInferenceModule(cfg, device="cuda", init_std=0.02)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(1, cfg.vocab_size, (batch, prompt), generator=g)   # id 0 would split a prompt into documents
+    model.generate(2, ids)                       # warm-up: library heuristics, allocator, caches
+    torch.cuda.synchronize()
+    t0 = time.time()
+    model.generate(1, ids)                       # prefill + first token
+    torch.cuda.synchronize()
+    t_prefill = time.time() - t0
+    t0 = time.time()
+    model.generate(steps + 1, ids)               # prefill again + steps decode iterations, one launch per kernel
+    torch.cuda.synchronize()
+    t_eager = max(time.time() - t0 - t_prefill, 1e-9)
+    model.generate_graph(4, ids)                 # warm-up of the capture path
+    torch.cuda.synchronize()
+    t0 = time.time()
+    model.generate_graph(steps + 1, ids)         # prefill + steps decode iterations replayed from one HIP graph
+    torch.cuda.synchronize()
+    t_decode = max(time.time() - t0 - t_prefill, 1e-9)
+    out = {"layers": layers, "batch": batch, "prompt": prompt, "decode_steps": steps, "prefill_s": t_prefill,
+           "decode_s": t_decode, "decode_tok_per_s": batch * steps / t_decode, "ms_per_decode_step": 1e3 * t_decode / steps,
+           "eager_decode_tok_per_s": batch * steps / t_eager, "eager_ms_per_decode_step": 1e3 * t_eager / steps,
+           "note": "decode time = (prefill + decode wall time) - prefill wall time; graph capture time is included"}
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(seconds_budget=25.0):
     """The reference's operation order (CPU oracle) on a bounded sample of the headline workload:
     same head_dim / GQA ratio / causal mask / bf16 with fp32 softmax, fewer heads and a shorter sequence."""
@@ -195,6 +235,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--decode-steps", type=int, default=256, help="greedy decode steps of the config-5 workload")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -237,6 +278,7 @@ def main():
         extra["config3_gqa_packed_rotary_s8192"] = attention_case(1, 8192, 32, 8, 128, cu3, args.steps, args.warmup, seed=3, rotary=True)
         extra["config3_gqa_packed_rotary_s8192"]["n_docs"] = len(cu3) - 1
         extra.update(bandwidth_cases(args.steps, args.warmup))
+        extra["config5_decode_8b_b32_ctx4096"] = decode_case(args.decode_steps)
 
     line = {
         "metric": "attn fwd+bwd TFLOP/s (% bf16 MFMA peak); decode tok/s; norm GB/s (% HBM)",

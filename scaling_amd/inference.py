@@ -120,9 +120,11 @@ class TransformerInferenceModule(torch.nn.Module):
     @torch.no_grad()
     def forward(self, token_ids: torch.Tensor, position_ids: Optional[torch.Tensor] = None,
                 cumulative_seq_lengths: Optional[torch.Tensor] = None,
-                inference_settings: Optional[InferenceSettings] = None) -> torch.Tensor:
+                inference_settings: Optional[InferenceSettings] = None, last_token_only: bool = False) -> torch.Tensor:
         """token_ids [b, s] -> logits [b, s, vocab]; ids / lengths default to the reference's batch
-        construction (transformer/data/text_dataset_batch.py:110-126)."""
+        construction (transformer/data/text_dataset_batch.py:110-126).  last_token_only=True applies the
+        final norm and the LM head to the last position only (logits [b, 1, vocab]): greedy decoding reads
+        nothing else, and a [32, 4096, 128256] logits tensor would not be worth its 33 GB."""
         token_ids = token_ids.to(self.device)
         if cumulative_seq_lengths is None:
             cumulative_seq_lengths = get_cumulative_seq_lengths(token_ids, self.architecture_config.reset_attention_mask)
@@ -131,14 +133,74 @@ class TransformerInferenceModule(torch.nn.Module):
         x = TransformerLayerIO(activations=self._layers[0](token_ids), position_ids=position_ids.to(self.device),
                                cumulative_seq_lengths=cumulative_seq_lengths.to(self.device),
                                inference_settings=inference_settings)
-        for layer in self._layers[1:-1]:
+        for layer in self._layers[1:-2]:
             x = layer(x)
+        if last_token_only:
+            x.activations = x.activations[:, -1:, :].contiguous()
+        x = self._layers[-2](x)
         return self._layers[-1](x.activations)
 
     def logits(self, input_tokens: Sequence[int]) -> torch.Tensor:
         return self.forward(torch.tensor([list(input_tokens)])).squeeze(0)
 
     # ---- generation ---------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def generate_graph(self, max_tokens: int, input_tokens: Union[Sequence[int], torch.Tensor]) -> List[List[int]]:
+        """Greedy cached completion whose per-token step (all layers, LM head, arg-max, cache append) is
+        captured once as a HIP graph and replayed: the host issues one launch per token instead of a few
+        hundred.  No early stop; returns the completion ids per prompt.  Same arithmetic as `generate`."""
+        ids = torch.as_tensor(input_tokens)
+        if ids.dim() == 1:
+            ids = ids.unsqueeze(0)
+        ids = ids.to(self.device)
+        b, n_prompt = ids.shape
+        layers = list(self._layers[1:-2])
+        assert n_prompt + max_tokens <= layers[0].self_attention._cache_capacity(), "KV cache too small"
+        logits = self.forward(ids, inference_settings=InferenceSettings(use_cache=True, reset_cache=True), last_token_only=True)
+        tok = sample_argmax(logits).unsqueeze(1).contiguous()             # [b, 1] static buffer
+        pos = torch.full((b,), n_prompt, dtype=torch.int64, device=self.device)
+        out = torch.zeros(b, max_tokens, dtype=torch.int64, device=self.device)
+        out[:, 0] = tok[:, 0]
+        step = torch.ones(1, dtype=torch.int64, device=self.device)      # column of `out` the next token goes to
+        if max_tokens == 1:
+            return out.tolist()
+        for layer in layers:                                              # decode workspaces exist before capture
+            att = layer.self_attention
+            cache = att.cache[0]
+            if cache.workspace is None:
+                from . import ops
+                cache.workspace = ops.decode_workspace(b, att.num_attention_heads, att.hidden_size_per_attention_head,
+                                                       cache.max_ctx, self.device)
+
+        def one_step():
+            h = self._layers[0](tok)
+            for layer in layers:
+                h = layer.decode_step(h, pos)
+            lg = self._layers[-1](self._layers[-2].norm(h))
+            nxt = torch.argmax(lg, dim=-1)                                # [b, 1]
+            out.index_copy_(1, step, nxt)
+            tok.copy_(nxt)
+            pos.add_(1)
+            step.add_(1)
+
+        n_eager = min(2, max_tokens - 1)                                  # warm-up steps run eagerly
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(n_eager):
+                one_step()
+        torch.cuda.current_stream().wait_stream(side)
+        remaining = max_tokens - 1 - n_eager
+        if remaining > 0:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                one_step()
+            for _ in range(remaining):   # capture only records; every remaining token is one replay
+                graph.replay()
+        for layer in layers:
+            layer.self_attention.cache[0].length = n_prompt + max_tokens - 1
+        return out.tolist()
+
     @torch.no_grad()
     def generate(self, max_tokens: int, input_tokens: Union[Sequence[int], torch.Tensor], use_cache: bool = True,
                  stop_tokens: Optional[Sequence[int]] = None) -> Tuple[List[List[int]], torch.Tensor]:
@@ -157,7 +219,7 @@ class TransformerInferenceModule(torch.nn.Module):
             settings = InferenceSettings(use_cache=True, reset_cache=True)
             cur, pos = ids, None
             for k in range(max_tokens):
-                logits = self.forward(cur, position_ids=pos, inference_settings=settings)
+                logits = self.forward(cur, position_ids=pos, inference_settings=settings, last_token_only=True)
                 nxt = sample_argmax(logits)
                 step_logits.append(logits[:, -1, :])
                 for i, t in enumerate(nxt.tolist()):

@@ -104,6 +104,11 @@ class TransformerLayer(torch.nn.Module):
         residual = self.mlp(self.post_attention_layernorm(hidden_state))
         return self.dropout_mlp(residual) + hidden_state
 
+    def decode_step(self, hidden_state: torch.Tensor, position_ids: torch.Tensor, cache_index: int = 0) -> torch.Tensor:
+        """Cached single-token step on plain tensors, free of host synchronisation (HIP-graph capturable)."""
+        h = hidden_state + self.self_attention.decode_forward(self.input_layernorm(hidden_state), position_ids, cache_index)
+        return h + self.mlp(self.post_attention_layernorm(h))
+
     def forward(self, x: TransformerLayerIO) -> TransformerLayerIO:
         s = x.inference_settings
         use_cache, reset_cache, cache_index = (False, False, 0) if s is None else (s.use_cache, s.reset_cache, s.cache_index)

@@ -311,6 +311,29 @@ class ParallelSelfAttention(torch.nn.Module):
         cache.length = s
         cache.ctx_len.fill_(s)
 
+    def decode_forward(self, x: torch.Tensor, position_ids: torch.Tensor, cache_index: int = 0) -> torch.Tensor:
+        """One cached decode step without any host synchronisation (usable under HIP graph capture):
+        x [b, 1, H], position_ids int64 [b].  The caller guarantees a prefilled cache with room for one
+        more token per sequence; only the device-side context lengths are advanced here."""
+        b = x.shape[0]
+        nq, d = self.num_attention_heads, self.hidden_size_per_attention_head
+        q, k, v = self._project(x)
+        if self.key_query_norm:
+            q, k = self.norm_query(q), self.norm_key(k)
+        cache = self.cache[cache_index]
+        cache.ctx_len.add_(1)
+        rotary = None
+        if self.rotary_embedding is not None:
+            cos, sin = self.rotary_embedding.tables()
+            if self.rotary_embedding.dimensions == d and d in (64, 128):
+                rotary = (cos, sin, position_ids)
+            else:
+                q = self.rotary_embedding.rotate_tokens(q, position_ids, 1)
+                k = self.rotary_embedding.rotate_tokens(k, position_ids, 1)
+        ctx = ops.decode_attention(q.contiguous(), cache.k, cache.v, cache.ctx_len, k.contiguous(), v.contiguous(),
+                                   rotary=rotary, softmax_scale=self.softmax_scale, workspace=cache.workspace)
+        return self.dense(ctx.view(b, 1, nq * d))
+
     def _decode_step(self, q, k, v, pos, b: int, s: int, cache_index: int) -> torch.Tensor:
         cache = self.cache.get(cache_index)
         assert cache is not None, "decode step without a prefilled cache"

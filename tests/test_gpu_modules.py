@@ -148,3 +148,17 @@ def test_index_construction_on_device_is_bit_exact():
     ids = torch.tensor([[1, 2, 3, 0, 1, 2], [1, 2, 3, 4, 5, 6], [1, 2, 3, 4, 5, 0]], device=DEV)
     assert D.get_cumulative_seq_lengths(ids).tolist() == [0, 4, 6, 12, 18]
     assert D.get_position_ids(ids).tolist() == [[0, 1, 2, 3, 0, 1], [0, 1, 2, 3, 4, 5], [0, 1, 2, 3, 4, 5]]
+
+
+@pytest.mark.parametrize("max_tokens", [1, 2, 3, 9])
+def test_graph_captured_decode_equals_eager_decode(max_tokens):
+    """Every replay of the captured per-token step must reproduce the eager step (tokens identical)."""
+    cfg = _arch(attention_num_kv_heads=2, hidden_size=512, num_attention_heads=4, sequence_length=64)
+    model = TransformerInferenceModule(cfg, device=DEV, init_std=0.1, seed=6)
+    g = torch.Generator().manual_seed(7)
+    prompts = torch.randint(1, cfg.vocab_size, (4, 11), generator=g)
+    eager, _ = model.generate(max_tokens, prompts)
+    graphed = model.generate_graph(max_tokens, prompts)
+    assert graphed == eager
+    # a second capture on the same module (fresh prefill) gives the same tokens again
+    assert model.generate_graph(max_tokens, prompts) == eager
