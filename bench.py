@@ -139,8 +139,9 @@ def bandwidth_cases(steps, warmup):
     out["rotary"] = {"ms": ms, "GBs": (2 * N * (nq + nkv) * d * 2 + 8 * N) / ms / 1e6}
     del qk
     B, ctx, max_ctx = 32, 4096, 4352
-    kc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16().to(dev)
-    vc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16().to(dev)
+    # head-major storage viewed as [batch, token, kv head, d]: the layout scaling_amd.nn.KVCache allocates
+    kc = torch.randn(B, nkv, max_ctx, d, generator=g).bfloat16().to(dev).transpose(1, 2)
+    vc = torch.randn(B, nkv, max_ctx, d, generator=g).bfloat16().to(dev).transpose(1, 2)
     q1 = torch.randn(B, nq, d, generator=g).bfloat16().to(dev)
     ctx_len = torch.full((B,), ctx, dtype=torch.int32, device=dev)
     wsd = ops.decode_workspace(B, nq, d, max_ctx, dev)

@@ -65,7 +65,7 @@ __global__ void decode_append_kernel(const DecodeParams p) {
 
 // ---- split kernel ----------------------------------------------------------------------------------
 template <int D, bool ROT>
-__global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeParams p) {
     constexpr int KS = D / 32;          // contraction steps of Q K^T (32 features each)
     constexpr int DT = D / 16;          // 16-row tiles of O^T
     constexpr int VROW = kChunk + 8;    // padded row of the transposed V chunk (elements)
@@ -127,33 +127,41 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodePara
     const __bf16* vbase = p.vc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
     char* vt = reinterpret_cast<char*>(vt_lds[wave]);
 
-    for (int it = 0; it < n_iter; ++it) {
-        const int key0 = s0 + (4 * it + wave) * kChunk;
-        const bool active = key0 < s1;          // wave-uniform
+    // K fragments and V rows of a chunk; two sets so that the loads of chunk i+1 are in flight while
+    // chunk i is being processed
+    struct ChunkRegs {
         bf16x8_t kf[2][KS];
         uint4 vraw[V_PER_LANE][4];
-        if (active) {
+    };
+    auto load_chunk = [&](ChunkRegs& c, int it) {
+        const int key0 = s0 + (4 * it + wave) * kChunk;
+        if (key0 >= s1) return;
+        const int last = s1 - 1;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                int tok = key0 + 16 * t + l16;
-                tok = tok < s1 ? tok : s1 - 1;
-                const __bf16* kr = kbase + (int64_t)tok * p.c_st + 8 * G;
+        for (int t = 0; t < 2; ++t) {
+            const int tok = min(key0 + 16 * t + l16, last);
+            const __bf16* kr = kbase + (int64_t)tok * p.c_st + 8 * G;
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) kf[t][ks] = *reinterpret_cast<const bf16x8_t*>(kr + 32 * ks);
-            }
+            for (int ks = 0; ks < KS; ++ks) c.kf[t][ks] = *reinterpret_cast<const bf16x8_t*>(kr + 32 * ks);
+        }
 #pragma unroll
-            for (int j = 0; j < V_PER_LANE; ++j) {
-                const int item = lane + 64 * j;
-                const int quad = item / (D / 8), dg = item % (D / 8);
+        for (int j = 0; j < V_PER_LANE; ++j) {
+            const int item = lane + 64 * j;
+            const int quad = item / (D / 8), dg = item % (D / 8);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    int tok = key0 + 4 * quad + r;
-                    tok = tok < s1 ? tok : s1 - 1;
-                    vraw[j][r] = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.c_st + 8 * dg);
-                }
+            for (int r = 0; r < 4; ++r) {
+                const int tok = min(key0 + 4 * quad + r, last);
+                c.vraw[j][r] = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.c_st + 8 * dg);
             }
         }
-        __syncthreads();  // every wavefront is done reading its LDS chunk of the previous iteration
+    };
+    auto process_chunk = [&](const ChunkRegs& c, int it) {
+        const int key0 = s0 + (4 * it + wave) * kChunk;
+        const bool active = key0 < s1;          // wave-uniform
+        // Each wavefront owns its LDS chunk; the LDS pipeline executes one wavefront's accesses in program
+        // order, so wavefront-scope fences (compiler ordering only) are enough and the wavefronts of a
+        // workgroup never wait for each other inside the loop.
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         bf16x8_t pf;
         float alpha = 1.f;
         if (active) {
@@ -162,7 +170,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodePara
             for (int t = 0; t < 2; ++t) {
                 s_acc[t] = f32x4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) s_acc[t] = mfma_16x16x32(kf[t][ks], qf[ks], s_acc[t]);
+                for (int ks = 0; ks < KS; ++ks) s_acc[t] = mfma_16x16x32(c.kf[t][ks], qf[ks], s_acc[t]);
             }
             // rows: keys key0 + 16*t + 4*G + r; column: head slot l16
             float mx = -INFINITY;
@@ -194,25 +202,12 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodePara
                 const int item = lane + 64 * j;
                 const int quad = item / (D / 8), dg = item % (D / 8);
                 const int col = 8 * (quad & 3) + 4 * (quad >> 2);
-                const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&vraw[j][0]);
-                const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&vraw[j][1]);
-                const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&vraw[j][2]);
-                const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&vraw[j][3]);
 #pragma unroll
-                for (int dd = 0; dd < 8; ++dd) {
-                    uint32_t lo, hi;
-                    if (dd & 1) {
-                        lo = (w0[dd >> 1] >> 16) | (w1[dd >> 1] & 0xffff0000u);
-                        hi = (w2[dd >> 1] >> 16) | (w3[dd >> 1] & 0xffff0000u);
-                    } else {
-                        lo = (w0[dd >> 1] & 0xffffu) | (w1[dd >> 1] << 16);
-                        hi = (w2[dd >> 1] & 0xffffu) | (w3[dd >> 1] << 16);
-                    }
-                    *reinterpret_cast<uint2*>(vt + ((8 * dg + dd) * VROW + col) * 2) = make_uint2(lo, hi);
-                }
+                for (int dd = 0; dd < 8; ++dd)
+                    *reinterpret_cast<uint2*>(vt + ((8 * dg + dd) * VROW + col) * 2) = transpose_quad(c.vraw[j], dd);
             }
         }
-        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         if (active) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
@@ -220,6 +215,17 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodePara
                 o_acc[dt] = o_acc[dt] * alpha;
                 o_acc[dt] = mfma_16x16x32(a, pf, o_acc[dt]);
             }
+        }
+    };
+
+    ChunkRegs ra, rb;
+    if (n_iter > 0) load_chunk(ra, 0);
+    for (int it = 0; it < n_iter; it += 2) {
+        if (it + 1 < n_iter) load_chunk(rb, it + 1);
+        process_chunk(ra, it);
+        if (it + 1 < n_iter) {
+            if (it + 2 < n_iter) load_chunk(ra, it + 2);
+            process_chunk(rb, it + 1);
         }
     }
 
@@ -276,7 +282,7 @@ __global__ void decode_merge_kernel(const DecodeParams p) {
 
 int choose_splits(int batch, int nkv, int max_ctx) {
     const int64_t pairs = (int64_t)batch * nkv;
-    int64_t s = (1024 + pairs - 1) / pairs;
+    int64_t s = (512 + pairs - 1) / pairs;   // two 256-thread workgroups per compute unit = one round of blocks
     const int64_t by_len = ((int64_t)max_ctx + 4 * kChunk - 1) / (4 * kChunk);
     if (s > by_len) s = by_len;
     if (s > kMaxSplits) s = kMaxSplits;
