@@ -95,6 +95,14 @@ int mi_rotary(const void* x, void* out, const void* cos, const void* sin, const 
               int64_t table_rows, int64_t seq_len_for_null_ids, int inverse,
               int dtype, int table_dtype, void* stream);
 
+/* Interleaved ("complex") rotary, pairs (2i, 2i+1) over the whole head, fp32 arithmetic.
+ * Replaces core/nn/rotary.py:45-90 / :216-255 (RotaryEmbeddingComplex): cos / sin are the real / imaginary
+ * parts of freqs_cis, fp32 [table_rows, head_dim/2].  Other arguments as mi_rotary. */
+int mi_rotary_complex(const void* x, void* out, const float* cos, const float* sin, const int64_t* position_ids,
+                      int64_t n_tokens, int32_t n_heads, int32_t head_dim,
+                      int64_t x_stride_token, int64_t x_stride_head, int64_t out_stride_token, int64_t out_stride_head,
+                      int64_t table_rows, int64_t seq_len_for_null_ids, int inverse, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Attention core.  Replaces core/nn/attention/attention.py:108-213 (multi_head_attention) with
  * core/nn/masked_softmax/masked_softmax.py:14-34 as softmax and :76-105 as mask, plus repeat_kv

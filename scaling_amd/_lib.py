@@ -19,7 +19,7 @@ _DTYPE_CODE = {torch.bfloat16: MI_BF16, torch.float16: MI_F16, torch.float32: MI
 EXPORTS = (
     "mi_version", "mi_last_error", "mi_status_string", "mi_check_device",
     "mi_rmsnorm_fwd", "mi_rmsnorm_bwd_workspace_bytes", "mi_rmsnorm_bwd",
-    "mi_swiglu_fwd", "mi_swiglu_bwd", "mi_rotary",
+    "mi_swiglu_fwd", "mi_swiglu_bwd", "mi_rotary", "mi_rotary_complex",
     "mi_attn_fwd", "mi_attn_bwd_workspace_bytes", "mi_attn_bwd",
     "mi_attn_decode_workspace_bytes", "mi_attn_decode",
 )
@@ -93,6 +93,9 @@ def _declare(lib):
     lib.mi_rotary.restype = c_int
     lib.mi_rotary.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_int32,
                               c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p]
+    lib.mi_rotary_complex.restype = c_int
+    lib.mi_rotary_complex.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32,
+                                      c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]
     lib.mi_attn_fwd.restype = c_int
     lib.mi_attn_fwd.argtypes = [POINTER(MiAttnArgs)]
     lib.mi_attn_bwd_workspace_bytes.restype = c_size_t

@@ -105,6 +105,34 @@ __global__ __launch_bounds__(kBlock) void rotary_scalar_kernel(RotaryParams p) {
     Elem<T>::store1(orow + i + half, o1);
 }
 
+// Interleaved ("complex") pairing (2i, 2i+1) over the whole head, fp32 tables [rows, head_dim/2].
+// One thread owns one 128-bit vector = V/2 complete pairs.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rotary_complex_kernel(RotaryParams p) {
+    constexpr int V = Elem<T>::kVec;
+    const int vec_per_head = p.head_dim / V;
+    const int64_t per_token = (int64_t)vec_per_head * p.n_heads;
+    const int64_t item = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (item >= per_token * p.n_tokens) return;
+    const int64_t t = item / per_token;
+    const int rem = (int)(item % per_token);
+    const int h = rem / vec_per_head, v = rem % vec_per_head;
+    const T* xrow = (const T*)p.x + t * p.xs_t + (int64_t)h * p.xs_h + v * V;
+    T* orow = (T*)p.out + t * p.os_t + (int64_t)h * p.os_h + v * V;
+    const int64_t r = table_row(p, t);
+    const float* cr = (const float*)p.cos + r * (p.head_dim / 2) + v * (V / 2);
+    const float* sr = (const float*)p.sin + r * (p.head_dim / 2) + v * (V / 2);
+    float x[V], o[V];
+    Elem<T>::unpack(*reinterpret_cast<const uint4*>(xrow), x);
+#pragma unroll
+    for (int i = 0; i < V / 2; ++i) {
+        const float c = cr[i], sn = p.sign * sr[i];
+        o[2 * i] = x[2 * i] * c - x[2 * i + 1] * sn;
+        o[2 * i + 1] = x[2 * i] * sn + x[2 * i + 1] * c;
+    }
+    *reinterpret_cast<uint4*>(orow) = Elem<T>::pack(o);
+}
+
 template <typename T, typename TT> int launch(const RotaryParams& p, hipStream_t st) {
     constexpr int V = Elem<T>::kVec;
     const bool vec_ok = (p.rot_dim / 2) % V == 0 && (p.head_dim - p.rot_dim) % V == 0 && p.xs_t % V == 0 &&
@@ -141,4 +169,28 @@ extern "C" int mi_rotary(const void* x, void* out, const void* cos, const void* 
         return launch<T, float>(p, (hipStream_t)stream);
     });
     return MI_OK;
+}
+
+extern "C" int mi_rotary_complex(const void* x, void* out, const float* cos, const float* sin, const int64_t* position_ids,
+                                 int64_t n_tokens, int32_t n_heads, int32_t head_dim, int64_t x_stride_token,
+                                 int64_t x_stride_head, int64_t out_stride_token, int64_t out_stride_head,
+                                 int64_t table_rows, int64_t seq_len_for_null_ids, int inverse, int dtype, void* stream) {
+    if (!x || !out || !cos || !sin) return mi_fail(MI_E_NULL, "rotary_complex: null pointer");
+    if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0 || table_rows <= 0)
+        return mi_fail(MI_E_SHAPE, "rotary_complex: bad shape tokens=%lld heads=%d head_dim=%d", (long long)n_tokens, n_heads, head_dim);
+    if (!position_ids && seq_len_for_null_ids <= 0) return mi_fail(MI_E_SHAPE, "rotary_complex: need position ids or a sequence length");
+    if (n_tokens == 0) return MI_OK;
+    RotaryParams p{x, out, cos, sin, position_ids, n_tokens, n_heads, head_dim, head_dim, x_stride_token, x_stride_head,
+                   out_stride_token, out_stride_head, table_rows, seq_len_for_null_ids, inverse ? -1.0f : 1.0f};
+    MI_DISPATCH_DTYPE(dtype, {
+        constexpr int V = Elem<T>::kVec;
+        if (head_dim % V || x_stride_token % V || x_stride_head % V || out_stride_token % V || out_stride_head % V ||
+            !mi_aligned16(x) || !mi_aligned16(out))
+            return mi_fail(MI_E_ALIGN, "rotary_complex: head_dim and strides must be multiples of %d elements, pointers 16-byte aligned", V);
+        const int64_t items = (int64_t)(head_dim / V) * n_heads * n_tokens;
+        const int64_t blocks = (items + kBlock - 1) / kBlock;
+        if (blocks > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "rotary_complex: too many elements");
+        rotary_complex_kernel<T><<<dim3((unsigned)blocks), dim3(kBlock), 0, (hipStream_t)stream>>>(p);
+    });
+    return mi_check_launch("rotary_complex");
 }

@@ -105,6 +105,39 @@ class RotaryEmbedding(torch.nn.Module):
         return one(query, query_position_ids), one(key, key_position_ids)
 
 
+class RotaryEmbeddingComplex(torch.nn.Module):
+    """Mirror of core/nn/rotary.py:216-255: interleaved pairs (2i, 2i+1), fp32 arithmetic; the real and
+    imaginary parts of freqs_cis (rotary.py:45-56) are non-persistent buffers [max_seq, dim/2]."""
+
+    def __init__(self, config: RotaryConfig, device: torch.device) -> None:
+        super().__init__()
+        assert config.dimensions > 1, "RotaryEmbedding cannot use `dim` == 1"
+        dim, n = config.dimensions, config.max_seq_length
+        freqs = 1.0 / (float(config.base) ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
+        ang = torch.outer(torch.arange(n), freqs).float().to(device)
+        self.register_buffer("freqs_cis_real", ang.cos(), persistent=False)
+        self.register_buffer("freqs_cis_imag", ang.sin(), persistent=False)
+        self.dimensions = dim
+        self.max_seq_length = n
+
+    def tables(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        return self.freqs_cis_real, self.freqs_cis_imag
+
+    def rotate_tokens(self, x: torch.Tensor, position_ids: Optional[torch.Tensor], seq_len: int) -> torch.Tensor:
+        assert x.shape[-1] == self.dimensions, "the interleaved variant rotates the whole head (rotary.py:69-70)"
+        return ops.rotary_embedding_complex(x, self.freqs_cis_real.float().contiguous(),
+                                            self.freqs_cis_imag.float().contiguous(), position_ids, seq_len)
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, query_position_ids: Optional[torch.Tensor] = None,
+                key_position_ids: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+        def one(x, ids):
+            s, b, n, d = x.shape
+            tok = x.permute(1, 0, 2, 3).reshape(b * s, n, d)
+            flat = None if ids is None else ids.transpose(0, 1).reshape(-1).contiguous()
+            return self.rotate_tokens(tok, flat, s).view(b, s, n, d).permute(1, 0, 2, 3)
+        return one(query, query_position_ids), one(key, key_position_ids)
+
+
 class ParallelSwiGLUMLP(torch.nn.Module):
     """Mirror of core/nn/mlp.py:149-282: dense_out(silu(dense_in(x)) * siglu_weight(x))."""
 
@@ -150,7 +183,7 @@ class ParallelSelfAttention(torch.nn.Module):
 
     Same constructor arguments and forward signature.  Differences, all documented errors rather than
     silent fall-backs: attention-probability dropout, attention-score manipulation, LoRA, local
-    attention windows, u-muP, fp8, `rotary_complex` and LayerNorm query/key norm are not available;
+    attention windows, u-muP, fp8 and LayerNorm query/key norm are not available;
     the dtype must be bfloat16.  The KV cache is pre-allocated (see `KVCache`), supports batches of
     single-document rows and is filled/extended in place.
     """
@@ -181,8 +214,6 @@ class ParallelSelfAttention(torch.nn.Module):
         if num_local_attention_heads > 0 or lora_config is not None or fp8_config is not None or \
                 fp8_config_dense_out is not None or bitfit_bias_name is not None:
             raise NotImplementedError("local attention, LoRA, fp8 and bitfit are outside the hip kernel's scope")
-        if relative_position_embedding_type == RelativePositionEmbeddingType.ROTARY_COMPLEX:
-            raise NotImplementedError("rotary_complex has no HIP kernel yet (supported: none, rotary)")
         if dtype != torch.bfloat16:
             raise NotImplementedError("the hip attention kernels compute in bfloat16; set precision: bfloat16")
 
@@ -215,10 +246,17 @@ class ParallelSelfAttention(torch.nn.Module):
             self.key = _Linear(hidden_size, hidden_size // self.num_repeat_kv, bias, self._device, dtype, init_method)
             self.value = _Linear(hidden_size, hidden_size // self.num_repeat_kv, bias, self._device, dtype, init_method)
 
-        self.rotary_embedding: Optional[RotaryEmbedding] = None
+        self.rotary_embedding = None
         if relative_position_embedding_type == RelativePositionEmbeddingType.ROTARY:
             assert rotary_config is not None
             self.rotary_embedding = RotaryEmbedding(config=rotary_config, device=self._device, dtype=dtype)
+        elif relative_position_embedding_type == RelativePositionEmbeddingType.ROTARY_COMPLEX:
+            assert rotary_config is not None
+            self.rotary_embedding = RotaryEmbeddingComplex(config=rotary_config, device=self._device)
+        # rotary can be applied inside the attention kernels (on the Q/K load) for the rotate-half variant
+        # when it covers the whole head
+        self._fusable_rotary = isinstance(self.rotary_embedding, RotaryEmbedding) and \
+            rotary_config.dimensions == self.hidden_size_per_attention_head and self.hidden_size_per_attention_head in (64, 128)
 
         self.key_query_norm = key_query_norm
         self.norm_query = self.norm_key = None
@@ -277,8 +315,7 @@ class ParallelSelfAttention(torch.nn.Module):
         elif reset_cache:
             self.cache[cache_index] = None
 
-        if (self.rotary_embedding is not None and not use_cache and not torch.is_grad_enabled() and pos is not None
-                and self.rotary_embedding.dimensions == d and d in (64, 128)):
+        if self._fusable_rotary and not use_cache and not torch.is_grad_enabled() and pos is not None:
             # inference without cache: rotary is applied while the kernel loads Q and K
             cos, sin = self.rotary_embedding.tables()
             cu_k = None if cumulative_seq_lengths_key is None else cumulative_seq_lengths_key.to(torch.int32)
@@ -326,8 +363,8 @@ class ParallelSelfAttention(torch.nn.Module):
         cache.ctx_len.add_(1)
         rotary = None
         if self.rotary_embedding is not None:
-            cos, sin = self.rotary_embedding.tables()
-            if self.rotary_embedding.dimensions == d and d in (64, 128):
+            if self._fusable_rotary:
+                cos, sin = self.rotary_embedding.tables()
                 rotary = (cos, sin, position_ids)
             else:
                 q = self.rotary_embedding.rotate_tokens(q, position_ids, 1)
@@ -349,10 +386,10 @@ class ParallelSelfAttention(torch.nn.Module):
         if self.rotary_embedding is not None:
             if pos is None:
                 pos = torch.full((b,), cache.length - 1, dtype=torch.int64, device=q.device)
-            cos, sin = self.rotary_embedding.tables()
-            if self.rotary_embedding.dimensions == d and d in (64, 128):
+            if self._fusable_rotary:
+                cos, sin = self.rotary_embedding.tables()
                 rotary = (cos, sin, pos)
-            else:  # partial rotary: stand-alone kernel, then a plain append
+            else:  # partial or interleaved rotary: stand-alone kernel, then a plain append
                 q = self.rotary_embedding.rotate_tokens(q, pos, 1)
                 k = self.rotary_embedding.rotate_tokens(k, pos, 1)
         if cache.workspace is None:

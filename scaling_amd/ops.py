@@ -16,7 +16,7 @@ from . import _lib
 from ._lib import MiAttnArgs, MiAttnBwdArgs, MiDecodeArgs, check, dtype_code, ptr, stream_ptr
 
 __all__ = [
-    "rms_norm", "swiglu", "rotary_embedding", "attention", "attention_forward", "attention_backward",
+    "rms_norm", "swiglu", "rotary_embedding", "rotary_embedding_complex", "attention", "attention_forward", "attention_backward",
     "decode_attention", "rms_norm_forward", "rms_norm_backward", "swiglu_forward", "swiglu_backward",
 ]
 
@@ -156,6 +156,44 @@ def rotary_embedding(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                      position_ids: Optional[torch.Tensor] = None, seq_len_for_null_ids: int = 0) -> torch.Tensor:
     """Rotate-half rotary on x [tokens, heads, head_dim]; position_ids int64 [tokens] (flattened (b s))."""
     return _Rotary.apply(x, cos, sin, position_ids, seq_len_for_null_ids)
+
+
+def _rotary_complex_launch(x, cos, sin, position_ids, seq_len_for_null_ids, inverse):
+    _need_cuda(x, cos, sin, position_ids)
+    assert x.dim() == 3 and x.stride(2) == 1
+    assert cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+    assert cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] * 2 == x.shape[2]
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if position_ids is not None:
+        position_ids = position_ids.contiguous()
+        assert position_ids.dtype == torch.int64 and position_ids.numel() == x.shape[0]
+    check(_lib.load().mi_rotary_complex(ptr(x), ptr(out), ptr(cos), ptr(sin), ptr(position_ids), x.shape[0], x.shape[1],
+                                        x.shape[2], x.stride(0), x.stride(1), out.stride(0), out.stride(1), cos.shape[0],
+                                        int(seq_len_for_null_ids), int(bool(inverse)), dtype_code(x.dtype), stream_ptr()),
+          "mi_rotary_complex")
+    return out
+
+
+class _RotaryComplex(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, cos, sin, position_ids, seq_len_for_null_ids):
+        ctx.save_for_backward(cos, sin, position_ids if position_ids is not None else torch.empty(0, device=x.device))
+        ctx.has_ids = position_ids is not None
+        ctx.seq_len = seq_len_for_null_ids
+        return _rotary_complex_launch(x, cos, sin, position_ids, seq_len_for_null_ids, False)
+
+    @staticmethod
+    def backward(ctx, dout):
+        cos, sin, ids = ctx.saved_tensors
+        if dout.stride(-1) != 1:
+            dout = dout.contiguous()
+        return _rotary_complex_launch(dout, cos, sin, ids if ctx.has_ids else None, ctx.seq_len, True), None, None, None, None
+
+
+def rotary_embedding_complex(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                             position_ids: Optional[torch.Tensor] = None, seq_len_for_null_ids: int = 0) -> torch.Tensor:
+    """Interleaved-pair rotary on x [tokens, heads, head_dim]; cos / sin fp32 [rows, head_dim/2]."""
+    return _RotaryComplex.apply(x, cos, sin, position_ids, seq_len_for_null_ids)
 
 
 # ------------------------------------------------------------------------------------------------

@@ -130,3 +130,37 @@ def test_rotary_reference_invariants_and_backward():
     out.backward(go.permute(1, 0, 2, 3).reshape(batch * seq, heads, dim).contiguous().to(DEV))
     torch.cuda.synchronize()
     check("rotary.dx", xg.grad.view(batch, seq, heads, dim).permute(1, 0, 2, 3), xr.grad)
+
+
+@pytest.mark.parametrize("seq,batch,heads,dim", [(10, 2, 2, 8), (17, 7, 4, 16), (64, 2, 8, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rotary_complex_parity(seq, batch, heads, dim, dtype):
+    print(f"case rotary_complex s={seq} b={batch} n={heads} d={dim} {dtype}", flush=True)
+    from scaling_amd.config import RotaryConfig
+    from scaling_amd.nn import RotaryEmbeddingComplex
+    g = torch.Generator().manual_seed(seq * dim)
+    q = _rand(g, seq, batch, heads, dim, dtype=dtype)
+    k = _rand(g, seq, batch, heads, dim, dtype=dtype)
+    ids = torch.randint(0, seq, (seq, batch), generator=g)
+    ref_q, ref_k = oracle.apply_rotary_complex(q.float(), k.float(), dim, seq, 10000.0, ids, ids)
+    refo_q, _ = oracle.apply_rotary_complex(q, k, dim, seq, 10000.0, ids, ids)     # reference: fp32 math, cast back
+    mod = RotaryEmbeddingComplex(RotaryConfig(dimensions=dim, max_seq_length=seq, base=10000), torch.device(DEV))
+    got_q, got_k = mod(q.to(DEV), k.to(DEV), ids.to(DEV), ids.to(DEV))
+    torch.cuda.synchronize()
+    tol = dict(max_abs_tol=1e-5, mean_rel_tol=1e-6) if dtype == torch.float32 else {}
+    check("rotary_complex.q", got_q, ref_q, refo_q, **tol)
+    check("rotary_complex.k", got_k, ref_k, **tol)
+    # no ids == arange ids (the reference's invariant), and the backward is the inverse rotation
+    a, _ = mod(q.to(DEV), k.to(DEV))
+    ar = torch.arange(seq).unsqueeze(1).expand(seq, batch).contiguous().to(DEV)
+    b_, _ = mod(q.to(DEV), k.to(DEV), ar, ar)
+    assert torch.equal(a, b_)
+    xr = q.float().clone().requires_grad_()
+    out_r, _ = oracle.apply_rotary_complex(xr, xr.detach(), dim, seq, 10000.0, ids, ids)
+    go = _rand(g, seq, batch, heads, dim, dtype=dtype)
+    out_r.backward(go.float())
+    xg = q.to(DEV).detach().requires_grad_()
+    out_g, _ = mod(xg, k.to(DEV), ids.to(DEV), ids.to(DEV))
+    out_g.backward(go.to(DEV))
+    torch.cuda.synchronize()
+    check("rotary_complex.dx", xg.grad, xr.grad, **tol)

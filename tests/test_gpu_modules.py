@@ -49,6 +49,8 @@ def _seeded_layer(cfg, seed):
 def _oracle_layer(cfg, weights, x, cu, pos, dy, dtype):
     """Runs the oracle layer in `dtype` on the (bf16-rounded) weights and inputs; returns y, dx, dweights."""
     spec = _spec(cfg, dtype)
+    spec.rotary = cfg.relative_position_embedding_type.value
+    spec.rotary_percentage = cfg.rotary_percentage
     w = {k: v.detach().cpu().to(dtype).clone().requires_grad_() for k, v in weights.items()}
     xx = x.to(dtype).clone().requires_grad_()
     # the module keeps its rotary tables in bf16 (reference behaviour); the oracle uses the same values
@@ -63,6 +65,8 @@ def _oracle_layer(cfg, weights, x, cu, pos, dy, dtype):
     ("config1_mha", dict(), 2, 128, ()),                                                    # config 1 shape, bf16 on the GPU
     ("gqa_packed", dict(hidden_size=512, num_attention_heads=8, attention_num_kv_heads=2, mlp_factor=2.5), 2, 96, (40, 130)),
     ("fused_qkv_bias", dict(attention_qkv_in_one=True, attention_bias=True, mlp_bias=True), 1, 64, ()),
+    ("rotary_complex", dict(relative_position_embedding_type="rotary_complex"), 2, 64, (20,)),
+    ("partial_rotary", dict(rotary_percentage=0.5), 1, 96, ()),
 ])
 def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
     print(f"case layer {name}", flush=True)

@@ -133,9 +133,10 @@ def test_unsupported_options_raise():
         ParallelSelfAttention(256, 4, hip, dropout_attention_probs=0.1, dtype=torch.bfloat16, device=CPU)
     with pytest.raises(NotImplementedError, match="bfloat16"):
         ParallelSelfAttention(256, 4, hip, dtype=torch.float32, device=CPU)
-    with pytest.raises(NotImplementedError, match="rotary_complex"):
-        ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU,
-                              relative_position_embedding_type=C.RelativePositionEmbeddingType.ROTARY_COMPLEX)
+    cplx = ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, rotary_config=C.RotaryConfig(dimensions=64, max_seq_length=16),
+                                 relative_position_embedding_type=C.RelativePositionEmbeddingType.ROTARY_COMPLEX)
+    assert cplx.rotary_embedding.freqs_cis_real.shape == (16, 32) and not cplx._fusable_rotary
+    assert all("freqs_cis" not in k for k in cplx.state_dict())
     with pytest.raises(AssertionError, match="kv heads"):
         ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, num_kv_heads=2, qkv_in_one=True,
                               rotary_config=C.RotaryConfig(dimensions=64))
