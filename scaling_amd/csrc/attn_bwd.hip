@@ -160,18 +160,20 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     // document needs the document's last queries, so the workgroups that share an XCD start on the same
     // tile and keep streaming the same Q / dO rows through that XCD's L2.
     const int total_iters = n_tiles * p.n_rep;
+    // Role-dependent sources are selected once, as values: a per-iteration select between kernel
+    // arguments turns into a load of the argument through a vector address, and a wait on it.
+    const __bf16* src_base = q_role ? p.q : p.d_o;
+    int64_t src_head_stride = q_role ? p.q_sh : p.o_sh;
+    int64_t src_tok_stride = q_role ? p.q_st : p.o_st;
+    const float* stat_base = (tid < BQ) ? p.lse : p.delta;
+    const float stat_scale = (tid < BQ) ? 1.4426950408889634f : 1.0f;  // log-sum-exp goes to the exp2 domain
     auto load_tile = [&](int iter) {
         const int rep = iter / n_tiles, qt = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ;
         const int head = kvh * p.n_rep + rep;
-        if (ltid < ITEMS) {
-            if (q_role) load_quad<D>(raw, p.q + (int64_t)head * p.q_sh, p.q_st, qt, p.total_q, quad, dg);
-            else load_quad<D>(raw, p.d_o + (int64_t)head * p.o_sh, p.o_st, qt, p.total_q, quad, dg);
-        }
+        if (ltid < ITEMS) load_quad<D>(raw, src_base + (int64_t)head * src_head_stride, src_tok_stride, qt, p.total_q, quad, dg);
         if (tid < 2 * BQ) {
             const int tok = min(qt + (tid & (BQ - 1)), p.total_q - 1);
-            const float* src = (tid < BQ) ? p.lse : p.delta;
-            stat = src[(int64_t)head * p.total_q + tok];
-            if (tid < BQ) stat *= 1.4426950408889634f;  // log-sum-exp in the exp2 domain
+            stat = stat_base[(int64_t)head * p.total_q + tok];
         }
     };
     auto store_tile = [&]() {
@@ -179,8 +181,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             store_rows<STR>(raw, q_role ? q_rm : do_rm, quad, dg);
             store_transposed(raw, q_role ? q_tr : do_tr, quad, dg);
         }
-        if (tid < BQ) lse_lds[tid] = stat;
-        else if (tid < 2 * BQ) delta_lds[tid - BQ] = stat;
+        if (tid < BQ) lse_lds[tid] = stat * stat_scale;
+        else if (tid < 2 * BQ) delta_lds[tid - BQ] = stat * stat_scale;
     };
 
     if (total_iters > 0) {
@@ -342,8 +344,14 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
             dof[ks] = *reinterpret_cast<const bf16x8_t*>(dr + 16 * ks);
         }
     }
-    const float lse2 = p.lse[(int64_t)head * p.total_q + tl] * 1.4426950408889634f;
-    const float delta = p.delta[(int64_t)head * p.total_q + tl];
+    const float lse_nat = p.lse[(int64_t)head * p.total_q + tl];
+    float delta = p.delta[(int64_t)head * p.total_q + tl];
+    float lse2 = lse_nat * 1.4426950408889634f;
+    // Consume the loaded registers here: otherwise their loads count as possibly outstanding at the
+    // loop entry and their uses inside the loop wait for the K / V prefetch issued just before.
+    asm volatile("" : "+v"(lse2), "+v"(delta));
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
 
     __syncthreads();
     int bmin = 0x7fffffff, bmax = 0;

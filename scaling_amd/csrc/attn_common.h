@@ -108,6 +108,53 @@ __device__ __forceinline__ uint2 transpose_quad(const uint4 (&raw)[4], int dd) {
                       __builtin_amdgcn_perm(w3[dd >> 1], w2[dd >> 1], sel));
 }
 
+// ---- LDS transpose read (gfx950 ds_read_b64_tr_b16) ---------------------------------------------------
+// Within each block of 16 lanes the instruction loads 16 x 8 bytes and hands lane j the j-th 16-bit element
+// of each of the four 32-byte rows formed by lanes {0..3}, {4..7}, {8..11}, {12..15}.  With a token-major
+// [token][feature] tile in LDS, pointing lane i of a block at token (t0 + i/4), features (f0 + 4*(i%4) ..)
+// returns to lane j the values of tokens t0..t0+3 at feature f0 + j: the transposed A operand of an MFMA
+// whose contraction index is the token, without a transposed copy of the tile.
+// Row stride: 4 rows x 2 feature halves of 32 bytes are touched per 32 lanes; a stride of 64 (mod 256)
+// bytes puts them on disjoint banks (measured: no conflicts), whereas 16-byte-odd strides conflict.
+typedef short v4i16_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ v4i16_t lds_read_tr16_b64(const void* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) v4i16_t*)(__attribute__((address_space(3))) void*)p);
+}
+
+// A operand (32 rows = features f0 + l32, 16-token chunk m in chunk order) of a token-major tile with
+// `stride_bytes` per token: lane_base = tr_lane_base(lane, stride_bytes), then for chunk m and feature tile
+// dt the two halves are at lane_base + (16*m + 8*half) * stride_bytes + 64*dt.
+__device__ __forceinline__ int tr_lane_base(int lane, int stride_bytes) {
+    const int g = lane >> 5, i = lane & 15, blk = (lane >> 4) & 1;
+    return (4 * g + (i >> 2)) * stride_bytes + (16 * blk + 4 * (i & 3)) * 2;
+}
+
+__device__ __forceinline__ bf16x8_t tr_operand(const char* tile, int lane_base, int stride_bytes, int m, int dt) {
+    const v4i16_t lo = lds_read_tr16_b64(tile + lane_base + (16 * m) * stride_bytes + 64 * dt);
+    const v4i16_t hi = lds_read_tr16_b64(tile + lane_base + (16 * m + 8) * stride_bytes + 64 * dt);
+    typedef short v8i16_t __attribute__((ext_vector_type(8)));
+    const v8i16_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8_t, both);
+}
+
+// 128-bit load / store through a native vector type.  Copying a uint4 (a struct) between address spaces
+// becomes a memcpy that keeps staging arrays in scratch memory; building the value element-wise lets
+// them live in registers.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint4 ld128(const void* p) {
+    const u32x4_t v = *reinterpret_cast<const u32x4_t*>(p);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
+__device__ __forceinline__ void st128(void* p, const uint4& x) {
+    u32x4_t v;
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+    *reinterpret_cast<u32x4_t*>(p) = v;
+}
+
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     bf16x2_t p;
     p[0] = (__bf16)lo;

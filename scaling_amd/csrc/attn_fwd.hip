@@ -10,7 +10,7 @@
 //                              only raised (and O rescaled) when it grows by more than 2^8, so the
 //                              rescale of the 64 accumulator registers is skipped on most tiles.
 //     O^T += V^T * P^T         B = P^T taken straight from the S^T accumulators (no LDS round trip),
-//                              A = V^T read from a transposed, chunk-ordered LDS copy of the V tile
+//                              A = V^T obtained with LDS transpose reads from the token-major V tile
 // The mask is a per-lane key interval [klo, khi) derived from the cumulative sequence lengths; tiles
 // outside the union of the intervals are never loaded, tiles inside every interval skip the compare.
 #include "attn_common.h"
@@ -26,13 +26,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     constexpr int KSTR = D + 8;           // padded K row (elements): conflict-free 128-bit row reads
     constexpr int KS = D / 16;            // contraction steps of Q K^T
     constexpr int DT = D / 32;            // 32-row tiles of O^T
-    constexpr int KV_VECS = D / 32;       // 128-bit K vectors per loader thread and tile
-    constexpr int V_ITEMS = 16 * (D / 8); // (key quad, 8-column group) items of a V tile
+    constexpr int KV_VECS = D / 32;       // 128-bit K (or V) vectors per loader thread and tile
+    constexpr int VSTR = D + 32;          // padded V row (elements): stride = 64 (mod 256) bytes for D = 64 / 128
     static_assert(D % 32 == 0 && D <= 128, "head_dim must be 32, 64, 96 or 128");
     static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts");
 
     __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KSTR];
-    __shared__ __attribute__((aligned(16))) uint16_t vt_lds[2][D * BN];
+    __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][BN * VSTR];
     __shared__ int range_lds[2 * NW];
 
     const int tid = threadIdx.x;
@@ -73,6 +73,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
     }
+    // Consume the Q registers here: otherwise their loads count as possibly outstanding at the loop
+    // entry, and every use inside the loop waits for the K/V prefetch issued just before it.
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         wmin = min(wmin, __shfl_xor(wmin, off, 64));
@@ -100,11 +104,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     const bool k_role = (NW == 4) || (tid >= 256);
     const int ltid = (NW == 4) ? tid : (tid & 255);
     uint4 kraw[KV_VECS];
-    uint4 vraw[4];
+    uint4 vraw[KV_VECS];
     uint4 craw[ROT ? KV_VECS / 2 : 1], sraw[ROT ? KV_VECS / 2 : 1];  // rotary table rows of the K tile
     const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
     const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
-    const int v_kg = ltid / (D / 8), v_dg = ltid % (D / 8);
     const int last_k = p.total_k - 1;
 
     auto load_tile = [&](int kt) {
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                     const int idx = ltid + 256 * j;
                     const int row = idx / (D / 8), c = idx % (D / 8);
                     const int tok = min(kt + row, last_k);
-                    kraw[j] = *reinterpret_cast<const uint4*>(kbase + (int64_t)tok * p.k_st + 8 * c);
+                    kraw[j] = ld128(kbase + (int64_t)tok * p.k_st + 8 * c);
                 }
             } else {
 #pragma unroll
@@ -124,20 +127,22 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                     const int row = idx / (D / 16), c = idx % (D / 16);
                     const int tok = min(kt + row, last_k);
                     const __bf16* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
-                    kraw[2 * j] = *reinterpret_cast<const uint4*>(kr);
-                    kraw[2 * j + 1] = *reinterpret_cast<const uint4*>(kr + D / 2);
+                    kraw[2 * j] = ld128(kr);
+                    kraw[2 * j + 1] = ld128(kr + D / 2);
                     int64_t pos = p.pos_k[tok];
                     pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
-                    craw[j] = *reinterpret_cast<const uint4*>(p.cos + pos * D + 8 * c);
-                    sraw[j] = *reinterpret_cast<const uint4*>(p.sin + pos * D + 8 * c);
+                    craw[j] = ld128(p.cos + pos * D + 8 * c);
+                    sraw[j] = ld128(p.sin + pos * D + 8 * c);
                 }
             }
         }
-        if (v_role && ltid < V_ITEMS) {
+        if (v_role) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int tok = min(kt + 4 * v_kg + j, last_k);
-                vraw[j] = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.v_st + 8 * v_dg);
+            for (int j = 0; j < KV_VECS; ++j) {
+                const int idx = ltid + 256 * j;
+                const int row = idx / (D / 8), c = idx % (D / 8);
+                const int tok = min(kt + row, last_k);
+                vraw[j] = ld128(vbase + (int64_t)tok * p.v_st + 8 * c);
             }
         }
     };
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 for (int j = 0; j < KV_VECS; ++j) {
                     const int idx = ltid + 256 * j;
                     const int row = idx / (D / 8), c = idx % (D / 8);
-                    *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[j];
+                    st128(ks + row * KSTR + 8 * c, kraw[j]);
                 }
             } else {
 #pragma unroll
@@ -158,16 +163,19 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                     const int idx = ltid + 256 * j;
                     const int row = idx / (D / 16), c = idx % (D / 16);
                     rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);  // after the MFMA section
-                    *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c) = kraw[2 * j];
-                    *reinterpret_cast<uint4*>(ks + row * KSTR + 8 * c + D / 2) = kraw[2 * j + 1];
+                    st128(ks + row * KSTR + 8 * c, kraw[2 * j]);
+                    st128(ks + row * KSTR + 8 * c + D / 2, kraw[2 * j + 1]);
                 }
             }
         }
-        if (v_role && ltid < V_ITEMS) {
-            char* vt = reinterpret_cast<char*>(vt_lds[buf]);
+        if (v_role) {
+            uint16_t* vs = v_lds[buf];
 #pragma unroll
-            for (int dd = 0; dd < 8; ++dd)
-                *reinterpret_cast<uint2*>(vt + chunk_quad_offset<BN>(8 * v_dg + dd, v_kg)) = transpose_quad(vraw, dd);
+            for (int j = 0; j < KV_VECS; ++j) {
+                const int idx = ltid + 256 * j;
+                const int row = idx / (D / 8), c = idx % (D / 8);
+                st128(vs + row * VSTR + 8 * c, vraw[j]);
+            }
         }
     };
 
@@ -179,6 +187,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     __syncthreads();
 
     const float c2 = p.scale_log2;
+    const int v_lane = tr_lane_base(lane, VSTR * 2);
     for (int it = 0; it < n_tiles; ++it) {
         const int kt = kt0 + it * BN;
         const int buf = it & 1;
@@ -187,7 +196,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         const bool wave_active = (kt < wmax) && (kt + BN > wmin);
         if (wave_active) {
             const uint16_t* ks = k_lds[buf] + l32 * KSTR + 8 * g;
-            const char* vt = reinterpret_cast<const char*>(vt_lds[buf]);
+            const char* vt = reinterpret_cast<const char*>(v_lds[buf]);
 
             f32x16_t s_acc[2];
 #pragma unroll
@@ -255,7 +264,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s_acc[t][r0 + e];
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(vt + chunk_unit_offset<BN>(32 * dt + l32, m, g));
+                    const bf16x8_t a = tr_operand(vt, v_lane, VSTR * 2, m, dt);
                     o_acc[dt] = mfma_32x32x16(a, pf, o_acc[dt]);
                 }
             }
