@@ -8,8 +8,9 @@
 //          dV^T += dO^T P        dK^T += Q^T dS         (P / dS feed the MFMA straight from registers)
 //   3. dQ: a workgroup owns 256 queries of one head (32 per wavefront, Q and dO fragments in registers),
 //      loops over 64-key tiles:  S^T = K Q^T, dP^T = V dO^T, dS^T, dQ^T += K^T dS^T.
-// Operands whose contraction index is a token index are kept in LDS transposed and "chunk ordered"
-// (see attn_common.h) so that score tiles can be consumed in their accumulator layout.
+// Tiles whose rows are needed both as row operands and transposed (Q / dO in kernel 2, K in kernel 3) are
+// staged once, token-major, in a layout that serves plain 128-bit reads and LDS transpose reads without
+// bank conflicts (TokTile in attn_common.h); score tiles are consumed in their accumulator layout.
 #include "attn_common.h"
 
 namespace {
@@ -43,65 +44,38 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_delta_kernel(const AttnPara
 }
 
 // ---------------------------------------------------------------------------------------------
-// helpers shared by kernels 2 and 3: stage a 64-token tile (row-major, padded) and its transposed
-// chunk-ordered copy from a thread-owned block of 4 tokens x 8 features
-// ---------------------------------------------------------------------------------------------
-template <int D>
-__device__ __forceinline__ void load_quad(uint4 (&raw)[4], const __bf16* base, int64_t stride, int tok0, int total,
-                                          int quad, int dg) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        int tok = tok0 + 4 * quad + j;
-        tok = tok < total ? tok : total - 1;
-        raw[j] = *reinterpret_cast<const uint4*>(base + (int64_t)tok * stride + 8 * dg);
-    }
-}
-
-template <int STR>
-__device__ __forceinline__ void store_rows(const uint4 (&raw)[4], uint16_t* rm, int quad, int dg) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(rm + (4 * quad + j) * STR + 8 * dg) = raw[j];
-}
-
-__device__ __forceinline__ void store_transposed(const uint4 (&raw)[4], char* tr, int quad, int dg) {
-#pragma unroll
-    for (int dd = 0; dd < 8; ++dd)
-        *reinterpret_cast<uint2*>(tr + chunk_quad_offset<64>(8 * dg + dd, quad)) = transpose_quad(raw, dd);
-}
-
-// ---------------------------------------------------------------------------------------------
 // 2. dK / dV
 // ---------------------------------------------------------------------------------------------
 // 8 wavefronts, two per SIMD.  The workgroup owns 128 keys of one KV head whose K and V rows stay in
 // LDS for its lifetime; wavefront w works on key group (w & 3) (32 keys) and on query sub-tile (w >> 2)
 // (32 of the 64 queries staged per iteration), so the pair (w, w + 4) accumulates the same dK / dV
-// rows and is summed once at the end.  The first four wavefronts stage Q, the last four dO.
+// rows and is summed once at the end.  The first four wavefronts stage Q, the last four dO; the staged
+// tiles are double buffered (one barrier per iteration).
 template <int D>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
     constexpr int NT = 512;
     constexpr int BNK = 128;              // keys per workgroup
     constexpr int BQ = 64;                // queries per tile
-    constexpr int STR = D + 8;
+    constexpr int STR = D + 8;            // K / V rows (elements): row operands only
     constexpr int KS = D / 16;
     constexpr int DT = D / 32;
-    constexpr int ITEMS = 16 * (D / 8);
+    constexpr int VECS = (BQ * (D / 8)) / 256;   // 128-bit vectors per loader thread and tile
+    using Tile = TokTile<D>;
+    constexpr int TSTR = Tile::kStride;
     constexpr int KV_BYTES = BNK * STR * 2;
-    constexpr int QROW_BYTES = BQ * STR * 2;
-    constexpr int QTR_BYTES = D * BQ * 2;
-    constexpr int STAGE_BYTES = 2 * KV_BYTES + 2 * QROW_BYTES + 2 * QTR_BYTES;
+    constexpr int TILE_BYTES = BQ * TSTR;
+    constexpr int STAGE_BYTES = 2 * KV_BYTES + 4 * TILE_BYTES;
     constexpr int RED_BYTES = 4 * 16 * DT * 64 * 4;   // one accumulator set of four wavefronts
     constexpr int SMEM_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
 
     __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
-    __shared__ __attribute__((aligned(16))) float lse_lds[BQ];
-    __shared__ __attribute__((aligned(16))) float delta_lds[BQ];
+    __shared__ __attribute__((aligned(16))) float lse_lds[2][BQ];
+    __shared__ __attribute__((aligned(16))) float delta_lds[2][BQ];
     __shared__ int range_lds[16];
     uint16_t* k_rm = reinterpret_cast<uint16_t*>(smem);
     uint16_t* v_rm = reinterpret_cast<uint16_t*>(smem + KV_BYTES);
-    uint16_t* q_rm = reinterpret_cast<uint16_t*>(smem + 2 * KV_BYTES);
-    uint16_t* do_rm = reinterpret_cast<uint16_t*>(smem + 2 * KV_BYTES + QROW_BYTES);
-    char* q_tr = smem + 2 * KV_BYTES + 2 * QROW_BYTES;
-    char* do_tr = q_tr + QTR_BYTES;
+    char* q_t = smem + 2 * KV_BYTES;                   // [2][BQ rows]
+    char* do_t = q_t + 2 * TILE_BYTES;                 // [2][BQ rows]
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -132,8 +106,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             const int idx = tid + NT * j;
             const int row = idx / (D / 8), c = idx % (D / 8);
             const int tok = min(kb * BNK + row, p.total_k - 1);
-            *reinterpret_cast<uint4*>(k_rm + row * STR + 8 * c) = *reinterpret_cast<const uint4*>(kbase + (int64_t)tok * p.k_st + 8 * c);
-            *reinterpret_cast<uint4*>(v_rm + row * STR + 8 * c) = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.v_st + 8 * c);
+            st128(k_rm + row * STR + 8 * c, ld128(kbase + (int64_t)tok * p.k_st + 8 * c));
+            st128(v_rm + row * STR + 8 * c, ld128(vbase + (int64_t)tok * p.v_st + 8 * c));
         }
     }
     __syncthreads();
@@ -152,8 +126,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 
     const bool q_role = tid < 256;
     const int ltid = tid & 255;
-    const int quad = ltid / (D / 8), dg = ltid % (D / 8);
-    uint4 raw[4];
+    uint4 raw[VECS];
     float stat = 0.f;
 
     // Query tiles are visited from the last one downwards: under a causal mask every key block of a
@@ -163,54 +136,73 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     // Role-dependent sources are selected once, as values: a per-iteration select between kernel
     // arguments turns into a load of the argument through a vector address, and a wait on it.
     const __bf16* src_base = q_role ? p.q : p.d_o;
-    int64_t src_head_stride = q_role ? p.q_sh : p.o_sh;
-    int64_t src_tok_stride = q_role ? p.q_st : p.o_st;
+    const int64_t src_head_stride = q_role ? p.q_sh : p.o_sh;
+    const int64_t src_tok_stride = q_role ? p.q_st : p.o_st;
     const float* stat_base = (tid < BQ) ? p.lse : p.delta;
     const float stat_scale = (tid < BQ) ? 1.4426950408889634f : 1.0f;  // log-sum-exp goes to the exp2 domain
+    char* dst_tile = q_role ? q_t : do_t;
+    const int last_q = p.total_q - 1;
     auto load_tile = [&](int iter) {
         const int rep = iter / n_tiles, qt = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ;
         const int head = kvh * p.n_rep + rep;
-        if (ltid < ITEMS) load_quad<D>(raw, src_base + (int64_t)head * src_head_stride, src_tok_stride, qt, p.total_q, quad, dg);
+        const __bf16* base = src_base + (int64_t)head * src_head_stride;
+#pragma unroll
+        for (int j = 0; j < VECS; ++j) {
+            const int idx = ltid + 256 * j;
+            const int row = idx / (D / 8), c = idx % (D / 8);
+            const int tok = min(qt + row, last_q);
+            raw[j] = ld128(base + (int64_t)tok * src_tok_stride + 8 * c);
+        }
         if (tid < 2 * BQ) {
-            const int tok = min(qt + (tid & (BQ - 1)), p.total_q - 1);
+            const int tok = min(qt + (tid & (BQ - 1)), last_q);
             stat = stat_base[(int64_t)head * p.total_q + tok];
         }
     };
-    auto store_tile = [&]() {
-        if (ltid < ITEMS) {
-            store_rows<STR>(raw, q_role ? q_rm : do_rm, quad, dg);
-            store_transposed(raw, q_role ? q_tr : do_tr, quad, dg);
+    auto store_tile = [&](int buf) {
+        char* dst = dst_tile + buf * TILE_BYTES;
+#pragma unroll
+        for (int j = 0; j < VECS; ++j) {
+            const int idx = ltid + 256 * j;
+            const int row = idx / (D / 8), c = idx % (D / 8);
+            st128(dst + Tile::unit_offset(row, c), raw[j]);
         }
-        if (tid < BQ) lse_lds[tid] = stat * stat_scale;
-        else if (tid < 2 * BQ) delta_lds[tid - BQ] = stat * stat_scale;
+        if (tid < BQ) lse_lds[buf][tid] = stat * stat_scale;
+        else if (tid < 2 * BQ) delta_lds[buf][tid - BQ] = stat * stat_scale;
     };
 
     if (total_iters > 0) {
         load_tile(0);
-        store_tile();
+        store_tile(0);
     }
     __syncthreads();
 
-    const uint16_t* a_q = q_rm + (32 * sub + l32) * STR + 8 * g;
-    const uint16_t* a_do = do_rm + (32 * sub + l32) * STR + 8 * g;
+    int row_even, row_odd, tr_h0, tr_h1;
+    Tile::row_bases(32 * sub + l32, g, row_even, row_odd);
+    Tile::tr_bases(lane, tr_h0, tr_h1);
+    tr_h0 += 32 * sub * TSTR;
+    tr_h1 += 32 * sub * TSTR;
     const uint16_t* b_k = k_rm + (32 * kgp + l32) * STR + 8 * g;
     const uint16_t* b_v = v_rm + (32 * kgp + l32) * STR + 8 * g;
     const float c2 = p.scale_log2;
 
     for (int iter = 0; iter < total_iters; ++iter) {
+        const int buf = iter & 1;
         const int qs = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ + 32 * sub;
         if (iter + 1 < total_iters) load_tile(iter + 1);
 
         if ((qs < wmax) && (qs + 32 > wmin)) {
+            const char* qt_ = q_t + buf * TILE_BYTES;
+            const char* dt_ = do_t + buf * TILE_BYTES;
             f32x16_t s_acc, dp_acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) { s_acc[r] = 0.f; dp_acc[r] = 0.f; }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(a_q + 16 * ks);
+                const int ro = ((ks & 1) ? row_odd : row_even) + 32 * ks;
+                const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(qt_ + ro);
                 const bf16x8_t bk = *reinterpret_cast<const bf16x8_t*>(b_k + 16 * ks);
                 s_acc = mfma_32x32x16(aq, bk, s_acc);
-                const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(a_do + 16 * ks);
+                const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(dt_ + ro);
                 const bf16x8_t bv = *reinterpret_cast<const bf16x8_t*>(b_v + 16 * ks);
                 dp_acc = mfma_32x32x16(ad, bv, dp_acc);
             }
@@ -228,8 +220,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             bf16x8_t pf[2], dsf[2];
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(lse_lds + 32 * sub + 8 * a + 4 * g);
-                const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(delta_lds + 32 * sub + 8 * a + 4 * g);
+                const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(&lse_lds[buf][32 * sub + 8 * a + 4 * g]);
+                const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(&delta_lds[buf][32 * sub + 8 * a + 4 * g]);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int r = 4 * a + c;
@@ -243,15 +235,15 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             for (int m = 0; m < 2; ++m) {
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t adt = *reinterpret_cast<const bf16x8_t*>(do_tr + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
-                    const bf16x8_t aqt = *reinterpret_cast<const bf16x8_t*>(q_tr + chunk_unit_offset<64>(32 * dt + l32, 2 * sub + m, g));
+                    const int off = 16 * m * TSTR + 64 * dt;
+                    const bf16x8_t adt = tr_pair(dt_ + tr_h0 + off, dt_ + tr_h1 + off);
+                    const bf16x8_t aqt = tr_pair(qt_ + tr_h0 + off, qt_ + tr_h1 + off);
                     dv_acc[dt] = mfma_32x32x16(adt, pf[m], dv_acc[dt]);
                     dk_acc[dt] = mfma_32x32x16(aqt, dsf[m], dk_acc[dt]);
                 }
             }
         }
-        __syncthreads();
-        if (iter + 1 < total_iters) store_tile();
+        if (iter + 1 < total_iters) store_tile(buf ^ 1);
         __syncthreads();
     }
 
@@ -296,8 +288,9 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 // ---------------------------------------------------------------------------------------------
 // 3. dQ
 // ---------------------------------------------------------------------------------------------
-// 8 wavefronts, two per SIMD, 32 queries each (256 per workgroup); the first four stage K (rows and the
-// transposed copy), the last four stage V.  Double-buffered LDS, one barrier per 64-key tile.
+// 8 wavefronts, two per SIMD, 32 queries each (256 per workgroup); the first four stage K (one
+// token-major tile read both as row operand and transposed), the last four stage V.  Double-buffered
+// LDS, one barrier per 64-key tile.
 template <int D>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p) {
     constexpr int BM = 256;
@@ -305,11 +298,12 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     constexpr int STR = D + 8;
     constexpr int KS = D / 16;
     constexpr int DT = D / 32;
-    constexpr int ITEMS = 16 * (D / 8);
+    constexpr int VECS = (BN * (D / 8)) / 256;   // 128-bit vectors per loader thread and tile
+    using Tile = TokTile<D>;
+    constexpr int TSTR = Tile::kStride;
 
-    __shared__ __attribute__((aligned(16))) uint16_t k_rm[2][BN * STR];
-    __shared__ __attribute__((aligned(16))) uint16_t v_rm[2][BN * STR];
-    __shared__ __attribute__((aligned(16))) uint16_t k_tr[2][D * BN];
+    __shared__ __attribute__((aligned(16))) char k_t[2][BN * TSTR];        // row operand and transposed operand
+    __shared__ __attribute__((aligned(16))) uint16_t v_rm[2][BN * STR];    // row operand only
     __shared__ int range_lds[16];
 
     const int tid = threadIdx.x;
@@ -369,25 +363,28 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
 
     const bool k_role = tid < 256;
     const int ltid = tid & 255;
-    const int quad = ltid / (D / 8), dg = ltid % (D / 8);
-    uint4 raw[4];
-    const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
-    const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
+    uint4 raw[VECS];
+    // selected once, as values (see the dK / dV kernel)
+    const __bf16* src_base = k_role ? p.k + (int64_t)kvh * p.k_sh : p.v + (int64_t)kvh * p.v_sh;
+    const int64_t src_tok_stride = k_role ? p.k_st : p.v_st;
+    const int last_k = p.total_k - 1;
 
     auto load_tile = [&](int kt) {
-        if (ltid < ITEMS) {
-            if (k_role) load_quad<D>(raw, kbase, p.k_st, kt, p.total_k, quad, dg);
-            else load_quad<D>(raw, vbase, p.v_st, kt, p.total_k, quad, dg);
+#pragma unroll
+        for (int j = 0; j < VECS; ++j) {
+            const int idx = ltid + 256 * j;
+            const int row = idx / (D / 8), c = idx % (D / 8);
+            const int tok = min(kt + row, last_k);
+            raw[j] = ld128(src_base + (int64_t)tok * src_tok_stride + 8 * c);
         }
     };
     auto store_tile = [&](int buf) {
-        if (ltid < ITEMS) {
-            if (k_role) {
-                store_rows<STR>(raw, k_rm[buf], quad, dg);
-                store_transposed(raw, reinterpret_cast<char*>(k_tr[buf]), quad, dg);
-            } else {
-                store_rows<STR>(raw, v_rm[buf], quad, dg);
-            }
+#pragma unroll
+        for (int j = 0; j < VECS; ++j) {
+            const int idx = ltid + 256 * j;
+            const int row = idx / (D / 8), c = idx % (D / 8);
+            if (k_role) st128(k_t[buf] + Tile::unit_offset(row, c), raw[j]);
+            else st128(v_rm[buf] + row * STR + 8 * c, raw[j]);
         }
     };
 
@@ -398,15 +395,17 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     __syncthreads();
 
     const float c2 = p.scale_log2;
+    int row_even, row_odd, tr_h0, tr_h1;
+    Tile::row_bases(l32, g, row_even, row_odd);
+    Tile::tr_bases(lane, tr_h0, tr_h1);
     for (int it = 0; it < n_tiles; ++it) {
         const int kt = kt0 + it * BN;
         const int buf = it & 1;
         if (it + 1 < n_tiles) load_tile(kt + BN);
 
         if ((kt < wmax) && (kt + BN > wmin)) {
-            const uint16_t* a_k = k_rm[buf] + l32 * STR + 8 * g;
+            const char* kt_ = k_t[buf];
             const uint16_t* a_v = v_rm[buf] + l32 * STR + 8 * g;
-            const char* a_kt = reinterpret_cast<const char*>(k_tr[buf]);
             f32x16_t s_acc[2], dp_acc[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
@@ -414,9 +413,10 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                 for (int r = 0; r < 16; ++r) { s_acc[t][r] = 0.f; dp_acc[t][r] = 0.f; }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
+                const int ro = ((ks & 1) ? row_odd : row_even) + 32 * ks;
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(a_k + 32 * t * STR + 16 * ks);
+                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(kt_ + ro + 32 * t * TSTR);
                     s_acc[t] = mfma_32x32x16(ak, qf[ks], s_acc[t]);
                     const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(a_v + 32 * t * STR + 16 * ks);
                     dp_acc[t] = mfma_32x32x16(av, dof[ks], dp_acc[t]);
@@ -445,7 +445,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                 }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t akt = *reinterpret_cast<const bf16x8_t*>(a_kt + chunk_unit_offset<64>(32 * dt + l32, m, g));
+                    const int off = 16 * m * TSTR + 64 * dt;
+                    const bf16x8_t akt = tr_pair(kt_ + tr_h0 + off, kt_ + tr_h1 + off);
                     dq_acc[dt] = mfma_32x32x16(akt, dsf, dq_acc[dt]);
                 }
             }

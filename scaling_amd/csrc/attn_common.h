@@ -75,39 +75,6 @@ __device__ __forceinline__ void query_range(const AttnParams& p, int u, int& qlo
     if (qlo > qhi) qlo = qhi;
 }
 
-// ---- "chunk order" LDS layout for operands whose contraction index is the row index of a C tile ----
-// A [R rows][64 contraction] matrix is stored row-major (128 bytes per row) with the 16-byte units of a
-// row XOR-swizzled; inside each 16-wide chunk the contraction indices are permuted so that lane group
-// g finds its 8 k-slots contiguous: unit (2*m + g) of row r holds indices 16*m + {4g..4g+3, 8+4g..8+4g+3}.
-// The swizzle depends on (row & 31) only, so the address of (row + 32*dt) is the address of row plus
-// an immediate, and 16 consecutive rows read by one lane group hit 16 different bank quads.
-__device__ __forceinline__ int swz(int row) { return ((row >> 1) & 7) ^ ((row >> 3) & 3); }
-
-// byte offset of the 8-byte group holding contraction indices 4*quad .. 4*quad+3 (quad = index / 4)
-template <int N> __device__ __forceinline__ int chunk_quad_offset(int row, int quad) {
-    static_assert(N == 64, "one row = 8 swizzled units of 16 bytes");
-    const int m = quad >> 2, kq = quad & 3;
-    const int unit = 2 * m + (kq & 1);
-    return row * (N * 2) + ((unit ^ swz(row)) << 4) + ((kq >> 1) << 3);
-}
-
-// byte offset of the 16-byte unit read by lane group g for chunk m of row `row`
-template <int N> __device__ __forceinline__ int chunk_unit_offset(int row, int m, int g) {
-    static_assert(N == 64, "one row = 8 swizzled units of 16 bytes");
-    return row * (N * 2) + (((2 * m + g) ^ swz(row)) << 4);
-}
-
-// 4 tokens x 8 features held as 4 row vectors -> for feature dd the 4 token values as one 8-byte group
-__device__ __forceinline__ uint2 transpose_quad(const uint4 (&raw)[4], int dd) {
-    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&raw[0]);
-    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&raw[1]);
-    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&raw[2]);
-    const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&raw[3]);
-    const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of the two words
-    return make_uint2(__builtin_amdgcn_perm(w1[dd >> 1], w0[dd >> 1], sel),
-                      __builtin_amdgcn_perm(w3[dd >> 1], w2[dd >> 1], sel));
-}
-
 // ---- LDS transpose read (gfx950 ds_read_b64_tr_b16) ---------------------------------------------------
 // Within each block of 16 lanes the instruction loads 16 x 8 bytes and hands lane j the j-th 16-bit element
 // of each of the four 32-byte rows formed by lanes {0..3}, {4..7}, {8..11}, {12..15}.  With a token-major
@@ -123,20 +90,74 @@ __device__ __forceinline__ v4i16_t lds_read_tr16_b64(const void* p) {
         (__attribute__((address_space(3))) v4i16_t*)(__attribute__((address_space(3))) void*)p);
 }
 
-// A operand (32 rows = features f0 + l32, 16-token chunk m in chunk order) of a token-major tile with
-// `stride_bytes` per token: lane_base = tr_lane_base(lane, stride_bytes), then for chunk m and feature tile
-// dt the two halves are at lane_base + (16*m + 8*half) * stride_bytes + 64*dt.
+// "Chunk order": a 32x32 accumulator tile holds, for lane group g, rows 8*(r/4) + 4g + r%4 in register r.
+// Used as the B operand of the next product (contraction over those rows), k-slot i of lane group g of
+// 16-row chunk m is row 16m + 8*(i/4) + 4g + i%4, so the matching A operand takes tokens
+// 16m + 4g + {0..3} (first transpose read) and 16m + 8 + 4g + {0..3} (second).
+typedef short v8i16_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ bf16x8_t tr_pair(const char* lo_addr, const char* hi_addr) {
+    const v4i16_t lo = lds_read_tr16_b64(lo_addr);
+    const v4i16_t hi = lds_read_tr16_b64(hi_addr);
+    const v8i16_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8_t, both);
+}
+
+// Plain token-major tile (stride = 64 mod 256 bytes) that is only read transposed.
+// lane_base = tr_lane_base(lane, stride); chunk m, feature tile dt: see tr_operand.
 __device__ __forceinline__ int tr_lane_base(int lane, int stride_bytes) {
     const int g = lane >> 5, i = lane & 15, blk = (lane >> 4) & 1;
     return (4 * g + (i >> 2)) * stride_bytes + (16 * blk + 4 * (i & 3)) * 2;
 }
 
 __device__ __forceinline__ bf16x8_t tr_operand(const char* tile, int lane_base, int stride_bytes, int m, int dt) {
-    const v4i16_t lo = lds_read_tr16_b64(tile + lane_base + (16 * m) * stride_bytes + 64 * dt);
-    const v4i16_t hi = lds_read_tr16_b64(tile + lane_base + (16 * m + 8) * stride_bytes + 64 * dt);
-    typedef short v8i16_t __attribute__((ext_vector_type(8)));
-    const v8i16_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8_t, both);
+    return tr_pair(tile + lane_base + (16 * m) * stride_bytes + 64 * dt,
+                   tile + lane_base + (16 * m + 8) * stride_bytes + 64 * dt);
+}
+
+// Token-major tile that is read both ways without bank conflicts: as a row operand (lane = token,
+// 16 bytes of features per k-step) and transposed (lane = feature, k-slots = tokens).  The row stride is
+// 4 or 12 (mod 16) 16-byte units and the unit index of a row is XORed with ((row >> 2) & 3):
+//   row operand   16 consecutive rows at one k-step land on 16 different units (mod 16),
+//   transposed    the 4 rows x 2 x 32 bytes touched by 32 lanes land on 16 different units (mod 16),
+//   loader        the units of one row are permuted inside aligned groups of four.
+// Rows of a tile start at a multiple of 16, so the XOR term of a lane is fixed per operand.
+template <int D> struct TokTile {
+    static constexpr int kStride = (D == 128) ? 320 : (D == 32 ? 64 : 192);   // bytes per token
+    static_assert(D == 32 || D == 64 || D == 96 || D == 128, "head_dim");
+
+    // byte offset of 16-byte unit c of row r (loader side)
+    static __device__ __forceinline__ int unit_offset(int r, int c) {
+        return r * kStride + ((c ^ ((r >> 2) & 3)) << 4);
+    }
+    // row operand of lane (row, g): k-step ks is at (ks even ? even : odd) + 32 * ks
+    static __device__ __forceinline__ void row_bases(int row, int g, int& even, int& odd) {
+        const int a = (row >> 2) & 3;
+        const int rb = row * kStride + ((g ^ (a & 1)) << 4);
+        even = rb + 32 * (a >> 1);
+        odd = rb - 32 * (a >> 1);
+    }
+    // transposed operand: chunk m (16 tokens, chunk order), feature tile dt (32 features):
+    //   tr_pair(tile + h0 + 16*m*kStride + 64*dt, tile + h1 + 16*m*kStride + 64*dt)
+    static __device__ __forceinline__ void tr_bases(int lane, int& h0, int& h1) {
+        const int g = lane >> 5, i = lane & 15, blk = (lane >> 4) & 1;
+        const int row = 4 * g + (i >> 2);
+        const int u = 2 * blk + ((i >> 1) & 1);
+        const int byte = (i & 1) * 8;
+        h0 = row * kStride + ((u ^ g) << 4) + byte;
+        h1 = (row + 8) * kStride + ((u ^ (2 + g)) << 4) + byte;
+    }
+};
+
+// 4 tokens x 8 features held as 4 row vectors -> for feature dd the 4 token values as one 8-byte group
+__device__ __forceinline__ uint2 transpose_quad(const uint4 (&raw)[4], int dd) {
+    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&raw[0]);
+    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&raw[1]);
+    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&raw[2]);
+    const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&raw[3]);
+    const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of the two words
+    return make_uint2(__builtin_amdgcn_perm(w1[dd >> 1], w0[dd >> 1], sel),
+                      __builtin_amdgcn_perm(w3[dd >> 1], w2[dd >> 1], sel));
 }
 
 // 128-bit load / store through a native vector type.  Copying a uint4 (a struct) between address spaces
