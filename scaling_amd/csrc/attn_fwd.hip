@@ -1,8 +1,9 @@
 // Attention forward for gfx950 (bf16 MFMA, fp32 online softmax, causal / packed-document masks, GQA).
 //
-// Workgroup = NW wavefronts (4 or 8); every wavefront owns 32 consecutive query tokens of one head and
-// two wavefronts share a SIMD, so one can issue MFMAs while the other runs its softmax on the VALU.
-// Keys/values stream through LDS in tiles of 64 tokens (double buffered, one barrier per tile).
+// Workgroup = NW wavefronts (4 or 8); every wavefront owns 32 consecutive query tokens of one head.
+// With 8 wavefronts, wavefronts w and w + 4 share a SIMD and run half a tile out of phase (enforced by
+// the barriers), so one issues MFMAs while the other runs its softmax on the VALU.
+// Keys/values stream through LDS in tiles of 64 tokens (double buffered).
 // Per tile:
 //     S^T = K * Q^T            A = K tile rows from LDS, B = Q fragment held in registers
 //     online softmax           each lane owns ONE query (C column): the row max / sum are in-lane
@@ -14,6 +15,8 @@
 // The mask is a per-lane key interval [klo, khi) derived from the cumulative sequence lengths; tiles
 // outside the union of the intervals are never loaded, tiles inside every interval skip the compare.
 #include "attn_common.h"
+
+#include <type_traits>
 
 namespace {
 
@@ -106,112 +109,188 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     uint4 kraw[KV_VECS];
     uint4 vraw[KV_VECS];
     uint4 craw[ROT ? KV_VECS / 2 : 1], sraw[ROT ? KV_VECS / 2 : 1];  // rotary table rows of the K tile
+    int64_t kpos[ROT ? KV_VECS / 2 : 1];                             // their positions, fetched a tile ahead
     const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
     const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
     const int last_k = p.total_k - 1;
 
-    auto load_tile = [&](int kt) {
-        if (k_role) {
-            if constexpr (!ROT) {
+    auto load_kpos = [&](int kt) {
+        if constexpr (ROT) {
 #pragma unroll
-                for (int j = 0; j < KV_VECS; ++j) {
-                    const int idx = ltid + 256 * j;
-                    const int row = idx / (D / 8), c = idx % (D / 8);
-                    const int tok = min(kt + row, last_k);
-                    kraw[j] = ld128(kbase + (int64_t)tok * p.k_st + 8 * c);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < KV_VECS / 2; ++j) {
-                    const int idx = ltid + 256 * j;
-                    const int row = idx / (D / 16), c = idx % (D / 16);
-                    const int tok = min(kt + row, last_k);
-                    const __bf16* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
-                    kraw[2 * j] = ld128(kr);
-                    kraw[2 * j + 1] = ld128(kr + D / 2);
-                    int64_t pos = p.pos_k[tok];
-                    pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
-                    craw[j] = ld128(p.cos + pos * D + 8 * c);
-                    sraw[j] = ld128(p.sin + pos * D + 8 * c);
-                }
+            for (int j = 0; j < KV_VECS / 2; ++j) {
+                const int row = (ltid + 256 * j) / (D / 16);
+                kpos[j] = p.pos_k[min(kt + row, last_k)];
             }
         }
-        if (v_role) {
+    };
+    auto load_k = [&](int kt) {
+        if constexpr (!ROT) {
 #pragma unroll
             for (int j = 0; j < KV_VECS; ++j) {
                 const int idx = ltid + 256 * j;
                 const int row = idx / (D / 8), c = idx % (D / 8);
                 const int tok = min(kt + row, last_k);
-                vraw[j] = ld128(vbase + (int64_t)tok * p.v_st + 8 * c);
+                kraw[j] = ld128(kbase + (int64_t)tok * p.k_st + 8 * c);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < KV_VECS / 2; ++j) {
+                const int idx = ltid + 256 * j;
+                const int row = idx / (D / 16), c = idx % (D / 16);
+                const int tok = min(kt + row, last_k);
+                const __bf16* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
+                kraw[2 * j] = ld128(kr);
+                kraw[2 * j + 1] = ld128(kr + D / 2);
+                int64_t pos = kpos[j];
+                pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+                craw[j] = ld128(p.cos + pos * D + 8 * c);
+                sraw[j] = ld128(p.sin + pos * D + 8 * c);
             }
         }
     };
-
-    auto store_tile = [&](int buf) {
-        if (k_role) {
-            uint16_t* ks = k_lds[buf];
-            if constexpr (!ROT) {
-#pragma unroll
-                for (int j = 0; j < KV_VECS; ++j) {
-                    const int idx = ltid + 256 * j;
-                    const int row = idx / (D / 8), c = idx % (D / 8);
-                    st128(ks + row * KSTR + 8 * c, kraw[j]);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < KV_VECS / 2; ++j) {
-                    const int idx = ltid + 256 * j;
-                    const int row = idx / (D / 16), c = idx % (D / 16);
-                    rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);  // after the MFMA section
-                    st128(ks + row * KSTR + 8 * c, kraw[2 * j]);
-                    st128(ks + row * KSTR + 8 * c + D / 2, kraw[2 * j + 1]);
-                }
-            }
-        }
-        if (v_role) {
-            uint16_t* vs = v_lds[buf];
+    auto store_k = [&](int buf) {
+        uint16_t* ks = k_lds[buf];
+        if constexpr (!ROT) {
 #pragma unroll
             for (int j = 0; j < KV_VECS; ++j) {
                 const int idx = ltid + 256 * j;
                 const int row = idx / (D / 8), c = idx % (D / 8);
-                st128(vs + row * VSTR + 8 * c, vraw[j]);
+                st128(ks + row * KSTR + 8 * c, kraw[j]);
             }
+        } else {
+#pragma unroll
+            for (int j = 0; j < KV_VECS / 2; ++j) {
+                const int idx = ltid + 256 * j;
+                const int row = idx / (D / 16), c = idx % (D / 16);
+                rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);
+                st128(ks + row * KSTR + 8 * c, kraw[2 * j]);
+                st128(ks + row * KSTR + 8 * c + D / 2, kraw[2 * j + 1]);
+            }
+        }
+    };
+    auto load_v = [&](int kt) {
+#pragma unroll
+        for (int j = 0; j < KV_VECS; ++j) {
+            const int idx = ltid + 256 * j;
+            const int row = idx / (D / 8), c = idx % (D / 8);
+            const int tok = min(kt + row, last_k);
+            vraw[j] = ld128(vbase + (int64_t)tok * p.v_st + 8 * c);
+        }
+    };
+    auto store_v = [&](int buf) {
+        uint16_t* vs = v_lds[buf];
+#pragma unroll
+        for (int j = 0; j < KV_VECS; ++j) {
+            const int idx = ltid + 256 * j;
+            const int row = idx / (D / 8), c = idx % (D / 8);
+            st128(vs + row * VSTR + 8 * c, vraw[j]);
         }
     };
 
     // ---- main loop ---------------------------------------------------------------------------
+    // Each wavefront alternates an MFMA phase (O^T += V^T P^T of the previous tile, then S^T of the
+    // current one) and a VALU phase (softmax of the current tile), with a workgroup barrier after each.
+    // The second group of four wavefronts runs one phase behind the first, so on every SIMD one
+    // wavefront is in its MFMA phase while the other is in its VALU phase.
+    //   K tile n is read in phases 2n (group 0) and 2n+1 (group 1): it is stored during phase 2n-1;
+    //   V tile n is read in phases 2n+2 and 2n+3: it is stored during phase 2n.
+    // wave-uniform by construction: the extra barriers below must sit behind scalar branches
+    const int grp = (NW == 8) ? __builtin_amdgcn_readfirstlane(wave >> 2) : 0;
     if (n_tiles > 0) {
-        load_tile(kt0);
-        store_tile(0);
+        if (k_role) {
+            load_kpos(kt0);
+            load_k(kt0);
+            if (n_tiles > 1) load_kpos(kt0 + BN);
+            store_k(0);
+            if (n_tiles > 1) {
+                load_k(kt0 + BN);
+                if (n_tiles > 2) load_kpos(kt0 + 2 * BN);
+            }
+        }
+        if (v_role) load_v(kt0);
     }
     __syncthreads();
+    if (grp == 1) __syncthreads();
 
     const float c2 = p.scale_log2;
     const int v_lane = tr_lane_base(lane, VSTR * 2);
-    for (int it = 0; it < n_tiles; ++it) {
-        const int kt = kt0 + it * BN;
-        const int buf = it & 1;
-        if (it + 1 < n_tiles) load_tile(kt + BN);
+    const uint16_t* k_lane = k_lds[0] + l32 * KSTR + 8 * g;
+    f32x16_t s_acc[2];
+    bf16x8_t pf[4];
+    bool pending = false;                 // pf holds the probabilities of the previous tile
 
-        const bool wave_active = (kt < wmax) && (kt + BN > wmin);
-        if (wave_active) {
-            const uint16_t* ks = k_lds[buf] + l32 * KSTR + 8 * g;
-            const char* vt = reinterpret_cast<const char*>(v_lds[buf]);
-
-            f32x16_t s_acc[2];
+    // One MFMA phase = up to 16 steps of O^T += V^T P^T (previous tile) followed by up to 16 steps of
+    // S^T = K Q^T (current tile).  The A operands come from LDS through a ring of kDepth registers
+    // filled kDepth steps ahead, so a wavefront that has its SIMD's matrix core to itself keeps it fed
+    // in spite of the LDS latency; sched_barrier pins that order.
+    constexpr int PV_STEPS = 4 * DT, S_STEPS = 2 * KS;
+    constexpr int kDepth = 6;
+    auto mfma_phase = [&](auto mode, const char* vt, const uint16_t* ks) {
+        constexpr bool kPV = (decltype(mode)::value & 1) != 0, kS = (decltype(mode)::value & 2) != 0;
+        constexpr int first = kPV ? 0 : PV_STEPS, last = kS ? PV_STEPS + S_STEPS : PV_STEPS;
+        bf16x8_t ring[kDepth];
+        auto fetch = [&](int i) -> bf16x8_t {
+            if (i < PV_STEPS) {
+                const int m = i / DT, dt = i % DT;
+                return tr_pair(vt + (16 * m) * (VSTR * 2) + 64 * dt, vt + (16 * m + 8) * (VSTR * 2) + 64 * dt);
+            }
+            const int ksi = (i - PV_STEPS) >> 1, t = (i - PV_STEPS) & 1;
+            return *reinterpret_cast<const bf16x8_t*>(ks + 32 * t * KSTR + 16 * ksi);
+        };
+        if constexpr (kS) {
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s_acc[t][r] = 0.f;
+        }
 #pragma unroll
-            for (int ksi = 0; ksi < KS; ++ksi) {
+        for (int i = first; i < first + kDepth && i < last; ++i) ring[(i - first) % kDepth] = fetch(i);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks + 32 * t * KSTR + 16 * ksi);
-                    s_acc[t] = mfma_32x32x16(a, qf[ksi], s_acc[t]);
+        for (int i = first; i < last; ++i) {
+            const bf16x8_t a = ring[(i - first) % kDepth];
+            if (i < PV_STEPS) {
+                const int m = i / DT, dt = i % DT;
+                o_acc[dt] = mfma_32x32x16(a, pf[m], o_acc[dt]);
+            } else {
+                const int ksi = (i - PV_STEPS) >> 1, t = (i - PV_STEPS) & 1;
+                s_acc[t] = mfma_32x32x16(a, qf[ksi], s_acc[t]);
+            }
+            if (i + kDepth < last) ring[(i - first) % kDepth] = fetch(i + kDepth);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (int it = 0; it <= n_tiles; ++it) {
+        const int kt = kt0 + it * BN;
+        // ---- staging ----
+        if (it < n_tiles) {
+            if (v_role) {
+                store_v(it & 1);
+                if (it + 1 < n_tiles) load_v(kt + BN);
+            }
+            if (k_role && it + 1 < n_tiles) {
+                store_k((it + 1) & 1);
+                if (it + 2 < n_tiles) {
+                    load_k(kt + 2 * BN);
+                    if (it + 3 < n_tiles) load_kpos(kt + 3 * BN);
                 }
             }
+        }
+        // ---- MFMA phase ----
+        const bool wave_active = it < n_tiles && (kt < wmax) && (kt + BN > wmin);
+        {
+            const char* vt = reinterpret_cast<const char*>(v_lds[(it - 1) & 1]) + v_lane;
+            const uint16_t* ks = k_lane + (it & 1) * (BN * KSTR);
+            if (pending && wave_active) mfma_phase(std::integral_constant<int, 3>{}, vt, ks);
+            else if (pending) mfma_phase(std::integral_constant<int, 1>{}, vt, ks);
+            else if (wave_active) mfma_phase(std::integral_constant<int, 2>{}, vt, ks);
+        }
+        if (it == n_tiles) break;
+        __syncthreads();
 
+        // ---- VALU phase ----
+        pending = wave_active;
+        if (wave_active) {
             // tiles that cross an interval boundary of some lane get the compare; the others skip it
             if (__any((kt < klo) || (kt + BN > khi))) {
                 int rel0 = kt + 4 * g - klo;
@@ -246,33 +325,20 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
             const float m_use = (m_i == -INFINITY) ? 0.f : m_i;
             float rs0 = 0.f, rs1 = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float e0 = fast_exp2(s_acc[0][r] * c2 - m_use);
-                const float e1 = fast_exp2(s_acc[1][r] * c2 - m_use);
-                s_acc[0][r] = e0;
-                s_acc[1][r] = e1;
-                rs0 += e0;
-                rs1 += e1;
-            }
-            l_i += rs0 + rs1;
-
-#pragma unroll
             for (int m = 0; m < 4; ++m) {
                 const int t = m >> 1, r0 = 8 * (m & 1);
-                bf16x8_t pf;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s_acc[t][r0 + e];
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const bf16x8_t a = tr_operand(vt, v_lane, VSTR * 2, m, dt);
-                    o_acc[dt] = mfma_32x32x16(a, pf, o_acc[dt]);
+                for (int e = 0; e < 8; ++e) {
+                    const float ev = fast_exp2(s_acc[t][r0 + e] * c2 - m_use);
+                    if (e & 1) rs1 += ev; else rs0 += ev;
+                    pf[m][e] = (__bf16)ev;
                 }
             }
+            l_i += rs0 + rs1;
         }
-
-        if (it + 1 < n_tiles) store_tile(buf ^ 1);
         __syncthreads();
     }
+    if (grp == 0) __syncthreads();
 
     // ---- epilogue ------------------------------------------------------------------------------
     const float l_tot = l_i + __shfl_xor(l_i, 32, 64);
