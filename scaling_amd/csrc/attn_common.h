@@ -149,6 +149,118 @@ template <int D> struct TokTile {
     }
 };
 
+// ---- token-major LDS tile filled by direct global -> LDS loads ------------------------------------------
+// 64 tokens, unpadded rows of UPR 16-byte units (head_dim 96 uses rows of 16 units, 12 of them live).
+// A direct load instruction writes 64 x 16 bytes to consecutive LDS addresses (lane i -> base + 16 i), so
+// padding is impossible; instead the unit index of row r is XORed with f(r), chosen so that
+//   row operand   (lane = token, 16 bytes per k-step): 16 consecutive rows at one k-step hit 16 different
+//                 16-byte bank groups,
+//   transposed    (ds_read_b64_tr_b16; lane = feature, k-slots = tokens): the 4 rows x 2 x 32 bytes touched by
+//                 32 lanes cover 256 distinct bytes (mod 256),
+// and a loader lane simply fetches the logical unit (physical ^ f(row)) of its row from global memory.
+// Rows of an operand start at a multiple of 16, so f is fixed per lane.
+template <int D> struct LdsTile {
+    static_assert(D == 32 || D == 64 || D == 96 || D == 128, "head_dim");
+    static constexpr int UPR = (D == 96) ? 16 : D / 8;   // physical units per row
+    static constexpr int RB = 16 * UPR;                  // bytes per row
+    static constexpr int kInstrs = UPR;                  // direct-load instructions per 64-token tile
+    static constexpr int kBytes = 64 * RB;
+
+    static __device__ __forceinline__ int f(int r) {
+        if constexpr (UPR == 16) return ((r & 3) << 2) | ((r >> 2) & 3);
+        else if constexpr (UPR == 8) return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
+        else return (r >> 2) & 3;
+    }
+    // byte offset of logical 16-byte unit c of row r (register-staged stores)
+    static __device__ __forceinline__ int unit_offset(int r, int c) { return r * RB + ((c ^ f(r)) << 4); }
+    // direct-load instruction n of a tile, lane -> source row and logical unit (unit >= D/8: nothing to fetch)
+    static __device__ __forceinline__ void dma_src(int n, int lane, int& row, int& unit) {
+        const int u = 64 * n + lane;
+        row = u / UPR;
+        unit = (u % UPR) ^ f(row);
+    }
+    // row operand of lane (row, g): k-step ks is at (row_base ^ (ks << 5))
+    static __device__ __forceinline__ int row_base(int row, int g) { return row * RB + ((g ^ f(row)) << 4); }
+    // transposed operand: 16-token chunk m (chunk order), feature tile dt:
+    //   tr_pair(tile + (h0 ^ (dt << 6)) + 16*m*RB, tile + (h1 ^ (dt << 6)) + 16*m*RB)
+    static __device__ __forceinline__ void tr_bases(int lane, int& h0, int& h1) {
+        const int g = lane >> 5, i = lane & 15, blk = (lane >> 4) & 1;
+        const int j = i >> 2, e = (i >> 1) & 1, hb = i & 1;
+        const int r0 = 4 * g + j, r1 = 8 + 4 * g + j;
+        h0 = r0 * RB + (((2 * blk + e) ^ f(r0)) << 4) + 8 * hb;
+        h1 = r1 * RB + (((2 * blk + e) ^ f(r1)) << 4) + 8 * hb;
+    }
+};
+
+// Direct global -> LDS loads of 64-token tiles by one wavefront: instructions [n0, n0 + COUNT) of each tile.
+// The per-lane byte offsets inside a tile are fixed for the kernel, so a tile costs COUNT instructions with
+// a scalar base address and no vector arithmetic; only a tile that runs past the last token recomputes its
+// offsets (rows past the end repeat the last token).
+// Issued through inline assembly on purpose: the compiler would otherwise wait for every outstanding
+// direct load (vmcnt(0)) before each barrier and LDS read, which serialises the ring; completion is
+// tracked by the explicit wait_vmcnt below instead.
+template <int D, int COUNT> struct DmaPlan {
+    using T = LdsTile<D>;
+    int row[COUNT];          // source row of this lane
+    int unit_off[COUNT];     // byte offset of its 16-byte unit inside the row
+    uint32_t off[COUNT];     // byte offset from the first token of a full tile
+    int n0;
+
+    __device__ __forceinline__ void init(int first_instr, int lane, int64_t tok_stride) {
+        n0 = first_instr;
+#pragma unroll
+        for (int j = 0; j < COUNT; ++j) {
+            int unit;
+            T::dma_src(n0 + j, lane, row[j], unit);
+            if (D == 96 && unit >= D / 8) unit = 0;      // dead physical units of the padded row
+            unit_off[j] = 16 * unit;
+            off[j] = (uint32_t)(row[j] * (int)tok_stride * 2 + unit_off[j]);
+        }
+    }
+    __device__ __forceinline__ static void issue_one(uint32_t voff, const void* sbase, char* dst_lds) {
+        const uint32_t dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)dst_lds;
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :: "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(dst)) : "memory", "m0");
+    }
+    // Instruction j of the tile whose first token is tok0.  tile: wave-uniform LDS address of the stage;
+    // base + tok0 * tok_stride must be wave-uniform too.
+    __device__ __forceinline__ void issue(int j, const __bf16* base, int64_t tok_stride, int tok0, int last_tok, char* tile) const {
+        const __bf16* tile_base = base + (int64_t)tok0 * tok_stride;
+        if (tok0 + 63 <= last_tok) {
+            issue_one(off[j], tile_base, tile + 1024 * (n0 + j));
+        } else {
+            const int r = min(row[j], last_tok - tok0);
+            issue_one((uint32_t)(r * (int)tok_stride * 2 + unit_off[j]), tile_base, tile + 1024 * (n0 + j));
+        }
+    }
+};
+
+// waits until at most n (wave-uniform, run-time) vector memory loads are outstanding; large n waits for less
+// than asked only in the sense of waiting for everything older than the newest 24
+template <int N> __device__ __forceinline__ void wait_vmcnt();
+__device__ __forceinline__ void wait_vmcnt_dyn(int n) {
+    switch (n) {
+        case 0: wait_vmcnt<0>(); break;
+        case 1: wait_vmcnt<1>(); break;
+        case 2: wait_vmcnt<2>(); break;
+        case 3: wait_vmcnt<3>(); break;
+        case 4: wait_vmcnt<4>(); break;
+        case 5: wait_vmcnt<5>(); break;
+        case 6: wait_vmcnt<6>(); break;
+        case 7: wait_vmcnt<7>(); break;
+        case 8: wait_vmcnt<8>(); break;
+        case 9: case 10: case 11: wait_vmcnt<9>(); break;
+        case 12: case 13: case 14: case 15: wait_vmcnt<12>(); break;
+        default: if (n >= 16) wait_vmcnt<16>(); else wait_vmcnt<0>(); break;
+    }
+}
+
+// waits until at most N of this wavefront's vector memory loads are outstanding (N compile-time)
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
 // 4 tokens x 8 features held as 4 row vectors -> for feature dd the 4 token values as one 8-byte group
 __device__ __forceinline__ uint2 transpose_quad(const uint4 (&raw)[4], int dd) {
     const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&raw[0]);

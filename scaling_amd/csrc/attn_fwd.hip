@@ -3,7 +3,8 @@
 // Workgroup = NW wavefronts (4 or 8); every wavefront owns 32 consecutive query tokens of one head.
 // With 8 wavefronts, wavefronts w and w + 4 share a SIMD and run half a tile out of phase (enforced by
 // the barriers), so one issues MFMAs while the other runs its softmax on the VALU.
-// Keys/values stream through LDS in tiles of 64 tokens (double buffered).
+// Keys/values stream through LDS in tiles of 64 tokens, loaded global -> LDS directly (no staging
+// registers) two tile-steps ahead into a ring of three swizzled stages.
 // Per tile:
 //     S^T = K * Q^T            A = K tile rows from LDS, B = Q fragment held in registers
 //     online softmax           each lane owns ONE query (C column): the row max / sum are in-lane
@@ -26,20 +27,24 @@ constexpr float kRescaleGap = 8.0f;  // log2 units by which a row max may lag be
 template <int D, int NW, bool ROT>
 __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p) {
     constexpr int BM = 32 * NW;
-    constexpr int KSTR = D + 8;           // padded K row (elements): conflict-free 128-bit row reads
     constexpr int KS = D / 16;            // contraction steps of Q K^T
     constexpr int DT = D / 32;            // 32-row tiles of O^T
-    constexpr int KV_VECS = D / 32;       // 128-bit K (or V) vectors per loader thread and tile
-    constexpr int VSTR = D + 32;          // padded V row (elements): stride = 64 (mod 256) bytes for D = 64 / 128
+    constexpr int NS = 4;                 // LDS stages per operand
+    using Tile = LdsTile<D>;
+    constexpr int RB = Tile::RB;
+    constexpr int TILE = Tile::kBytes;
+    constexpr int IPW = Tile::kInstrs / 4;   // direct-load instructions per loader wavefront and tile
+    constexpr int KV_VECS = D / 32;       // 128-bit vectors per loader thread and tile (register-staged K, fused rotary)
     static_assert(D % 32 == 0 && D <= 128, "head_dim must be 32, 64, 96 or 128");
     static_assert(NW == 4 || NW == 8, "4 or 8 wavefronts");
 
-    __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KSTR];
-    __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][BN * VSTR];
+    __shared__ __attribute__((aligned(1024))) char k_lds[NS * TILE];
+    __shared__ __attribute__((aligned(1024))) char v_lds[NS * TILE];
     __shared__ int range_lds[2 * NW];
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: role and phase branches stay uniform
+    const int lane = tid & 63, l32 = lane & 31, g = lane >> 5;
 
     // ---- work item ---------------------------------------------------------------------------
     const int nqb = (p.total_q + BM - 1) / BM;
@@ -91,8 +96,9 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
 #pragma unroll
     for (int w = 0; w < NW; ++w) { bmin = min(bmin, range_lds[w]); bmax = max(bmax, range_lds[NW + w]); }
     if (bmax <= bmin) { bmin = 0; bmax = 0; }
-    const int kt0 = bmin & ~(BN - 1);
-    const int n_tiles = (bmax - kt0 + BN - 1) / BN;
+    // the same in every lane; made scalar so that loop control and tile addresses stay on the scalar unit
+    const int kt0 = __builtin_amdgcn_readfirstlane(bmin & ~(BN - 1));
+    const int n_tiles = __builtin_amdgcn_readfirstlane((bmax - kt0 + BN - 1) / BN);
 
     // ---- accumulators ----------------------------------------------------------------------
     f32x16_t o_acc[DT];
@@ -103,11 +109,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     float m_i = -INFINITY, l_i = 0.f;
 
     // ---- tile loaders: with 8 wavefronts the first four stage V, the last four stage K ----------
-    const bool v_role = (NW == 4) || (tid < 256);
-    const bool k_role = (NW == 4) || (tid >= 256);
+    // V (and K unless the rotary embedding is fused) goes global -> LDS directly, two tile-steps ahead of
+    // its use; with fused rotary K passes through registers to be rotated.
+    const bool v_role = (NW == 4) || (wave < 4);
+    const bool k_role = (NW == 4) || (wave >= 4);
+    const int lw = wave & 3;                                         // loader index within the role
     const int ltid = (NW == 4) ? tid : (tid & 255);
-    uint4 kraw[KV_VECS];
-    uint4 vraw[KV_VECS];
+    uint4 kraw[ROT ? KV_VECS : 1];
     uint4 craw[ROT ? KV_VECS / 2 : 1], sraw[ROT ? KV_VECS / 2 : 1];  // rotary table rows of the K tile
     int64_t kpos[ROT ? KV_VECS / 2 : 1];                             // their positions, fetched a tile ahead
     const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
@@ -124,15 +132,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         }
     };
     auto load_k = [&](int kt) {
-        if constexpr (!ROT) {
-#pragma unroll
-            for (int j = 0; j < KV_VECS; ++j) {
-                const int idx = ltid + 256 * j;
-                const int row = idx / (D / 8), c = idx % (D / 8);
-                const int tok = min(kt + row, last_k);
-                kraw[j] = ld128(kbase + (int64_t)tok * p.k_st + 8 * c);
-            }
-        } else {
+        if constexpr (ROT) {
 #pragma unroll
             for (int j = 0; j < KV_VECS / 2; ++j) {
                 const int idx = ltid + 256 * j;
@@ -148,73 +148,82 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
             }
         }
     };
-    auto store_k = [&](int buf) {
-        uint16_t* ks = k_lds[buf];
-        if constexpr (!ROT) {
-#pragma unroll
-            for (int j = 0; j < KV_VECS; ++j) {
-                const int idx = ltid + 256 * j;
-                const int row = idx / (D / 8), c = idx % (D / 8);
-                st128(ks + row * KSTR + 8 * c, kraw[j]);
-            }
-        } else {
+    auto store_k = [&](int stage) {
+        if constexpr (ROT) {
+            char* ks = k_lds + stage * TILE;
 #pragma unroll
             for (int j = 0; j < KV_VECS / 2; ++j) {
                 const int idx = ltid + 256 * j;
                 const int row = idx / (D / 16), c = idx % (D / 16);
                 rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);
-                st128(ks + row * KSTR + 8 * c, kraw[2 * j]);
-                st128(ks + row * KSTR + 8 * c + D / 2, kraw[2 * j + 1]);
+                st128(ks + Tile::unit_offset(row, c), kraw[2 * j]);
+                st128(ks + Tile::unit_offset(row, c + D / 16), kraw[2 * j + 1]);
             }
         }
     };
-    auto load_v = [&](int kt) {
-#pragma unroll
-        for (int j = 0; j < KV_VECS; ++j) {
-            const int idx = ltid + 256 * j;
-            const int row = idx / (D / 8), c = idx % (D / 8);
-            const int tok = min(kt + row, last_k);
-            vraw[j] = ld128(vbase + (int64_t)tok * p.v_st + 8 * c);
-        }
-    };
-    auto store_v = [&](int buf) {
-        uint16_t* vs = v_lds[buf];
-#pragma unroll
-        for (int j = 0; j < KV_VECS; ++j) {
-            const int idx = ltid + 256 * j;
-            const int row = idx / (D / 8), c = idx % (D / 8);
-            st128(vs + row * VSTR + 8 * c, vraw[j]);
-        }
-    };
+    DmaPlan<D, IPW> k_plan, v_plan;
+    k_plan.init(lw * IPW, lane, p.k_st);
+    v_plan.init(lw * IPW, lane, p.v_st);
+    // one direct-load instruction of K / V tile `tile_idx` (j-th of this wavefront's share)
+    auto dma_k = [&](int tile_idx, int j) { k_plan.issue(j, kbase, p.k_st, kt0 + tile_idx * BN, last_k, k_lds + (tile_idx % NS) * TILE); };
+    auto dma_v = [&](int tile_idx, int j) { v_plan.issue(j, vbase, p.v_st, kt0 + tile_idx * BN, last_k, v_lds + (tile_idx % NS) * TILE); };
 
     // ---- main loop ---------------------------------------------------------------------------
     // Each wavefront alternates an MFMA phase (O^T += V^T P^T of the previous tile, then S^T of the
     // current one) and a VALU phase (softmax of the current tile), with a workgroup barrier after each.
     // The second group of four wavefronts runs one phase behind the first, so on every SIMD one
     // wavefront is in its MFMA phase while the other is in its VALU phase.
-    //   K tile n is read in phases 2n (group 0) and 2n+1 (group 1): it is stored during phase 2n-1;
-    //   V tile n is read in phases 2n+2 and 2n+3: it is stored during phase 2n.
+    //   K tile n is read in phases 2n (group 0) and 2n+1 (group 1); V tile n in phases 2n+2 and 2n+3.
+    //   At the end of its VALU phase i the V loader group (0) issues V tile i+2 and the K loader group (1)
+    //   issues K tile i+3, each into the stage (of four) whose last reader finished two phases earlier; a
+    //   loader waits for a tile right before the barrier that precedes its first read.
     // wave-uniform by construction: the extra barriers below must sit behind scalar branches
-    const int grp = (NW == 8) ? __builtin_amdgcn_readfirstlane(wave >> 2) : 0;
+    const int grp = (NW == 8) ? wave >> 2 : 0;
+    auto dma_k_tile = [&](int tile_idx) {
+        if (tile_idx < n_tiles) {
+#pragma unroll
+            for (int j = 0; j < IPW; ++j) dma_k(tile_idx, j);
+        }
+    };
+    auto dma_v_tile = [&](int tile_idx) {
+        if (tile_idx < n_tiles) {
+#pragma unroll
+            for (int j = 0; j < IPW; ++j) dma_v(tile_idx, j);
+        }
+    };
+    // number of direct-load instructions a loader issues for tiles [a, b)
+    auto n_issued = [&](int a, int b) { return IPW * max(0, min(b, n_tiles) - a); };
     if (n_tiles > 0) {
         if (k_role) {
-            load_kpos(kt0);
-            load_k(kt0);
-            if (n_tiles > 1) load_kpos(kt0 + BN);
-            store_k(0);
-            if (n_tiles > 1) {
-                load_k(kt0 + BN);
-                if (n_tiles > 2) load_kpos(kt0 + 2 * BN);
+            if constexpr (ROT) {
+                load_kpos(kt0);
+                load_k(kt0);
+                if (n_tiles > 1) load_kpos(kt0 + BN);
+                store_k(0);
+                if (n_tiles > 1) {
+                    load_k(kt0 + BN);
+                    if (n_tiles > 2) load_kpos(kt0 + 2 * BN);
+                }
+            } else {
+                dma_k_tile(0);
+                dma_k_tile(1);
+                dma_k_tile(2);
             }
         }
-        if (v_role) load_v(kt0);
+        if (v_role) {
+            dma_v_tile(0);
+            dma_v_tile(1);
+        }
+        // K tile 0 must have landed; whatever was issued after it may still be in flight
+        if (!ROT && k_role) wait_vmcnt_dyn(n_issued(1, 3) + (NW == 4 ? n_issued(0, 2) : 0));
     }
     __syncthreads();
     if (grp == 1) __syncthreads();
 
     const float c2 = p.scale_log2;
-    const int v_lane = tr_lane_base(lane, VSTR * 2);
-    const uint16_t* k_lane = k_lds[0] + l32 * KSTR + 8 * g;
+    int v_h0, v_h1;
+    Tile::tr_bases(lane, v_h0, v_h1);
+    const int k_row = Tile::row_base(l32, g);
     f32x16_t s_acc[2];
     bf16x8_t pf[4];
     bool pending = false;                 // pf holds the probabilities of the previous tile
@@ -224,18 +233,18 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     // filled kDepth steps ahead, so a wavefront that has its SIMD's matrix core to itself keeps it fed
     // in spite of the LDS latency; sched_barrier pins that order.
     constexpr int PV_STEPS = 4 * DT, S_STEPS = 2 * KS;
-    constexpr int kDepth = 6;
-    auto mfma_phase = [&](auto mode, const char* vt, const uint16_t* ks) {
+    constexpr int kDepth = 3;
+    auto mfma_phase = [&](auto mode, const char* vt, const char* ks) {
         constexpr bool kPV = (decltype(mode)::value & 1) != 0, kS = (decltype(mode)::value & 2) != 0;
         constexpr int first = kPV ? 0 : PV_STEPS, last = kS ? PV_STEPS + S_STEPS : PV_STEPS;
         bf16x8_t ring[kDepth];
         auto fetch = [&](int i) -> bf16x8_t {
             if (i < PV_STEPS) {
                 const int m = i / DT, dt = i % DT;
-                return tr_pair(vt + (16 * m) * (VSTR * 2) + 64 * dt, vt + (16 * m + 8) * (VSTR * 2) + 64 * dt);
+                return tr_pair(vt + (v_h0 ^ (dt << 6)) + 16 * m * RB, vt + (v_h1 ^ (dt << 6)) + 16 * m * RB);
             }
             const int ksi = (i - PV_STEPS) >> 1, t = (i - PV_STEPS) & 1;
-            return *reinterpret_cast<const bf16x8_t*>(ks + 32 * t * KSTR + 16 * ksi);
+            return *reinterpret_cast<const bf16x8_t*>(ks + (k_row ^ (ksi << 5)) + 32 * t * RB);
         };
         if constexpr (kS) {
 #pragma unroll
@@ -262,14 +271,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     };
     for (int it = 0; it <= n_tiles; ++it) {
         const int kt = kt0 + it * BN;
-        // ---- staging ----
-        if (it < n_tiles) {
-            if (v_role) {
-                store_v(it & 1);
-                if (it + 1 < n_tiles) load_v(kt + BN);
-            }
+        // ---- staging (register path of the fused rotary only) ----
+        if constexpr (ROT) {
             if (k_role && it + 1 < n_tiles) {
-                store_k((it + 1) & 1);
+                store_k((it + 1) % NS);
                 if (it + 2 < n_tiles) {
                     load_k(kt + 2 * BN);
                     if (it + 3 < n_tiles) load_kpos(kt + 3 * BN);
@@ -279,13 +284,16 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         // ---- MFMA phase ----
         const bool wave_active = it < n_tiles && (kt < wmax) && (kt + BN > wmin);
         {
-            const char* vt = reinterpret_cast<const char*>(v_lds[(it - 1) & 1]) + v_lane;
-            const uint16_t* ks = k_lane + (it & 1) * (BN * KSTR);
+            const char* vt = v_lds + ((it + NS - 1) % NS) * TILE;
+            const char* ks = k_lds + (it % NS) * TILE;
             if (pending && wave_active) mfma_phase(std::integral_constant<int, 3>{}, vt, ks);
             else if (pending) mfma_phase(std::integral_constant<int, 1>{}, vt, ks);
             else if (wave_active) mfma_phase(std::integral_constant<int, 2>{}, vt, ks);
         }
         if (it == n_tiles) break;
+        // K tile it+1 is read after this barrier (by group 0): the K loaders of group 1 make sure it
+        // has landed; only K tile it+2 was issued after it
+        if (NW == 8 && !ROT && k_role) wait_vmcnt_dyn(n_issued(it + 2, it + 3));
         __syncthreads();
 
         // ---- VALU phase ----
@@ -335,6 +343,17 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 }
             }
             l_i += rs0 + rs1;
+        }
+        // Direct loads are issued here, at the end of the shorter phase: the texture path takes a few
+        // hundred cycles to accept a tile's worth of them, and this wavefront would otherwise idle at
+        // the barrier while its SIMD neighbour finishes the MFMA phase.
+        if (v_role) dma_v_tile(it + 2);
+        if (!ROT && k_role) dma_k_tile(it + 3);
+        // V tile it (and with one group K tile it+1) is read after this barrier
+        if (NW == 8) {
+            if (v_role) wait_vmcnt_dyn(n_issued(it + 1, it + 3));
+        } else {
+            wait_vmcnt_dyn(n_issued(it + 1, it + 3) + (ROT ? 0 : n_issued(it + 2, it + 4)));
         }
         __syncthreads();
     }
