@@ -53,32 +53,30 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_delta_kernel(const AttnPara
 // tiles are double buffered (one barrier per iteration).
 template <int D>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
-    constexpr int NT = 512;
     constexpr int BNK = 128;              // keys per workgroup
     constexpr int BQ = 64;                // queries per tile
-    constexpr int STR = D + 8;            // K / V rows (elements): row operands only
     constexpr int KS = D / 16;
     constexpr int DT = D / 32;
-    constexpr int VECS = (BQ * (D / 8)) / 256;   // 128-bit vectors per loader thread and tile
-    using Tile = TokTile<D>;
-    constexpr int TSTR = Tile::kStride;
-    constexpr int KV_BYTES = BNK * STR * 2;
-    constexpr int TILE_BYTES = BQ * TSTR;
-    constexpr int STAGE_BYTES = 2 * KV_BYTES + 4 * TILE_BYTES;
+    using Tile = LdsTile<D>;
+    constexpr int RB = Tile::RB;
+    constexpr int TILE = Tile::kBytes;    // one 64-token tile
+    constexpr int IPW = Tile::kInstrs / 4;   // direct-load instructions per loader wavefront and 64-token tile
+    constexpr int STAGE_BYTES = 4 * TILE + 4 * TILE;  // K, V (two tiles each) + Q, dO (two stages each)
     constexpr int RED_BYTES = 4 * 16 * DT * 64 * 4;   // one accumulator set of four wavefronts
     constexpr int SMEM_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
 
-    __shared__ __attribute__((aligned(16))) char smem[SMEM_BYTES];
+    __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
     __shared__ __attribute__((aligned(16))) float lse_lds[2][BQ];
     __shared__ __attribute__((aligned(16))) float delta_lds[2][BQ];
     __shared__ int range_lds[16];
-    uint16_t* k_rm = reinterpret_cast<uint16_t*>(smem);
-    uint16_t* v_rm = reinterpret_cast<uint16_t*>(smem + KV_BYTES);
-    char* q_t = smem + 2 * KV_BYTES;                   // [2][BQ rows]
-    char* do_t = q_t + 2 * TILE_BYTES;                 // [2][BQ rows]
+    char* k_t = smem;                     // [2 tiles of 64 keys]
+    char* v_t = smem + 2 * TILE;
+    char* q_t = smem + 4 * TILE;          // [2 stages]
+    char* do_t = smem + 6 * TILE;         // [2 stages]
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int kgp = wave & 3, sub = wave >> 2;
 
     const int nkb = (p.total_k + BNK - 1) / BNK;
@@ -97,26 +95,27 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     }
     if (lane == 0) { range_lds[wave] = wmin; range_lds[8 + wave] = wmax; }
 
-    // stage the K / V rows of this key block (row-major, padded rows)
+    // K / V rows of this key block: loaded once, global -> LDS directly; wavefronts 0-3 fetch K, 4-7 fetch V
+    const bool q_role = wave < 4;         // later: wavefronts 0-3 stage Q, 4-7 stage dO
+    const int lw = wave & 3;
     {
-        const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
-        const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
+        DmaPlan<D, IPW> plan;
+        plan.init(lw * IPW, lane, q_role ? p.k_st : p.v_st);
+        const __bf16* base = q_role ? p.k + (int64_t)kvh * p.k_sh : p.v + (int64_t)kvh * p.v_sh;
+        const int64_t st = q_role ? p.k_st : p.v_st;
+        char* dst = q_role ? k_t : v_t;
 #pragma unroll
-        for (int j = 0; j < (BNK * (D / 8)) / NT; ++j) {
-            const int idx = tid + NT * j;
-            const int row = idx / (D / 8), c = idx % (D / 8);
-            const int tok = min(kb * BNK + row, p.total_k - 1);
-            st128(k_rm + row * STR + 8 * c, ld128(kbase + (int64_t)tok * p.k_st + 8 * c));
-            st128(v_rm + row * STR + 8 * c, ld128(vbase + (int64_t)tok * p.v_st + 8 * c));
-        }
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int j = 0; j < IPW; ++j) plan.issue(j, base, st, kb * BNK + 64 * half, p.total_k - 1, dst + half * TILE);
     }
-    __syncthreads();
+    __syncthreads();                      // publishes range_lds (the loads are waited for below)
     int bmin = 0x7fffffff, bmax = 0;
 #pragma unroll
     for (int w = 0; w < 8; ++w) { bmin = min(bmin, range_lds[w]); bmax = max(bmax, range_lds[8 + w]); }
     if (bmax <= bmin) { bmin = 0; bmax = 0; }
-    const int qt0 = bmin & ~(BQ - 1);
-    const int n_tiles = (bmax - qt0 + BQ - 1) / BQ;
+    const int qt0 = __builtin_amdgcn_readfirstlane(bmin & ~(BQ - 1));
+    const int n_tiles = __builtin_amdgcn_readfirstlane((bmax - qt0 + BQ - 1) / BQ);
 
     f32x16_t dk_acc[DT], dv_acc[DT];
 #pragma unroll
@@ -124,86 +123,76 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk_acc[dt][r] = 0.f; dv_acc[dt][r] = 0.f; }
 
-    const bool q_role = tid < 256;
-    const int ltid = tid & 255;
-    uint4 raw[VECS];
-    float stat = 0.f;
-
     // Query tiles are visited from the last one downwards: under a causal mask every key block of a
     // document needs the document's last queries, so the workgroups that share an XCD start on the same
     // tile and keep streaming the same Q / dO rows through that XCD's L2.
     const int total_iters = n_tiles * p.n_rep;
-    // Role-dependent sources are selected once, as values: a per-iteration select between kernel
-    // arguments turns into a load of the argument through a vector address, and a wait on it.
+    const int last_q = p.total_q - 1;
     const __bf16* src_base = q_role ? p.q : p.d_o;
     const int64_t src_head_stride = q_role ? p.q_sh : p.o_sh;
     const int64_t src_tok_stride = q_role ? p.q_st : p.o_st;
-    const float* stat_base = (tid < BQ) ? p.lse : p.delta;
-    const float stat_scale = (tid < BQ) ? 1.4426950408889634f : 1.0f;  // log-sum-exp goes to the exp2 domain
     char* dst_tile = q_role ? q_t : do_t;
-    const int last_q = p.total_q - 1;
-    auto load_tile = [&](int iter) {
-        const int rep = iter / n_tiles, qt = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ;
-        const int head = kvh * p.n_rep + rep;
-        const __bf16* base = src_base + (int64_t)head * src_head_stride;
+    DmaPlan<D, IPW> plan;
+    plan.init(lw * IPW, lane, src_tok_stride);
+    // log-sum-exp (to the exp2 domain) and delta rows of a tile pass through one register of threads 0..127
+    const float* stat_base = (tid < BQ) ? p.lse : p.delta;
+    const float stat_scale = (tid < BQ) ? 1.4426950408889634f : 1.0f;
+    float stat = 0.f;
+    auto tile_of = [&](int iter, int& head, int& qt) {
+        const int rep = iter / n_tiles;
+        head = kvh * p.n_rep + rep;
+        qt = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ;
+    };
+    auto issue_tile = [&](int iter) {     // Q / dO tile of iteration `iter` -> stage iter & 1
+        int head, qt;
+        tile_of(iter, head, qt);
 #pragma unroll
-        for (int j = 0; j < VECS; ++j) {
-            const int idx = ltid + 256 * j;
-            const int row = idx / (D / 8), c = idx % (D / 8);
-            const int tok = min(qt + row, last_q);
-            raw[j] = ld128(base + (int64_t)tok * src_tok_stride + 8 * c);
-        }
+        for (int j = 0; j < IPW; ++j)
+            plan.issue(j, src_base + (int64_t)head * src_head_stride, src_tok_stride, qt, last_q, dst_tile + (iter & 1) * TILE);
         if (tid < 2 * BQ) {
             const int tok = min(qt + (tid & (BQ - 1)), last_q);
             stat = stat_base[(int64_t)head * p.total_q + tok];
         }
     };
-    auto store_tile = [&](int buf) {
-        char* dst = dst_tile + buf * TILE_BYTES;
-#pragma unroll
-        for (int j = 0; j < VECS; ++j) {
-            const int idx = ltid + 256 * j;
-            const int row = idx / (D / 8), c = idx % (D / 8);
-            st128(dst + Tile::unit_offset(row, c), raw[j]);
-        }
-        if (tid < BQ) lse_lds[buf][tid] = stat * stat_scale;
-        else if (tid < 2 * BQ) delta_lds[buf][tid - BQ] = stat * stat_scale;
+    auto store_stat = [&](int iter) {
+        if (tid < BQ) lse_lds[iter & 1][tid] = stat * stat_scale;
+        else if (tid < 2 * BQ) delta_lds[iter & 1][tid - BQ] = stat * stat_scale;
     };
 
     if (total_iters > 0) {
-        load_tile(0);
-        store_tile(0);
+        issue_tile(0);
+        store_stat(0);
     }
+    wait_vmcnt<0>();
     __syncthreads();
 
-    int row_even, row_odd, tr_h0, tr_h1;
-    Tile::row_bases(32 * sub + l32, g, row_even, row_odd);
+    int tr_h0, tr_h1;
     Tile::tr_bases(lane, tr_h0, tr_h1);
-    tr_h0 += 32 * sub * TSTR;
-    tr_h1 += 32 * sub * TSTR;
-    const uint16_t* b_k = k_rm + (32 * kgp + l32) * STR + 8 * g;
-    const uint16_t* b_v = v_rm + (32 * kgp + l32) * STR + 8 * g;
+    tr_h0 += 32 * sub * RB;
+    tr_h1 += 32 * sub * RB;
+    const int a_row = Tile::row_base(32 * sub + l32, g);                       // Q / dO rows of this wavefront's sub-tile
+    const int b_row = (kgp >> 1) * TILE + Tile::row_base(32 * (kgp & 1) + l32, g);   // its K / V rows
     const float c2 = p.scale_log2;
 
     for (int iter = 0; iter < total_iters; ++iter) {
         const int buf = iter & 1;
         const int qs = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ + 32 * sub;
-        if (iter + 1 < total_iters) load_tile(iter + 1);
+        if (iter + 1 < total_iters) issue_tile(iter + 1);
 
         if ((qs < wmax) && (qs + 32 > wmin)) {
-            const char* qt_ = q_t + buf * TILE_BYTES;
-            const char* dt_ = do_t + buf * TILE_BYTES;
+            const char* qt_ = q_t + buf * TILE;
+            const char* dt_ = do_t + buf * TILE;
             f32x16_t s_acc, dp_acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) { s_acc[r] = 0.f; dp_acc[r] = 0.f; }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const int ro = ((ks & 1) ? row_odd : row_even) + 32 * ks;
-                const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(qt_ + ro);
-                const bf16x8_t bk = *reinterpret_cast<const bf16x8_t*>(b_k + 16 * ks);
+                const int ao = a_row ^ (ks << 5), bo = b_row ^ (ks << 5);
+                const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(qt_ + ao);
+                const bf16x8_t bk = *reinterpret_cast<const bf16x8_t*>(k_t + bo);
                 s_acc = mfma_32x32x16(aq, bk, s_acc);
-                const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(dt_ + ro);
-                const bf16x8_t bv = *reinterpret_cast<const bf16x8_t*>(b_v + 16 * ks);
+                const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(dt_ + ao);
+                const bf16x8_t bv = *reinterpret_cast<const bf16x8_t*>(v_t + bo);
                 dp_acc = mfma_32x32x16(ad, bv, dp_acc);
             }
             // rows of the accumulators are queries qs + 8a + 4g + c, the column is this lane's key
@@ -235,15 +224,16 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             for (int m = 0; m < 2; ++m) {
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const int off = 16 * m * TSTR + 64 * dt;
-                    const bf16x8_t adt = tr_pair(dt_ + tr_h0 + off, dt_ + tr_h1 + off);
-                    const bf16x8_t aqt = tr_pair(qt_ + tr_h0 + off, qt_ + tr_h1 + off);
+                    const int o0 = (tr_h0 ^ (dt << 6)) + 16 * m * RB, o1 = (tr_h1 ^ (dt << 6)) + 16 * m * RB;
+                    const bf16x8_t adt = tr_pair(dt_ + o0, dt_ + o1);
+                    const bf16x8_t aqt = tr_pair(qt_ + o0, qt_ + o1);
                     dv_acc[dt] = mfma_32x32x16(adt, pf[m], dv_acc[dt]);
                     dk_acc[dt] = mfma_32x32x16(aqt, dsf[m], dk_acc[dt]);
                 }
             }
         }
-        if (iter + 1 < total_iters) store_tile(buf ^ 1);
+        if (iter + 1 < total_iters) store_stat(iter + 1);
+        wait_vmcnt<0>();                  // the next Q / dO tile has landed
         __syncthreads();
     }
 
@@ -295,19 +285,21 @@ template <int D>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p) {
     constexpr int BM = 256;
     constexpr int BN = 64;
-    constexpr int STR = D + 8;
     constexpr int KS = D / 16;
     constexpr int DT = D / 32;
-    constexpr int VECS = (BN * (D / 8)) / 256;   // 128-bit vectors per loader thread and tile
-    using Tile = TokTile<D>;
-    constexpr int TSTR = Tile::kStride;
+    constexpr int NS = 3;                 // LDS stages per operand
+    using Tile = LdsTile<D>;
+    constexpr int RB = Tile::RB;
+    constexpr int TILE = Tile::kBytes;
+    constexpr int IPW = Tile::kInstrs / 4;   // direct-load instructions per loader wavefront and tile
 
-    __shared__ __attribute__((aligned(16))) char k_t[2][BN * TSTR];        // row operand and transposed operand
-    __shared__ __attribute__((aligned(16))) uint16_t v_rm[2][BN * STR];    // row operand only
+    __shared__ __attribute__((aligned(1024))) char k_t[NS * TILE];   // row operand and transposed operand
+    __shared__ __attribute__((aligned(1024))) char v_t[NS * TILE];   // row operand
     __shared__ int range_lds[16];
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, l32 = lane & 31, g = lane >> 5;
 
     const int nqb = (p.total_q + BM - 1) / BM;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
@@ -342,7 +334,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     float delta = p.delta[(int64_t)head * p.total_q + tl];
     float lse2 = lse_nat * 1.4426950408889634f;
     // Consume the loaded registers here: otherwise their loads count as possibly outstanding at the
-    // loop entry and their uses inside the loop wait for the K / V prefetch issued just before.
+    // loop entry and their uses inside the loop wait for them again.
     asm volatile("" : "+v"(lse2), "+v"(delta));
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
@@ -352,8 +344,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
 #pragma unroll
     for (int w = 0; w < 8; ++w) { bmin = min(bmin, range_lds[w]); bmax = max(bmax, range_lds[8 + w]); }
     if (bmax <= bmin) { bmin = 0; bmax = 0; }
-    const int kt0 = bmin & ~(BN - 1);
-    const int n_tiles = (bmax - kt0 + BN - 1) / BN;
+    const int kt0 = __builtin_amdgcn_readfirstlane(bmin & ~(BN - 1));
+    const int n_tiles = __builtin_amdgcn_readfirstlane((bmax - kt0 + BN - 1) / BN);
 
     f32x16_t dq_acc[DT];
 #pragma unroll
@@ -361,51 +353,38 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq_acc[dt][r] = 0.f;
 
-    const bool k_role = tid < 256;
-    const int ltid = tid & 255;
-    uint4 raw[VECS];
-    // selected once, as values (see the dK / dV kernel)
+    // wavefronts 0-3 fetch K tiles, 4-7 fetch V tiles: global -> LDS directly, two tiles ahead, into the
+    // stage whose readers passed the previous barrier
+    const bool k_role = wave < 4;
+    const int lw = wave & 3;
     const __bf16* src_base = k_role ? p.k + (int64_t)kvh * p.k_sh : p.v + (int64_t)kvh * p.v_sh;
     const int64_t src_tok_stride = k_role ? p.k_st : p.v_st;
+    char* dst_ring = k_role ? k_t : v_t;
     const int last_k = p.total_k - 1;
-
-    auto load_tile = [&](int kt) {
+    DmaPlan<D, IPW> plan;
+    plan.init(lw * IPW, lane, src_tok_stride);
+    auto issue_tile = [&](int t) {
+        if (t < n_tiles) {
 #pragma unroll
-        for (int j = 0; j < VECS; ++j) {
-            const int idx = ltid + 256 * j;
-            const int row = idx / (D / 8), c = idx % (D / 8);
-            const int tok = min(kt + row, last_k);
-            raw[j] = ld128(src_base + (int64_t)tok * src_tok_stride + 8 * c);
+            for (int j = 0; j < IPW; ++j) plan.issue(j, src_base, src_tok_stride, kt0 + t * BN, last_k, dst_ring + (t % NS) * TILE);
         }
     };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int j = 0; j < VECS; ++j) {
-            const int idx = ltid + 256 * j;
-            const int row = idx / (D / 8), c = idx % (D / 8);
-            if (k_role) st128(k_t[buf] + Tile::unit_offset(row, c), raw[j]);
-            else st128(v_rm[buf] + row * STR + 8 * c, raw[j]);
-        }
-    };
-
-    if (n_tiles > 0) {
-        load_tile(kt0);
-        store_tile(0);
-    }
+    issue_tile(0);
+    issue_tile(1);
+    if (n_tiles > 1) wait_vmcnt<IPW>(); else wait_vmcnt<0>();
     __syncthreads();
 
     const float c2 = p.scale_log2;
-    int row_even, row_odd, tr_h0, tr_h1;
-    Tile::row_bases(l32, g, row_even, row_odd);
+    int tr_h0, tr_h1;
     Tile::tr_bases(lane, tr_h0, tr_h1);
+    const int a_row = Tile::row_base(l32, g);
     for (int it = 0; it < n_tiles; ++it) {
         const int kt = kt0 + it * BN;
-        const int buf = it & 1;
-        if (it + 1 < n_tiles) load_tile(kt + BN);
+        issue_tile(it + 2);
 
         if ((kt < wmax) && (kt + BN > wmin)) {
-            const char* kt_ = k_t[buf];
-            const uint16_t* a_v = v_rm[buf] + l32 * STR + 8 * g;
+            const char* kt_ = k_t + (it % NS) * TILE;
+            const char* vt_ = v_t + (it % NS) * TILE;
             f32x16_t s_acc[2], dp_acc[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
@@ -413,12 +392,12 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                 for (int r = 0; r < 16; ++r) { s_acc[t][r] = 0.f; dp_acc[t][r] = 0.f; }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const int ro = ((ks & 1) ? row_odd : row_even) + 32 * ks;
+                const int ao = a_row ^ (ks << 5);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(kt_ + ro + 32 * t * TSTR);
+                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(kt_ + ao + 32 * t * RB);
                     s_acc[t] = mfma_32x32x16(ak, qf[ks], s_acc[t]);
-                    const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(a_v + 32 * t * STR + 16 * ks);
+                    const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(vt_ + ao + 32 * t * RB);
                     dp_acc[t] = mfma_32x32x16(av, dof[ks], dp_acc[t]);
                 }
             }
@@ -445,13 +424,14 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                 }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    const int off = 16 * m * TSTR + 64 * dt;
-                    const bf16x8_t akt = tr_pair(kt_ + tr_h0 + off, kt_ + tr_h1 + off);
+                    const int o0 = (tr_h0 ^ (dt << 6)) + 16 * m * RB, o1 = (tr_h1 ^ (dt << 6)) + 16 * m * RB;
+                    const bf16x8_t akt = tr_pair(kt_ + o0, kt_ + o1);
                     dq_acc[dt] = mfma_32x32x16(akt, dsf, dq_acc[dt]);
                 }
             }
         }
-        if (it + 1 < n_tiles) store_tile(buf ^ 1);
+        // tile it+1 must have landed; tile it+2 (just issued) may still be in flight
+        if (it + 2 < n_tiles) wait_vmcnt<IPW>(); else wait_vmcnt<0>();
         __syncthreads();
     }
 

@@ -225,12 +225,12 @@ template <int D, int COUNT> struct DmaPlan {
     // Instruction j of the tile whose first token is tok0.  tile: wave-uniform LDS address of the stage;
     // base + tok0 * tok_stride must be wave-uniform too.
     __device__ __forceinline__ void issue(int j, const __bf16* base, int64_t tok_stride, int tok0, int last_tok, char* tile) const {
-        const __bf16* tile_base = base + (int64_t)tok0 * tok_stride;
         if (tok0 + 63 <= last_tok) {
-            issue_one(off[j], tile_base, tile + 1024 * (n0 + j));
+            issue_one(off[j], base + (int64_t)tok0 * tok_stride, tile + 1024 * (n0 + j));
         } else {
-            const int r = min(row[j], last_tok - tok0);
-            issue_one((uint32_t)(r * (int)tok_stride * 2 + unit_off[j]), tile_base, tile + 1024 * (n0 + j));
+            const int first = min(tok0, last_tok);            // the lane offset below must not be negative
+            const int r = min(row[j], last_tok - first);
+            issue_one((uint32_t)(r * (int)tok_stride * 2 + unit_off[j]), base + (int64_t)first * tok_stride, tile + 1024 * (n0 + j));
         }
     }
 };
