@@ -105,9 +105,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
         const int64_t st = q_role ? p.k_st : p.v_st;
         char* dst = q_role ? k_t : v_t;
 #pragma unroll
-        for (int half = 0; half < 2; ++half)
-#pragma unroll
-            for (int j = 0; j < IPW; ++j) plan.issue(j, base, st, kb * BNK + 64 * half, p.total_k - 1, dst + half * TILE);
+        for (int half = 0; half < 2; ++half) plan.issue(base, st, kb * BNK + 64 * half, p.total_k - 1, dst + half * TILE);
     }
     __syncthreads();                      // publishes range_lds (the loads are waited for below)
     int bmin = 0x7fffffff, bmax = 0;
@@ -146,9 +144,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     auto issue_tile = [&](int iter) {     // Q / dO tile of iteration `iter` -> stage iter & 1
         int head, qt;
         tile_of(iter, head, qt);
-#pragma unroll
-        for (int j = 0; j < IPW; ++j)
-            plan.issue(j, src_base + (int64_t)head * src_head_stride, src_tok_stride, qt, last_q, dst_tile + (iter & 1) * TILE);
+        plan.issue(src_base + (int64_t)head * src_head_stride, src_tok_stride, qt, last_q, dst_tile + (iter & 1) * TILE);
         if (tid < 2 * BQ) {
             const int tok = min(qt + (tid & (BQ - 1)), last_q);
             stat = stat_base[(int64_t)head * p.total_q + tok];
@@ -364,10 +360,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     DmaPlan<D, IPW> plan;
     plan.init(lw * IPW, lane, src_tok_stride);
     auto issue_tile = [&](int t) {
-        if (t < n_tiles) {
-#pragma unroll
-            for (int j = 0; j < IPW; ++j) plan.issue(j, src_base, src_tok_stride, kt0 + t * BN, last_k, dst_ring + (t % NS) * TILE);
-        }
+        if (t < n_tiles) plan.issue(src_base, src_tok_stride, kt0 + t * BN, last_k, dst_ring + (t % NS) * TILE);
     };
     issue_tile(0);
     issue_tile(1);

@@ -222,15 +222,22 @@ template <int D, int COUNT> struct DmaPlan {
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :: "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(dst)) : "memory", "m0");
     }
-    // Instruction j of the tile whose first token is tok0.  tile: wave-uniform LDS address of the stage;
-    // base + tok0 * tok_stride must be wave-uniform too.
-    __device__ __forceinline__ void issue(int j, const __bf16* base, int64_t tok_stride, int tok0, int last_tok, char* tile) const {
+    // All COUNT instructions of the tile whose first token is tok0, straight-line when the tile is full.
+    // tile: wave-uniform LDS address of the stage; base + tok0 * tok_stride must be wave-uniform too.
+    __device__ __forceinline__ void issue(const __bf16* base, int64_t tok_stride, int tok0, int last_tok, char* tile) const {
+        char* dst = tile + 1024 * n0;
         if (tok0 + 63 <= last_tok) {
-            issue_one(off[j], base + (int64_t)tok0 * tok_stride, tile + 1024 * (n0 + j));
+            const __bf16* tile_base = base + (int64_t)tok0 * tok_stride;
+#pragma unroll
+            for (int j = 0; j < COUNT; ++j) issue_one(off[j], tile_base, dst + 1024 * j);
         } else {
-            const int first = min(tok0, last_tok);            // the lane offset below must not be negative
-            const int r = min(row[j], last_tok - first);
-            issue_one((uint32_t)(r * (int)tok_stride * 2 + unit_off[j]), base + (int64_t)first * tok_stride, tile + 1024 * (n0 + j));
+            const int first = min(tok0, last_tok);            // the lane offsets below must not be negative
+            const __bf16* tile_base = base + (int64_t)first * tok_stride;
+#pragma unroll
+            for (int j = 0; j < COUNT; ++j) {
+                const int r = min(row[j], last_tok - first);
+                issue_one((uint32_t)(r * (int)tok_stride * 2 + unit_off[j]), tile_base, dst + 1024 * j);
+            }
         }
     }
 };

@@ -164,10 +164,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     DmaPlan<D, IPW> k_plan, v_plan;
     k_plan.init(lw * IPW, lane, p.k_st);
     v_plan.init(lw * IPW, lane, p.v_st);
-    // one direct-load instruction of K / V tile `tile_idx` (j-th of this wavefront's share)
-    auto dma_k = [&](int tile_idx, int j) { k_plan.issue(j, kbase, p.k_st, kt0 + tile_idx * BN, last_k, k_lds + (tile_idx % NS) * TILE); };
-    auto dma_v = [&](int tile_idx, int j) { v_plan.issue(j, vbase, p.v_st, kt0 + tile_idx * BN, last_k, v_lds + (tile_idx % NS) * TILE); };
-
+    // this wavefront's share of the direct loads of K / V tile `tile_idx`
+    auto dma_k_tile = [&](int tile_idx) {
+        if (tile_idx < n_tiles) k_plan.issue(kbase, p.k_st, kt0 + tile_idx * BN, last_k, k_lds + (tile_idx % NS) * TILE);
+    };
+    auto dma_v_tile = [&](int tile_idx) {
+        if (tile_idx < n_tiles) v_plan.issue(vbase, p.v_st, kt0 + tile_idx * BN, last_k, v_lds + (tile_idx % NS) * TILE);
+    };
     // ---- main loop ---------------------------------------------------------------------------
     // Each wavefront alternates an MFMA phase (O^T += V^T P^T of the previous tile, then S^T of the
     // current one) and a VALU phase (softmax of the current tile), with a workgroup barrier after each.
@@ -179,18 +182,6 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     //   loader waits for a tile right before the barrier that precedes its first read.
     // wave-uniform by construction: the extra barriers below must sit behind scalar branches
     const int grp = (NW == 8) ? wave >> 2 : 0;
-    auto dma_k_tile = [&](int tile_idx) {
-        if (tile_idx < n_tiles) {
-#pragma unroll
-            for (int j = 0; j < IPW; ++j) dma_k(tile_idx, j);
-        }
-    };
-    auto dma_v_tile = [&](int tile_idx) {
-        if (tile_idx < n_tiles) {
-#pragma unroll
-            for (int j = 0; j < IPW; ++j) dma_v(tile_idx, j);
-        }
-    };
     // number of direct-load instructions a loader issues for tiles [a, b)
     auto n_issued = [&](int a, int b) { return IPW * max(0, min(b, n_tiles) - a); };
     if (n_tiles > 0) {
