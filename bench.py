@@ -29,6 +29,15 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, vendor figure
 
+# HBM bytes per launch of the attention kernels on the headline workload: rocprofv3 FETCH_SIZE and WRITE_SIZE
+# (KiB per dispatch, one counter per run), scaled by what the same counters read for a plain 1 GiB device copy
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Summary and commands: profiles/attention_fwd_bwd_gqa32x8_d128_s8192_hbm_traffic.md
+MEASURED_TRAFFIC_KIB = {
+    "attn_fwd_kernel": 2.0 * 72047 + 66562,
+    "attn_bwd_dkdv_kernel": 2.0 * 705646 + 32820,
+    "attn_bwd_dq_kernel": 2.0 * 106418 + 65537,
+}
+
 
 def causal_pairs(cu):
     return sum((b - a) * (b - a + 1) // 2 for a, b in zip(cu[:-1], cu[1:]))
@@ -269,7 +278,8 @@ def main():
     dom_ms, dom_mult = kernels[dom]
     achieved = dom_mult * flops_unit / (dom_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None, "avg_launch_ms": dom_ms}
+                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_KIB[dom] * 1024.0, "traffic_unit": "bytes per launch",
+                "avg_launch_ms": dom_ms}
 
     extra = {"headline": main_res}
     if not args.no_extra:
