@@ -16,7 +16,6 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int kThreads = 256;
 constexpr int kChunk = 32;           // keys per wavefront and iteration
 constexpr int kMaxSplits = 32;
 
@@ -64,18 +63,21 @@ __global__ void decode_append_kernel(const DecodeParams p) {
 }
 
 // ---- split kernel ----------------------------------------------------------------------------------
-template <int D, bool ROT>
-__global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeParams p) {
+// NWV wavefronts (4 or 8) share the keys of one (batch, KV head, split); with a single split the merged result
+// is the attention output and goes straight to `o`, otherwise the partial goes to the workspace.
+template <int D, bool ROT, int NWV>
+__global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeParams p) {
+    constexpr int kThreads = 64 * NWV;
     constexpr int KS = D / 32;          // contraction steps of Q K^T (32 features each)
     constexpr int DT = D / 16;          // 16-row tiles of O^T
-    constexpr int VROW = kChunk + 8;    // padded row of the transposed V chunk (elements)
+    constexpr int VSTR = 2 * D + 32;    // bytes per key row of the staged V chunk: transpose reads of 8 rows x 32 bytes hit 256 distinct bytes
     constexpr int V_ITEMS = 8 * (D / 8);  // (key quad, feature group) items of a 32-key chunk
     constexpr int V_PER_LANE = V_ITEMS / 64;
 
-    __shared__ __attribute__((aligned(16))) uint16_t vt_lds[4][D * VROW];
-    __shared__ float wm_lds[4][16];
-    __shared__ float wl_lds[4][16];
-    __shared__ float wo_lds[4][16][D + 1];
+    __shared__ __attribute__((aligned(16))) char v_lds[NWV][kChunk * VSTR];
+    __shared__ float wm_lds[NWV][16];
+    __shared__ float wl_lds[NWV][16];
+    __shared__ float wo_lds[NWV][16][D + 1];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, l16 = lane & 15, G = lane >> 4;
@@ -88,10 +90,10 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
     ctx = ctx < 0 ? 0 : (ctx > p.max_ctx ? p.max_ctx : ctx);
     // keys of this split: [s0, s1), split length rounded up to whole workgroup iterations
     int per = (ctx + p.n_splits - 1) / p.n_splits;
-    per = (per + 4 * kChunk - 1) / (4 * kChunk) * (4 * kChunk);
+    per = (per + NWV * kChunk - 1) / (NWV * kChunk) * (NWV * kChunk);
     const int s0 = split * per;
     const int s1 = min(ctx, s0 + per);
-    const int n_iter = s1 > s0 ? (s1 - s0 + 4 * kChunk - 1) / (4 * kChunk) : 0;
+    const int n_iter = s1 > s0 ? (s1 - s0 + NWV * kChunk - 1) / (NWV * kChunk) : 0;
 
     // Q^T fragments: column = head slot l16 (valid when < n_rep), contraction = features 32*ks + 8*G + i
     bf16x8_t qf[KS];
@@ -125,7 +127,9 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
 
     const __bf16* kbase = p.kc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
     const __bf16* vbase = p.vc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
-    char* vt = reinterpret_cast<char*>(vt_lds[wave]);
+    char* vt = v_lds[wave];
+    // transpose-read base of this lane: keys 4G + (l16 >> 2), features 4 * (l16 & 3) (+ 16 per feature tile, + 16 keys for the second half)
+    const char* vt_lane = vt + (4 * G + (l16 >> 2)) * VSTR + 8 * (l16 & 3);
 
     // K fragments and V rows of a chunk; two sets so that the loads of chunk i+1 are in flight while
     // chunk i is being processed
@@ -134,7 +138,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
         uint4 vraw[V_PER_LANE][4];
     };
     auto load_chunk = [&](ChunkRegs& c, int it) {
-        const int key0 = s0 + (4 * it + wave) * kChunk;
+        const int key0 = s0 + (NWV * it + wave) * kChunk;
         if (key0 >= s1) return;
         const int last = s1 - 1;
 #pragma unroll
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
         }
     };
     auto process_chunk = [&](const ChunkRegs& c, int it) {
-        const int key0 = s0 + (4 * it + wave) * kChunk;
+        const int key0 = s0 + (NWV * it + wave) * kChunk;
         const bool active = key0 < s1;          // wave-uniform
         // Each wavefront owns its LDS chunk; the LDS pipeline executes one wavefront's accesses in program
         // order, so wavefront-scope fences (compiler ordering only) are enough and the wavefronts of a
@@ -196,22 +200,21 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
                     pf[4 * t + r] = (__bf16)e;   // slot (G, i): key 16*(i/4) + 4*G + (i%4)
                 }
             l_i = l_i * alpha + rs;
-            // transposed, slot-ordered copy of the V chunk: row = feature, 8 slots of lane group G contiguous
+            // key-major copy of the V chunk (rows as loaded); the PV operand is read back transposed
 #pragma unroll
             for (int j = 0; j < V_PER_LANE; ++j) {
                 const int item = lane + 64 * j;
                 const int quad = item / (D / 8), dg = item % (D / 8);
-                const int col = 8 * (quad & 3) + 4 * (quad >> 2);
 #pragma unroll
-                for (int dd = 0; dd < 8; ++dd)
-                    *reinterpret_cast<uint2*>(vt + ((8 * dg + dd) * VROW + col) * 2) = transpose_quad(c.vraw[j], dd);
+                for (int r = 0; r < 4; ++r) st128(vt + (4 * quad + r) * VSTR + 16 * dg, c.vraw[j][r]);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         if (active) {
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(vt + ((16 * dt + l16) * VROW + 8 * G) * 2);
+                // slots 0-3: keys 4G..4G+3, slots 4-7: keys 16+4G..16+4G+3 (the order of pf)
+                const bf16x8_t a = tr_pair(vt_lane + 32 * dt, vt_lane + 16 * VSTR + 32 * dt);
                 o_acc[dt] = o_acc[dt] * alpha;
                 o_acc[dt] = mfma_16x16x32(a, pf, o_acc[dt]);
             }
@@ -245,18 +248,23 @@ __global__ __launch_bounds__(kThreads, 2) void decode_split_kernel(const DecodeP
         const int hs = idx / D, d = idx % D;
         float M = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) M = fmaxf(M, wm_lds[w][hs]);
+        for (int w = 0; w < NWV; ++w) M = fmaxf(M, wm_lds[w][hs]);
         float L = 0.f, O = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < NWV; ++w) {
             const float wm = wm_lds[w][hs];
             const float f = wm == -INFINITY ? 0.f : fast_exp2(wm - M);
             L += f * wl_lds[w][hs];
             O += f * wo_lds[w][hs][d];
         }
-        const int64_t slot = ((int64_t)b * p.nq + kvh * p.n_rep + hs) * p.n_splits + split;
-        p.ws_o[slot * D + d] = O;
-        if (d == 0) { p.ws_ml[slot * 2] = M; p.ws_ml[slot * 2 + 1] = L; }
+        const int64_t bh = (int64_t)b * p.nq + kvh * p.n_rep + hs;
+        if (p.n_splits == 1) {
+            p.o[bh * D + d] = (__bf16)(L > 0.f ? O / L : 0.f);
+        } else {
+            const int64_t slot = bh * p.n_splits + split;
+            p.ws_o[slot * D + d] = O;
+            if (d == 0) { p.ws_ml[slot * 2] = M; p.ws_ml[slot * 2 + 1] = L; }
+        }
     }
 }
 
@@ -280,14 +288,31 @@ __global__ void decode_merge_kernel(const DecodeParams p) {
     p.o[bh * D + d] = (__bf16)(L > 0.f ? O / L : 0.f);
 }
 
+// 8-wavefront workgroups (one per compute unit) once there is a (batch, KV head) pair for most of the 256
+// compute units: then one split does and the merge kernel is not launched; otherwise 4-wavefront workgroups
+// and enough splits for about two workgroups per compute unit.
+bool wide_blocks(int batch, int nkv) { return (int64_t)batch * nkv >= 192; }
+
 int choose_splits(int batch, int nkv, int max_ctx) {
     const int64_t pairs = (int64_t)batch * nkv;
-    int64_t s = (512 + pairs - 1) / pairs;   // two 256-thread workgroups per compute unit = one round of blocks
+    if (wide_blocks(batch, nkv)) return 1;
+    int64_t s = (512 + pairs - 1) / pairs;
     const int64_t by_len = ((int64_t)max_ctx + 4 * kChunk - 1) / (4 * kChunk);
     if (s > by_len) s = by_len;
     if (s > kMaxSplits) s = kMaxSplits;
     if (s < 1) s = 1;
     return (int)s;
+}
+
+template <int D, int NWV> int launch_split(const DecodeParams& p, bool rot, hipStream_t st) {
+    const unsigned grid = (unsigned)p.batch * p.nkv * p.n_splits;
+    if (rot) {
+        if constexpr (D == 64 || D == 128) decode_split_kernel<D, true, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
+        else return mi_fail(MI_E_SHAPE, "attn_decode: fused rotary needs head_dim 64 or 128");
+    } else {
+        decode_split_kernel<D, false, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
+    }
+    return mi_check_launch("decode_split");
 }
 
 template <int D> int launch_decode(const DecodeParams& p, bool append, bool rot, hipStream_t st) {
@@ -297,15 +322,8 @@ template <int D> int launch_decode(const DecodeParams& p, bool append, bool rot,
         int rc = mi_check_launch("decode_append");
         if (rc != MI_OK) return rc;
     }
-    const unsigned grid = (unsigned)p.batch * p.nkv * p.n_splits;
-    if (rot) {
-        if constexpr (D == 64 || D == 128) decode_split_kernel<D, true><<<dim3(grid), dim3(kThreads), 0, st>>>(p);
-        else return mi_fail(MI_E_SHAPE, "attn_decode: fused rotary needs head_dim 64 or 128");
-    } else {
-        decode_split_kernel<D, false><<<dim3(grid), dim3(kThreads), 0, st>>>(p);
-    }
-    int rc = mi_check_launch("decode_split");
-    if (rc != MI_OK) return rc;
+    const int rc = wide_blocks(p.batch, p.nkv) ? launch_split<D, 8>(p, rot, st) : launch_split<D, 4>(p, rot, st);
+    if (rc != MI_OK || p.n_splits == 1) return rc;
     const int64_t n = (int64_t)p.batch * p.nq * D;
     decode_merge_kernel<D><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(p);
     return mi_check_launch("decode_merge");

@@ -35,6 +35,9 @@ def _oracle_decode(q, kc, vc, ctx, scale, dtype):
     (2, 4, 4, 64, 128, [128, 5]),
     (4, 32, 8, 128, 1100, [1024, 1025, 33, 1100]),
     (1, 16, 1, 128, 64, [64]),
+    # batch x KV heads >= 192: the 8-wavefront workgroups (a single split writes the output directly)
+    (24, 16, 8, 128, 300, [300, 1, 257, 31] * 6),
+    (48, 8, 4, 64, 520, [520, 256, 255, 7, 300, 513] * 8),
 ])
 @pytest.mark.parametrize("n_splits", [0, 1, 3])
 def test_decode_parity(B, nq, nkv, d, max_ctx, lens, n_splits):
