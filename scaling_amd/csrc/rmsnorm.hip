@@ -173,7 +173,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
 // flight per block and the per-thread slices (raw row vectors, packed weight, fp32 dweight) are small
 // enough for 16 wavefronts per compute unit; the number of per-block dweight partial rows stays <= 512.
 // One barrier per row step (both row sums travel through a double-buffered LDS slot).
-constexpr int kWideBlock = 1024;
+constexpr int kWideBlock = 512;     // two blocks per compute unit: one loads while the other computes
+constexpr int kWideMaxBlocks = 512;
 
 template <typename T, int TPR, int CH>
 __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T* __restrict__ x, const T* __restrict__ w,
@@ -203,19 +204,28 @@ __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T
     __syncthreads();
     const int64_t row_step = (int64_t)gridDim.x * RPB;
     const int64_t iters = (n_rows + row_step - 1) / row_step;
-    for (int64_t it = 0; it < iters; ++it) {
+    // the rows of iteration it + 1 are fetched while iteration it is reduced, so loads stay in flight
+    // across the block-wide reductions
+    uint4 xraw[CH], graw[CH], xnext[CH], gnext[CH];
+    auto fetch = [&](int64_t it, uint4 (&xv)[CH], uint4 (&gv)[CH]) {
         const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
         const bool row_ok = row < n_rows;
         const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
         const uint4* gr = reinterpret_cast<const uint4*>(dy + (row_ok ? row : 0) * hidden);
-        uint4 xraw[CH], graw[CH];
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int v = c * TPR + tr;
             const bool ok = row_ok && v < vecs;
-            xraw[c] = ok ? xr[v] : make_uint4(0, 0, 0, 0);
-            graw[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
+            xv[c] = ok ? xr[v] : make_uint4(0, 0, 0, 0);
+            gv[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
         }
+    };
+    constexpr bool kPrefetch = CH <= 2;   // beyond that the second register set would spill
+    if (iters > 0) fetch(0, xraw, graw);
+    for (int64_t it = 0; it < iters; ++it) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        if (kPrefetch) { if (it + 1 < iters) fetch(it + 1, xnext, gnext); }
         float ss = 0.f, dot = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
@@ -265,6 +275,12 @@ __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T
                     dxr[v] = Elem<T>::pack(o);
                 }
             }
+        }
+        if (kPrefetch) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) { xraw[c] = xnext[c]; graw[c] = gnext[c]; }
+        } else if (it + 1 < iters) {
+            fetch(it + 1, xraw, graw);
         }
     }
     for (int i = threadIdx.x; i < hidden; i += kWideBlock) dw_lds[i] = 0.f;
@@ -380,10 +396,13 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
         return mi_fail(MI_E_SHAPE, "rmsnorm: hidden=%lld unsupported", (long long)hidden);
     const int64_t vecs = hidden / Elem<T>::kVec;
     const bool wide = vecs >= 256;
-    // wide rows: 128 threads per row up to 512 vectors (8 rows per block), 256 threads per row beyond
-    const int wide_tpr = vecs <= 512 ? 128 : 256;
-    // one 1024-thread block per compute unit: a single round of blocks, each amortising its epilogue over more rows
-    const int blocks = wide ? (bwd_blocks(n_rows, wide_tpr / 4) > 256 ? 256 : bwd_blocks(n_rows, wide_tpr / 4)) : bwd_blocks(n_rows, plan.tpr);
+    // wide rows: 256 threads per row up to 512 vectors (2 rows per block), the whole block per row beyond
+    const int wide_tpr = vecs <= 512 ? 256 : 512;
+    // wide rows: a single round of blocks (two per compute unit), each amortising its epilogue over many rows
+    const int wide_rpb = kWideBlock / wide_tpr;
+    const int64_t wide_blocks = (n_rows + wide_rpb - 1) / wide_rpb;
+    const int blocks = wide ? (int)(wide_blocks > kWideMaxBlocks ? kWideMaxBlocks : (wide_blocks < 1 ? 1 : wide_blocks))
+                            : bwd_blocks(n_rows, plan.tpr);
     if (ws == nullptr || ws_bytes < (size_t)blocks * hidden * sizeof(float))
         return mi_fail(MI_E_WORKSPACE, "rmsnorm_bwd: workspace needs %zu bytes, got %zu",
                        (size_t)blocks * hidden * sizeof(float), ws_bytes);
@@ -392,8 +411,8 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
         const size_t lds = 2 * hidden * sizeof(float);
 #define RMS_WIDE(TPRV, CHV) rmsnorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kWideBlock), lds, st>>>( \
             (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps)
-        if (wide_tpr == 128) { if (ch <= 2) RMS_WIDE(128, 2); else RMS_WIDE(128, 4); }
-        else { if (ch <= 4) RMS_WIDE(256, 4); else RMS_WIDE(256, 8); }
+        if (wide_tpr == 256) { if (ch <= 1) RMS_WIDE(256, 1); else RMS_WIDE(256, 2); }
+        else { if (ch <= 2) RMS_WIDE(512, 2); else RMS_WIDE(512, 4); }
 #undef RMS_WIDE
         int rcw = mi_check_launch("rmsnorm_bwd_wide");
         if (rcw != MI_OK) return rcw;

@@ -16,7 +16,7 @@ def _rand(gen, *shape, dtype=torch.bfloat16, scale=1.0):
     return (torch.randn(*shape, generator=gen) * scale).to(dtype)
 
 
-@pytest.mark.parametrize("rows,hidden", [(2 * 128, 256), (37, 128), (1024, 4096), (19, 8192), (5, 1000 * 8), (64, 64)])
+@pytest.mark.parametrize("rows,hidden", [(2 * 128, 256), (37, 128), (1024, 4096), (19, 8192), (5, 1000 * 8), (64, 64), (7, 16384)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_rmsnorm_parity(rows, hidden, dtype):
     print(f"case rmsnorm rows={rows} hidden={hidden} dtype={dtype}", flush=True)
