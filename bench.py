@@ -131,6 +131,11 @@ def bandwidth_cases(steps, warmup):
     out["rmsnorm_fwd"] = {"ms": ms, "GBs": 2 * N * H * 2 / ms / 1e6}
     ms = time_gpu(lambda: ops.rms_norm_backward(x, w, dy, 1e-5), steps, warmup)
     out["rmsnorm_bwd"] = {"ms": ms, "GBs": 3 * N * H * 2 / ms / 1e6}
+    bias = torch.zeros(H, dtype=torch.bfloat16, device=dev)
+    ms = time_gpu(lambda: ops.layer_norm_forward(x, w, bias, 1e-5), steps, warmup)
+    out["layernorm_fwd"] = {"ms": ms, "GBs": 2 * N * H * 2 / ms / 1e6}
+    ms = time_gpu(lambda: ops.layer_norm_backward(x, w, dy, 1e-5), steps, warmup)
+    out["layernorm_bwd"] = {"ms": ms, "GBs": 3 * N * H * 2 / ms / 1e6}
     a = torch.randn(N, I, generator=g).bfloat16().to(dev)
     gate = torch.randn(N, I, generator=g).bfloat16().to(dev)
     dout = torch.randn(N, I, generator=g).bfloat16().to(dev)
@@ -138,6 +143,10 @@ def bandwidth_cases(steps, warmup):
     out["swiglu_fwd"] = {"ms": ms, "GBs": 3 * N * I * 2 / ms / 1e6}
     ms = time_gpu(lambda: ops.swiglu_backward(a, gate, dout), steps, warmup)
     out["swiglu_bwd"] = {"ms": ms, "GBs": 5 * N * I * 2 / ms / 1e6}
+    ms = time_gpu(lambda: ops.gelu_forward(a), steps, warmup)
+    out["gelu_fwd"] = {"ms": ms, "GBs": 2 * N * I * 2 / ms / 1e6}
+    ms = time_gpu(lambda: ops.gelu_backward(a, dout), steps, warmup)
+    out["gelu_bwd"] = {"ms": ms, "GBs": 3 * N * I * 2 / ms / 1e6}
     del a, gate, dout
     nq, nkv, d = 32, 8, 128
     qk = torch.randn(N, nq + nkv, d, generator=g).bfloat16().to(dev)

@@ -71,6 +71,30 @@ int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, 
                    int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * LayerNorm.  Replaces core/nn/norm/layernorm.py:75-86 (torch.nn.functional.layer_norm over the last
+ * dimension):  y = (x - mean) * rsqrt(var + eps) * weight + bias, biased variance, fp32 arithmetic, one
+ * rounding to `dtype` on store.  bias may be NULL.  Backward recomputes mean / rstd from x:
+ *   dx = rstd * (dy*w - mean(dy*w) - xhat * mean(dy*w*xhat)),  dweight = sum_rows dy*xhat,  dbias = sum_rows dy
+ * (dbias may be NULL).  `workspace`: fp32, at least mi_layernorm_bwd_workspace_bytes(n_rows, hidden) bytes;
+ * partial sums are reduced in a fixed order.  Algorithmic HBM bytes as for RMSNorm.
+ * ------------------------------------------------------------------------------------------ */
+int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* y,
+                     int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
+size_t mi_layernorm_bwd_workspace_bytes(int64_t n_rows, int64_t hidden);
+int mi_layernorm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dweight, void* dbias,
+                     void* workspace, size_t workspace_bytes,
+                     int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * GELU activation of the default MLP.  Replaces core/nn/mlp.py:135-139 with
+ * core/nn/activation_function.py:13-14 (torch.nn.functional.gelu, exact erf form):
+ *   y = 0.5 * x * (1 + erf(x / sqrt 2)),   dx = dy * (0.5 * (1 + erf(x / sqrt 2)) + x * exp(-x^2/2) / sqrt(2 pi)).
+ * Algorithmic HBM bytes: fwd 2*n_elem*e, bwd 3*n_elem*e.
+ * ------------------------------------------------------------------------------------------ */
+int mi_gelu_fwd(const void* x, void* y, int64_t n_elem, int dtype, void* stream);
+int mi_gelu_bwd(const void* x, const void* dy, void* dx, int64_t n_elem, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * SwiGLU activation.  Replaces core/nn/mlp.py:248-249:  out = silu(a) * gate, elementwise over
  * n_elem contiguous elements.  Backward: da = dout*gate*sig(a)*(1 + a*(1 - sig(a))), dgate = dout*silu(a).
  * Algorithmic HBM bytes: fwd 3*n_elem*e, bwd 5*n_elem*e.

@@ -88,6 +88,11 @@ def self_attention(spec: LayerSpec, w: Dict[str, torch.Tensor], x: torch.Tensor,
         k = F.linear(x, w[prefix + ".key.weight"], w.get(prefix + ".key.bias")).view(b, s, nkv, d).permute(1, 0, 2, 3)
         v = F.linear(x, w[prefix + ".value.weight"], w.get(prefix + ".value.bias")).view(b, s, nkv, d).permute(1, 0, 2, 3)
 
+    # query / key norm over head_dim, before the rotary embedding (attention.py:712-732, 819-834)
+    if prefix + ".norm_query.weight" in w:
+        q = _norm(spec, q, w, prefix + ".norm_query")
+        k = _norm(spec, k, w, prefix + ".norm_key")
+
     ids = None if position_ids is None else position_ids.transpose(0, 1)  # "b sq -> sq b", line 838-839
     if spec.rotary == "rotary":
         q, k = apply_rotary(q, k, tables if tables is not None else spec.tables(), ids, ids)

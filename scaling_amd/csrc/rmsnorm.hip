@@ -434,6 +434,221 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
     return mi_check_launch("rmsnorm_dw_reduce");
 }
 
+// ---- LayerNorm (weight and optional bias) -----------------------------------------------------------------
+// Same row ownership as the RMSNorm kernels.  Mean and variance are taken in fp32 from the register copy of
+// the row (two passes over registers, one over HBM).
+template <typename T, int TPR, int CH>
+__global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                const T* __restrict__ b, T* __restrict__ y,
+                                                                int64_t n_rows, int hidden, float eps) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int RPB = kBlock / TPR;
+    __shared__ float lds[4];
+    const int tr = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+    const bool row_ok = row < n_rows;
+    const int vecs = hidden / V;
+    const float inv_h = 1.0f / (float)hidden;
+    const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
+    float f[CH][V];
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int v = c * TPR + tr;
+        const uint4 raw = (row_ok && v < vecs) ? xr[v] : make_uint4(0, 0, 0, 0);
+        Elem<T>::unpack(raw, f[c]);
+#pragma unroll
+        for (int i = 0; i < V; ++i) sum += f[c][i];
+    }
+    const float mean = row_sum<TPR>(sum, lds) * inv_h;
+    float sq = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool live = c * TPR + tr < vecs;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const float dlt = live ? f[c][i] - mean : 0.f;
+            sq += dlt * dlt;
+        }
+    }
+    const float rstd = rsqrtf(row_sum<TPR>(sq, lds) * inv_h + eps);
+    if (!row_ok) return;
+    const uint4* wr = reinterpret_cast<const uint4*>(w);
+    const uint4* br = reinterpret_cast<const uint4*>(b);
+    uint4* yr = reinterpret_cast<uint4*>(y + row * hidden);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int v = c * TPR + tr;
+        if (v < vecs) {
+            float g[V], bb[V], o[V];
+            Elem<T>::unpack(wr[v], g);
+            if (b != nullptr) Elem<T>::unpack(br[v], bb);
+#pragma unroll
+            for (int i = 0; i < V; ++i) o[i] = (f[c][i] - mean) * rstd * g[i] + (b != nullptr ? bb[i] : 0.f);
+            yr[v] = Elem<T>::pack(o);
+        }
+    }
+}
+
+// dx = rstd * (g*w - mean(g*w) - xhat * mean(g*w*xhat)),  dw = sum_rows g * xhat,  db = sum_rows g
+// partial rows: [gridDim.x][hidden] of dw followed by [gridDim.x][hidden] of db
+template <typename T, int TPR, int CH>
+__global__ __launch_bounds__(kBlock) void layernorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                const T* __restrict__ dy, T* __restrict__ dx,
+                                                                float* __restrict__ partial, int64_t n_rows, int hidden,
+                                                                float eps) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int RPB = kBlock / TPR;
+    extern __shared__ float comb_lds[];  // [2][hidden]
+    __shared__ float lds[4];
+    const int tr = threadIdx.x % TPR;
+    const int rg = threadIdx.x / TPR;
+    const int vecs = hidden / V;
+    const float inv_h = 1.0f / (float)hidden;
+    const uint4* wr = reinterpret_cast<const uint4*>(w);
+
+    float acc_w[CH][V], acc_b[CH][V];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < V; ++i) { acc_w[c][i] = 0.f; acc_b[c][i] = 0.f; }
+
+    const int64_t row_step = (int64_t)gridDim.x * RPB;
+    const int64_t iters = (n_rows + row_step - 1) / row_step;   // same count in every thread (barriers in row_sum)
+    for (int64_t it = 0; it < iters; ++it) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
+        const uint4* gr = reinterpret_cast<const uint4*>(dy + (row_ok ? row : 0) * hidden);
+        float xf[CH][V], gw[CH][V];
+        uint4 graw[CH];
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int v = c * TPR + tr;
+            const bool ok = row_ok && v < vecs;
+            const uint4 xraw = ok ? xr[v] : make_uint4(0, 0, 0, 0);
+            graw[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
+            Elem<T>::unpack(xraw, xf[c]);
+#pragma unroll
+            for (int i = 0; i < V; ++i) sum += xf[c][i];
+        }
+        const float mean = row_sum<TPR>(sum, lds) * inv_h;
+        float sq = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const bool live = row_ok && c * TPR + tr < vecs;
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                xf[c][i] = live ? xf[c][i] - mean : 0.f;
+                sq += xf[c][i] * xf[c][i];
+            }
+        }
+        const float rstd = rsqrtf(row_sum<TPR>(sq, lds) * inv_h + eps);
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int v = c * TPR + tr;
+            float gf[V], wf[V];
+            Elem<T>::unpack(graw[c], gf);
+            Elem<T>::unpack(v < vecs ? wr[v] : make_uint4(0, 0, 0, 0), wf);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                xf[c][i] *= rstd;                       // xhat
+                gw[c][i] = gf[i] * wf[i];
+                s1 += gw[c][i];
+                s2 += gw[c][i] * xf[c][i];
+                acc_w[c][i] += gf[i] * xf[c][i];
+                acc_b[c][i] += gf[i];
+            }
+        }
+        s1 = row_sum<TPR>(s1, lds) * inv_h;
+        s2 = row_sum<TPR>(s2, lds) * inv_h;
+        if (row_ok) {
+            uint4* dxr = reinterpret_cast<uint4*>(dx + row * hidden);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+                    float o[V];
+#pragma unroll
+                    for (int i = 0; i < V; ++i) o[i] = rstd * (gw[c][i] - s1 - xf[c][i] * s2);
+                    dxr[v] = Elem<T>::pack(o);
+                }
+            }
+        }
+    }
+
+    // combine the row groups of this block in a fixed order, then emit one partial row each for dw and db
+    for (int i = threadIdx.x; i < 2 * hidden; i += kBlock) comb_lds[i] = 0.f;
+    __syncthreads();
+    for (int g = 0; g < RPB; ++g) {
+        if (rg == g) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        comb_lds[v * V + i] += acc_w[c][i];
+                        comb_lds[hidden + v * V + i] += acc_b[c][i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out_w = partial + (int64_t)blockIdx.x * hidden;
+    float* out_b = partial + ((int64_t)gridDim.x + blockIdx.x) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kBlock) { out_w[i] = comb_lds[i]; out_b[i] = comb_lds[hidden + i]; }
+}
+
+template <typename T>
+int launch_ln_fwd(const void* x, const void* w, const void* b, void* y, int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
+    Plan plan;
+    if (!make_plan<T>(hidden, &plan))
+        return mi_fail(MI_E_SHAPE, "layernorm: hidden=%lld unsupported (must be a multiple of %d and <= %d)",
+                       (long long)hidden, Elem<T>::kVec, 256 * 8 * Elem<T>::kVec);
+    const bool launched = dispatch_plan(plan, [&](auto tag) {
+        constexpr int TPR = decltype(tag)::TPR;
+        constexpr int CH = decltype(tag)::CH;
+        const int rpb = kBlock / TPR;
+        const unsigned grid = (unsigned)((n_rows + rpb - 1) / rpb);
+        layernorm_fwd_kernel<T, TPR, CH><<<dim3(grid), dim3(kBlock), 0, st>>>((const T*)x, (const T*)w, (const T*)b, (T*)y,
+                                                                              n_rows, (int)hidden, eps);
+    });
+    if (!launched) return mi_fail(MI_E_SHAPE, "layernorm: no kernel for hidden=%lld", (long long)hidden);
+    return mi_check_launch("layernorm_fwd");
+}
+
+template <typename T>
+int launch_ln_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, void* db, void* ws, size_t ws_bytes,
+                  int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
+    Plan plan;
+    if (!make_plan<T>(hidden, &plan)) return mi_fail(MI_E_SHAPE, "layernorm: hidden=%lld unsupported", (long long)hidden);
+    int blocks = bwd_blocks(n_rows, plan.tpr);
+    if (blocks > 256) blocks = 256;
+    if (ws == nullptr || ws_bytes < (size_t)2 * blocks * hidden * sizeof(float))
+        return mi_fail(MI_E_WORKSPACE, "layernorm_bwd: workspace needs %zu bytes, got %zu",
+                       (size_t)2 * blocks * hidden * sizeof(float), ws_bytes);
+    const bool launched = dispatch_plan(plan, [&](auto tag) {
+        constexpr int TPR = decltype(tag)::TPR;
+        constexpr int CH = decltype(tag)::CH;
+        layernorm_bwd_kernel<T, TPR, CH><<<dim3(blocks), dim3(kBlock), 2 * hidden * sizeof(float), st>>>(
+            (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps);
+    });
+    if (!launched) return mi_fail(MI_E_SHAPE, "layernorm: no kernel for hidden=%lld", (long long)hidden);
+    int rc = mi_check_launch("layernorm_bwd");
+    if (rc != MI_OK) return rc;
+    const unsigned rgrid = (unsigned)((hidden + 15) / 16);
+    rmsnorm_dw_reduce_kernel<T><<<dim3(rgrid), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw, blocks, (int)hidden);
+    rc = mi_check_launch("layernorm_dw_reduce");
+    if (rc != MI_OK || db == nullptr) return rc;
+    rmsnorm_dw_reduce_kernel<T><<<dim3(rgrid), dim3(kBlock), 0, st>>>((const float*)ws + (size_t)blocks * hidden, (T*)db, blocks,
+                                                                      (int)hidden);
+    return mi_check_launch("layernorm_db_reduce");
+}
+
 }  // namespace
 
 extern "C" {
@@ -462,6 +677,35 @@ int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, 
     if (2 * hidden * sizeof(float) > 160 * 1024 - 256) return mi_fail(MI_E_SHAPE, "rmsnorm_bwd: hidden too large for LDS");
     MI_DISPATCH_DTYPE(dtype, return launch_bwd<T>(x, weight, dy, dx, dweight, workspace, workspace_bytes, n_rows, hidden,
                                                   eps, (hipStream_t)stream));
+    return MI_OK;
+}
+
+int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* y, int64_t n_rows, int64_t hidden,
+                     float eps, int dtype, void* stream) {
+    if (!x || !weight || !y) return mi_fail(MI_E_NULL, "layernorm_fwd: null pointer");
+    if (n_rows < 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "layernorm_fwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
+    if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(y) || (bias && !mi_aligned16(bias)))
+        return mi_fail(MI_E_ALIGN, "layernorm_fwd: pointers must be 16-byte aligned");
+    if (n_rows == 0) return MI_OK;
+    MI_DISPATCH_DTYPE(dtype, return launch_ln_fwd<T>(x, weight, bias, y, n_rows, hidden, eps, (hipStream_t)stream));
+    return MI_OK;
+}
+
+size_t mi_layernorm_bwd_workspace_bytes(int64_t n_rows, int64_t hidden) {
+    (void)n_rows;
+    return (size_t)2 * 256 * (size_t)(hidden > 0 ? hidden : 0) * sizeof(float);
+}
+
+int mi_layernorm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dweight, void* dbias,
+                     void* workspace, size_t workspace_bytes, int64_t n_rows, int64_t hidden, float eps, int dtype,
+                     void* stream) {
+    if (!x || !weight || !dy || !dx || !dweight) return mi_fail(MI_E_NULL, "layernorm_bwd: null pointer");
+    if (n_rows <= 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "layernorm_bwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
+    if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(dy) || !mi_aligned16(dx) || !mi_aligned16(workspace))
+        return mi_fail(MI_E_ALIGN, "layernorm_bwd: pointers must be 16-byte aligned");
+    if (2 * hidden * sizeof(float) > 160 * 1024 - 256) return mi_fail(MI_E_SHAPE, "layernorm_bwd: hidden too large for LDS");
+    MI_DISPATCH_DTYPE(dtype, return launch_ln_bwd<T>(x, weight, dy, dx, dweight, dbias, workspace, workspace_bytes, n_rows,
+                                                     hidden, eps, (hipStream_t)stream));
     return MI_OK;
 }
 

@@ -1,4 +1,4 @@
-// SwiGLU activation forward / backward for gfx950: elementwise, 128-bit accesses, fp32 math.
+// Activation kernels for gfx950 (SwiGLU, exact GELU), forward / backward: elementwise, 128-bit accesses, fp32 math.
 #include "common.h"
 
 namespace {
@@ -87,6 +87,47 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const T* __restrict_
     }
 }
 
+// exact (erf) GELU, the reference's default activation (torch.nn.functional.gelu with approximate='none')
+__device__ __forceinline__ float gelu_f(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
+__device__ __forceinline__ float gelu_grad_f(float x) {
+    return 0.5f * (1.0f + erff(x * 0.7071067811865476f)) + x * 0.3989422804014327f * __expf(-0.5f * x * x);
+}
+
+// BWD = false: y = gelu(x) (dy unused);  BWD = true: y = dy * gelu'(x)
+template <typename T, bool BWD>
+__global__ __launch_bounds__(kBlock) void gelu_kernel(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ y,
+                                                       int64_t n_vec, int64_t n_elem) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t base = ((int64_t)blockIdx.x * kBlock) * kUnroll + threadIdx.x;
+    uint4 rx[kUnroll], rd[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = base + (int64_t)u * kBlock;
+        if (v < n_vec) {
+            rx[u] = reinterpret_cast<const uint4*>(x)[v];
+            if (BWD) rd[u] = reinterpret_cast<const uint4*>(dy)[v];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const int64_t v = base + (int64_t)u * kBlock;
+        if (v < n_vec) {
+            float fx[V], fd[V];
+            Elem<T>::unpack(rx[u], fx);
+            if (BWD) Elem<T>::unpack(rd[u], fd);
+#pragma unroll
+            for (int i = 0; i < V; ++i) fx[i] = BWD ? fd[i] * gelu_grad_f(fx[i]) : gelu_f(fx[i]);
+            reinterpret_cast<uint4*>(y)[v] = Elem<T>::pack(fx);
+        }
+    }
+    if (blockIdx.x == gridDim.x - 1) {
+        for (int64_t i = n_vec * V + threadIdx.x; i < n_elem; i += kBlock) {
+            const float a = Elem<T>::load1(x + i);
+            Elem<T>::store1(y + i, BWD ? Elem<T>::load1(dy + i) * gelu_grad_f(a) : gelu_f(a));
+        }
+    }
+}
+
 template <typename T> unsigned grid_for(int64_t n_elem, int64_t* n_vec) {
     *n_vec = n_elem / Elem<T>::kVec;
     int64_t blocks = (*n_vec + (int64_t)kBlock * kUnroll - 1) / ((int64_t)kBlock * kUnroll);
@@ -127,6 +168,34 @@ int mi_swiglu_bwd(const void* a, const void* gate, const void* dout, void* da, v
                                                                                   (T*)da, (T*)dgate, n_vec, n_elem);
     });
     return mi_check_launch("swiglu_bwd");
+}
+
+int mi_gelu_fwd(const void* x, void* y, int64_t n_elem, int dtype, void* stream) {
+    if (!x || !y) return mi_fail(MI_E_NULL, "gelu_fwd: null pointer");
+    if (n_elem < 0) return mi_fail(MI_E_SHAPE, "gelu_fwd: negative size");
+    if (!mi_aligned16(x) || !mi_aligned16(y)) return mi_fail(MI_E_ALIGN, "gelu_fwd: pointers must be 16-byte aligned");
+    if (n_elem == 0) return MI_OK;
+    if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "gelu_fwd: too many elements");
+    MI_DISPATCH_DTYPE(dtype, {
+        int64_t n_vec;
+        const unsigned grid = grid_for<T>(n_elem, &n_vec);
+        gelu_kernel<T, false><<<dim3(grid), dim3(kBlock), 0, (hipStream_t)stream>>>((const T*)x, nullptr, (T*)y, n_vec, n_elem);
+    });
+    return mi_check_launch("gelu_fwd");
+}
+
+int mi_gelu_bwd(const void* x, const void* dy, void* dx, int64_t n_elem, int dtype, void* stream) {
+    if (!x || !dy || !dx) return mi_fail(MI_E_NULL, "gelu_bwd: null pointer");
+    if (n_elem < 0) return mi_fail(MI_E_SHAPE, "gelu_bwd: negative size");
+    if (!mi_aligned16(x) || !mi_aligned16(dy) || !mi_aligned16(dx)) return mi_fail(MI_E_ALIGN, "gelu_bwd: pointers must be 16-byte aligned");
+    if (n_elem == 0) return MI_OK;
+    if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "gelu_bwd: too many elements");
+    MI_DISPATCH_DTYPE(dtype, {
+        int64_t n_vec;
+        const unsigned grid = grid_for<T>(n_elem, &n_vec);
+        gelu_kernel<T, true><<<dim3(grid), dim3(kBlock), 0, (hipStream_t)stream>>>((const T*)x, (const T*)dy, (T*)dx, n_vec, n_elem);
+    });
+    return mi_check_launch("gelu_bwd");
 }
 
 }  // extern "C"

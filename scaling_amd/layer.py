@@ -10,7 +10,7 @@ from typing import Callable, List, Optional
 import torch
 
 from .config import MLPType, TransformerArchitectureConfig
-from .nn import ParallelSelfAttention, ParallelSwiGLUMLP, get_norm
+from .nn import ParallelMLP, ParallelSelfAttention, ParallelSwiGLUMLP, get_norm
 
 
 class InferenceSettings:
@@ -55,8 +55,6 @@ def _check_architecture(cfg: TransformerArchitectureConfig) -> None:
     bad = [k for k, v in unsupported.items() if v]
     if bad:
         raise NotImplementedError(f"architecture options outside the hip layer's scope are set: {bad}")
-    if cfg.mlp_type != MLPType.SWIGLU:
-        raise NotImplementedError("mlp_type 'default' (GELU) has no HIP kernel in this package (supported: swiglu)")
 
 
 class TransformerLayer(torch.nn.Module):
@@ -84,8 +82,9 @@ class TransformerLayer(torch.nn.Module):
             num_kv_heads=cfg.attention_num_kv_heads, use_matmul=cfg.attention_use_matmul)
         self.dropout_attention = torch.nn.Dropout(cfg.dropout_after_attention)
         self.post_attention_layernorm = get_norm(cfg.norm_type, cfg.layernorm, cfg.hidden_size, device, dtype)
-        self.mlp = ParallelSwiGLUMLP(io_features=cfg.hidden_size, intermediate_feature_factor=cfg.mlp_factor,
-                                     bias=cfg.mlp_bias, device=device, dtype=dtype, init_method=init_method)
+        mlp_class = ParallelSwiGLUMLP if cfg.mlp_type == MLPType.SWIGLU else ParallelMLP   # layer.py:150-189 of the reference
+        self.mlp = mlp_class(io_features=cfg.hidden_size, intermediate_feature_factor=cfg.mlp_factor,
+                             bias=cfg.mlp_bias, device=device, dtype=dtype, init_method=init_method)
         self.dropout_mlp = torch.nn.Dropout(cfg.dropout_after_mlp)
 
     def attention_block(self, hidden_state: torch.Tensor, cumulative_seq_lengths: torch.Tensor,

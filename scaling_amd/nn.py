@@ -61,13 +61,38 @@ class RMSNorm(torch.nn.Module):
         return ops.rms_norm(x, self.weight, self.eps)
 
 
+class LayerNorm(torch.nn.Module):
+    """Mirror of core/nn/norm/layernorm.py:16-86 (`optimization_type: torch`; u-muP and bitfit bias names
+    excluded): weight ones, bias zeros, torch.nn.functional.layer_norm semantics."""
+
+    def __init__(self, config: Optional[LayerNormConfig], normalized_shape: int, device: Optional[torch.device] = None,
+                 dtype: torch.dtype = torch.float32, bitfit_bias_name: Optional[str] = None, topology=None,
+                 umup_on_residual: Optional[bool] = None) -> None:
+        super().__init__()
+        if bitfit_bias_name:
+            raise NotImplementedError("bitfit bias names are outside the layer hot path of this package")
+        device = _default_device(device, topology)
+        self.config = config if config is not None else LayerNormConfig()
+        self.eps = self.config.layernorm_epsilon
+        self.normalized_shape = torch.Size((normalized_shape,))
+        self.topology = None
+        self.weight = torch.nn.Parameter(torch.ones(normalized_shape, dtype=dtype, device=device))
+        self.bias = torch.nn.Parameter(torch.zeros(normalized_shape, dtype=dtype, device=device))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.layer_norm(x, self.weight, self.bias, self.eps)
+
+
 def get_norm(norm_type: NormType, layernorm_config: Optional[LayerNormConfig], dimensions: int,
              device: Optional[torch.device], dtype: torch.dtype, bitfit_bias_name: Optional[str] = None,
-             topology=None, umup_on_residual: Optional[bool] = None) -> RMSNorm:
-    """Mirror of core/nn/norm/get_norm.py:17-49; only the RMS branch has a kernel in this package."""
+             topology=None, umup_on_residual: Optional[bool] = None) -> torch.nn.Module:
+    """Mirror of core/nn/norm/get_norm.py:17-49."""
     if norm_type == NormType.RMS:
         return RMSNorm(dimensions=dimensions, device=device, config=layernorm_config, dtype=dtype, topology=topology)
-    raise NotImplementedError(f"norm_type {norm_type} has no HIP kernel in this package (supported: rms)")
+    if norm_type == NormType.LAYERNORM:
+        return LayerNorm(config=layernorm_config, normalized_shape=dimensions, device=device, dtype=dtype,
+                         bitfit_bias_name=bitfit_bias_name, topology=topology)
+    raise NotImplementedError(f"norm_type {norm_type} is not known")
 
 
 class RotaryEmbedding(torch.nn.Module):
@@ -163,6 +188,33 @@ class ParallelSwiGLUMLP(torch.nn.Module):
         return self.dense_out(ops.swiglu(self.dense_in(x), self.siglu_weight(x)))
 
 
+class ParallelMLP(torch.nn.Module):
+    """Mirror of core/nn/mlp.py:25-146 with the GELU activation (activation_function.py:13-14):
+    dense_out(gelu(dense_in(x)))."""
+
+    def __init__(self, io_features: int, intermediate_feature_factor: float, bias: bool = True,
+                 device: Optional[torch.device] = None, dtype: torch.dtype = torch.float32, topology=None,
+                 init_method: InitMethod = torch.nn.init.xavier_normal_, bitfit_bias_name: Optional[str] = None,
+                 activation_function: str = "gelu", umup_mult: Optional[float] = None,
+                 umup_is_first_layer: Optional[bool] = None, umup_is_last_layer: Optional[bool] = None,
+                 umup_on_residual: Optional[bool] = None, fp8_config=None, fp8_config_dense_out=None) -> None:
+        super().__init__()
+        device = _default_device(device, topology)
+        if fp8_config is not None or fp8_config_dense_out is not None or bitfit_bias_name is not None:
+            raise NotImplementedError("fp8 / bitfit options are outside the layer hot path of this package")
+        if getattr(activation_function, "value", activation_function) != "gelu":
+            raise NotImplementedError("ParallelMLP has a HIP kernel for the GELU activation only")
+        assert float(int(io_features * intermediate_feature_factor)) == io_features * intermediate_feature_factor, \
+            "io_features * intermediate_feature_factor does not result in a natural number for feature dimensions"
+        inter = int(io_features * intermediate_feature_factor)
+        self.topology = None
+        self.dense_in = _Linear(io_features, inter, bias, device, dtype, init_method)
+        self.dense_out = _Linear(inter, io_features, bias, device, dtype, init_method)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.dense_out(ops.gelu(self.dense_in(x)))
+
+
 class KVCache:
     """Pre-allocated cache of post-rotary K and un-repeated V, indexed [batch, token, kv head, d], replacing
     the reference's per-step torch.cat (core/nn/attention/attention.py:862-869).  Storage is head-major
@@ -183,7 +235,7 @@ class ParallelSelfAttention(torch.nn.Module):
 
     Same constructor arguments and forward signature.  Differences, all documented errors rather than
     silent fall-backs: attention-probability dropout, attention-score manipulation, LoRA, local
-    attention windows, u-muP, fp8 and LayerNorm query/key norm are not available;
+    attention windows, u-muP and fp8 are not available;
     the dtype must be bfloat16.  The KV cache is pre-allocated (see `KVCache`), supports batches of
     single-document rows and is filled/extended in place.
     """

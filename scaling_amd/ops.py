@@ -77,6 +77,90 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.
 
 
 # ------------------------------------------------------------------------------------------------
+# LayerNorm, GELU (the reference's default norm / activation)
+# ------------------------------------------------------------------------------------------------
+def layer_norm_forward(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    _need_cuda(x, weight, bias)
+    assert x.shape[-1] == weight.shape[0] and weight.dtype == x.dtype
+    x2 = x.contiguous().view(-1, x.shape[-1])
+    w = weight.contiguous()
+    b = bias.contiguous() if bias is not None else None
+    y = torch.empty_like(x2)
+    check(_lib.load().mi_layernorm_fwd(ptr(x2), ptr(w), ptr(b), ptr(y), x2.shape[0], x2.shape[1], float(eps),
+                                       dtype_code(x.dtype), stream_ptr()), "mi_layernorm_fwd")
+    return y.view(x.shape)
+
+
+def layer_norm_backward(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor, eps: float, need_bias_grad: bool = True):
+    _need_cuda(x, weight, dy)
+    lib = _lib.load()
+    x2 = x.contiguous().view(-1, x.shape[-1])
+    dy2 = dy.contiguous().view(-1, x.shape[-1])
+    w = weight.contiguous()
+    dx = torch.empty_like(x2)
+    dw = torch.empty_like(w)
+    db = torch.empty_like(w) if need_bias_grad else None
+    nbytes = lib.mi_layernorm_bwd_workspace_bytes(x2.shape[0], x2.shape[1])
+    ws = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
+    check(lib.mi_layernorm_bwd(ptr(x2), ptr(w), ptr(dy2), ptr(dx), ptr(dw), ptr(db), ptr(ws), nbytes, x2.shape[0],
+                               x2.shape[1], float(eps), dtype_code(x.dtype), stream_ptr()), "mi_layernorm_bwd")
+    return dx.view(x.shape), dw, db
+
+
+class _LayerNorm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        ctx.save_for_backward(x, weight)
+        ctx.eps = eps
+        ctx.has_bias = bias is not None
+        return layer_norm_forward(x, weight, bias, eps)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        dx, dw, db = layer_norm_backward(x, weight, dy, ctx.eps, ctx.has_bias)
+        return dx, dw, db, None
+
+
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
+    """(x - mean) * rsqrt(var + eps) * weight + bias over the last dimension (fp32 math, one rounding)."""
+    return _LayerNorm.apply(x, weight, bias, eps)
+
+
+def gelu_forward(x: torch.Tensor) -> torch.Tensor:
+    _need_cuda(x)
+    x = x.contiguous()
+    y = torch.empty_like(x)
+    check(_lib.load().mi_gelu_fwd(ptr(x), ptr(y), x.numel(), dtype_code(x.dtype), stream_ptr()), "mi_gelu_fwd")
+    return y
+
+
+def gelu_backward(x: torch.Tensor, dy: torch.Tensor) -> torch.Tensor:
+    _need_cuda(x, dy)
+    x, dy = x.contiguous(), dy.contiguous()
+    dx = torch.empty_like(x)
+    check(_lib.load().mi_gelu_bwd(ptr(x), ptr(dy), ptr(dx), x.numel(), dtype_code(x.dtype), stream_ptr()), "mi_gelu_bwd")
+    return dx
+
+
+class _GELU(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        ctx.save_for_backward(x)
+        return gelu_forward(x)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (x,) = ctx.saved_tensors
+        return gelu_backward(x, dy)
+
+
+def gelu(x: torch.Tensor) -> torch.Tensor:
+    """Exact (erf) GELU."""
+    return _GELU.apply(x)
+
+
+# ------------------------------------------------------------------------------------------------
 # SwiGLU
 # ------------------------------------------------------------------------------------------------
 def swiglu_forward(a: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:

@@ -1,5 +1,7 @@
-"""GPU parity of the bandwidth-bound kernels (RMSNorm, SwiGLU, rotary) against the CPU oracle,
+"""GPU parity of the bandwidth-bound kernels (RMSNorm, LayerNorm, SwiGLU, GELU, rotary) against the CPU oracle,
 called through the C ABI."""
+
+import os
 
 import pytest
 import torch
@@ -20,6 +22,8 @@ def _rand(gen, *shape, dtype=torch.bfloat16, scale=1.0):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_rmsnorm_parity(rows, hidden, dtype):
     print(f"case rmsnorm rows={rows} hidden={hidden} dtype={dtype}", flush=True)
+    if hidden // (8 if dtype == torch.bfloat16 else 4) > 2048:
+        pytest.skip("rows wider than 2048 vectors of 16 bytes are outside the kernels' range")
     g = torch.Generator().manual_seed(rows * 7 + hidden)
     x = _rand(g, rows, hidden, dtype=dtype)
     w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
@@ -164,3 +168,84 @@ def test_rotary_complex_parity(seq, batch, heads, dim, dtype):
     out_g.backward(go.to(DEV))
     torch.cuda.synchronize()
     check("rotary_complex.dx", xg.grad, xr.grad, **tol)
+
+
+@pytest.mark.parametrize("rows,hidden", [(2 * 128, 256), (37, 128), (1024, 4096), (19, 8192), (5, 1000 * 8), (64, 64), (300, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_layernorm_parity(rows, hidden, dtype, with_bias):
+    print(f"case layernorm rows={rows} hidden={hidden} dtype={dtype} bias={with_bias}", flush=True)
+    g = torch.Generator().manual_seed(rows * 11 + hidden)
+    x = (_rand(g, rows, hidden, dtype=torch.float32) + 0.5).to(dtype)       # non-zero mean
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(hidden, generator=g)).to(dtype) if with_bias else None
+    dy = _rand(g, rows, hidden, dtype=dtype)
+
+    def run(cast):
+        xs, ws = cast(x).clone().requires_grad_(), cast(w).clone().requires_grad_()
+        bs = cast(b).clone().requires_grad_() if with_bias else None
+        y = oracle.layer_norm(xs, ws, bs, 1e-5)
+        y.backward(cast(dy))
+        return y, xs.grad, ws.grad, (bs.grad if with_bias else None)
+
+    ref = run(lambda t: t.float())
+    ref_o = run(lambda t: t)                       # torch's own layer_norm in `dtype`
+    xg, wg = x.to(DEV).requires_grad_(), w.to(DEV).requires_grad_()
+    bg = b.to(DEV).requires_grad_() if with_bias else None
+    y = ops.layer_norm(xg, wg, bg, 1e-5)
+    y.backward(dy.to(DEV))
+    torch.cuda.synchronize()
+    tol = dict(max_abs_tol=2e-2, mean_rel_tol=1e-3) if dtype == torch.bfloat16 else dict(max_abs_tol=1e-4, mean_rel_tol=1e-5)
+    check("layernorm.y", y, ref[0], ref_o[0], **tol)
+    check("layernorm.dx", xg.grad, ref[1], ref_o[1], **tol)
+    check("layernorm.dw", wg.grad, ref[2], ref_o[2], **tol)
+    if with_bias:
+        check("layernorm.db", bg.grad, ref[3], ref_o[3], **tol)
+
+
+@pytest.mark.parametrize("shape", [(2, 128, 1024), (3, 7, 5), (4, 1000, 4096), (1, 1, 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_gelu_parity(shape, dtype):
+    print(f"case gelu shape={shape} dtype={dtype}", flush=True)
+    g = torch.Generator().manual_seed(sum(shape) + 1)
+    x, dy = (_rand(g, *shape, dtype=dtype, scale=2.0) for _ in range(2))
+    xr = x.float().clone().requires_grad_()
+    ref = torch.nn.functional.gelu(xr)             # the reference's activation (activation_function.py:13-14)
+    ref.backward(dy.float())
+    xo = x.clone().requires_grad_()
+    ref_o = torch.nn.functional.gelu(xo)
+    ref_o.backward(dy)
+    xg = x.to(DEV).requires_grad_()
+    y = ops.gelu(xg)
+    y.backward(dy.to(DEV))
+    torch.cuda.synchronize()
+    tol = dict(max_abs_tol=1e-5, mean_rel_tol=1e-5) if dtype == torch.float32 else dict(max_abs_tol=2e-2, mean_rel_tol=1e-3)
+    check("gelu.y", y, ref, ref_o, **tol)
+    check("gelu.dx", xg.grad, xr.grad, xo.grad, **tol)
+    # closed-form spot values: gelu(0) = 0, gelu'(0) = 0.5, gelu(x) -> x for large x
+    pts = torch.tensor([0.0, 10.0, -10.0, 1.0], device=DEV)
+    assert torch.allclose(ops.gelu_forward(pts), torch.tensor([0.0, 10.0, 0.0, 0.8413447], device=DEV), atol=1e-6)
+    assert torch.allclose(ops.gelu_backward(pts, torch.ones_like(pts))[:1], torch.tensor([0.5], device=DEV), atol=1e-7)
+
+
+def test_layernorm_and_gelu_mlp_reproduce_the_reference_golden(golden_dir):
+    """fp32 LayerNorm and GELU-MLP kernels on the activations held by the reference's own test-suite
+    (tests/transformer/files/backward_compatibility_checkpoint, gate 3e-3 in test_backwards_compatibility.py:175)."""
+    d = os.path.join(golden_dir, "backward_compatibility")
+    gt = torch.load(os.path.join(d, "ground_truth.pt"), weights_only=True)
+    sd = torch.load(os.path.join(d, "state_dict.pt"), weights_only=True)
+    dev = lambda k: sd[k].to(DEV)
+    gt = {k: (v.detach() if torch.is_tensor(v) else v) for k, v in gt.items()}
+    h0 = gt["hidden_states_embedding"].to(DEV)
+    ln1 = ops.layer_norm(h0, dev("transformer.layer0.input_layernorm.weight"), dev("transformer.layer0.input_layernorm.bias"), 1e-5)
+    assert float((ln1.cpu() - gt["hidden_states_input_layernorm"]).abs().max()) < 1e-5
+    att = gt["hidden_states_attention"].to(DEV)
+    ln2 = ops.layer_norm(att, dev("transformer.layer0.post_attention_layernorm.weight"),
+                         dev("transformer.layer0.post_attention_layernorm.bias"), 1e-5)
+    assert float((ln2.cpu() - gt["hidden_states_post_attention_layernorm"]).abs().max()) < 1e-4
+    # mlp block: residual + dense_out(gelu(dense_in(ln2)))
+    h = torch.nn.functional.linear(ln2, dev("transformer.layer0.mlp.dense_h_to_4h.weight"), dev("transformer.layer0.mlp.dense_h_to_4h.bias"))
+    h = torch.nn.functional.linear(ops.gelu(h), dev("transformer.layer0.mlp.dense_4h_to_h.weight"), dev("transformer.layer0.mlp.dense_4h_to_h.bias"))
+    assert float(((att + h).cpu() - gt["hidden_states_mlp"]).abs().max()) < 1e-4
+    fin = ops.layer_norm(gt["hidden_states_layer0"].to(DEV), dev("transformer.norm.weight"), dev("transformer.norm.bias"), 1e-5)
+    assert float((fin.cpu() - gt["hidden_states_norm"]).abs().max()) < 1e-3

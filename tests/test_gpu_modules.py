@@ -26,8 +26,8 @@ def _arch(**kw):
 
 def _spec(cfg, dtype):
     return oracle.LayerSpec(hidden_size=cfg.hidden_size, num_attention_heads=cfg.num_attention_heads,
-                            num_kv_heads=cfg.attention_num_kv_heads, qkv_in_one=cfg.attention_qkv_in_one, norm_type="rms",
-                            mlp_type="swiglu", layernorm_epsilon=cfg.layernorm.layernorm_epsilon,
+                            num_kv_heads=cfg.attention_num_kv_heads, qkv_in_one=cfg.attention_qkv_in_one,
+                            norm_type=cfg.norm_type.value, mlp_type=cfg.mlp_type.value, layernorm_epsilon=cfg.layernorm.layernorm_epsilon,
                             rotary_base=cfg.rotary_embedding_base, sequence_length=cfg.sequence_length, causal=cfg.causal,
                             softmax_in_fp32=True, dtype=dtype)
 
@@ -67,6 +67,9 @@ def _oracle_layer(cfg, weights, x, cu, pos, dy, dtype):
     ("fused_qkv_bias", dict(attention_qkv_in_one=True, attention_bias=True, mlp_bias=True), 1, 64, ()),
     ("rotary_complex", dict(relative_position_embedding_type="rotary_complex"), 2, 64, (20,)),
     ("partial_rotary", dict(rotary_percentage=0.5), 1, 96, ()),
+    # the reference's default architecture: LayerNorm + GELU MLP with biases
+    ("layernorm_gelu", dict(norm_type="layernorm", mlp_type="default", mlp_factor=4.0, attention_bias=True, mlp_bias=True), 2, 64, (50,)),
+    ("key_query_layernorm", dict(norm_type="layernorm", mlp_type="default", mlp_factor=4.0, key_query_norm=True), 1, 64, ()),
 ])
 def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
     print(f"case layer {name}", flush=True)
@@ -95,6 +98,11 @@ def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
         m = metrics(p.grad, ref[2][k])
         f = metrics(ref_o[2][k], ref[2][k], torch.bfloat16)
         print(f"[parity] {name}.d{k}: mean_rel={m['mean_rel']:.3e} (reference bf16 order {f['mean_rel']:.3e})", flush=True)
+        if k.endswith("self_attention.key.bias"):
+            # analytically zero (a constant added to every key shifts all scores of a query alike, and softmax is
+            # shift invariant): both sides hold rounding noise only, so bound its size instead of its relative error
+            assert m["finite"] and m["max_abs"] <= 2.0 * f["max_abs"] + 1e-3, (k, m, f)
+            continue
         assert m["finite"] and m["mean_rel"] <= max(1e-3, 1.25 * f["mean_rel"]), (k, m, f)
 
 

@@ -142,10 +142,11 @@ def test_unsupported_options_raise():
                               rotary_config=C.RotaryConfig(dimensions=64))
     with pytest.raises(AssertionError):
         ParallelSwiGLUMLP(10, 0.33, device=CPU)
-    with pytest.raises(NotImplementedError, match="swiglu"):
-        TransformerLayer(_arch(mlp_type="default"), 0, device=CPU)
-    with pytest.raises(NotImplementedError, match="rms"):
-        TransformerLayer(_arch(norm_type="layernorm"), 0, device=CPU)
+    # the reference's default architecture (LayerNorm + GELU MLP) builds, with the reference's parameter names
+    dflt = TransformerLayer(_arch(mlp_type="default", norm_type="layernorm", mlp_factor=4.0, mlp_bias=True), 0, device=CPU)
+    names = set(dflt.state_dict())
+    assert {"input_layernorm.weight", "input_layernorm.bias", "post_attention_layernorm.bias", "mlp.dense_in.weight",
+            "mlp.dense_in.bias", "mlp.dense_out.weight"} <= names and "mlp.siglu_weight.weight" not in names
     with pytest.raises(NotImplementedError):
         TransformerLayer(_arch(umup={"enable": True}), 0, device=CPU)
     assert RMSNorm(16, CPU).weight.tolist() == [1.0] * 16
