@@ -201,20 +201,23 @@ template <int D> struct LdsTile {
 // tracked by the explicit wait_vmcnt below instead.
 template <int D, int COUNT> struct DmaPlan {
     using T = LdsTile<D>;
-    int row[COUNT];          // source row of this lane
-    int unit_off[COUNT];     // byte offset of its 16-byte unit inside the row
-    uint32_t off[COUNT];     // byte offset from the first token of a full tile
-    int n0;
+    uint32_t off[COUNT];     // byte offset of this lane's 16 bytes from the first token of a full tile
+    int n0, lane;
 
-    __device__ __forceinline__ void init(int first_instr, int lane, int64_t tok_stride) {
+    __device__ __forceinline__ static void src_of(int n, int lane_, int& row, int& unit_off) {
+        int unit;
+        T::dma_src(n, lane_, row, unit);
+        if (D == 96 && unit >= D / 8) unit = 0;          // dead physical units of the padded row
+        unit_off = 16 * unit;
+    }
+    __device__ __forceinline__ void init(int first_instr, int lane_, int64_t tok_stride) {
         n0 = first_instr;
+        lane = lane_;
 #pragma unroll
         for (int j = 0; j < COUNT; ++j) {
-            int unit;
-            T::dma_src(n0 + j, lane, row[j], unit);
-            if (D == 96 && unit >= D / 8) unit = 0;      // dead physical units of the padded row
-            unit_off[j] = 16 * unit;
-            off[j] = (uint32_t)(row[j] * (int)tok_stride * 2 + unit_off[j]);
+            int row, unit_off;
+            src_of(n0 + j, lane, row, unit_off);
+            off[j] = (uint32_t)(row * (int)tok_stride * 2 + unit_off);
         }
     }
     __device__ __forceinline__ static void issue_one(uint32_t voff, const void* sbase, char* dst_lds) {
@@ -233,10 +236,14 @@ template <int D, int COUNT> struct DmaPlan {
         } else {
             const int first = min(tok0, last_tok);            // the lane offsets below must not be negative
             const __bf16* tile_base = base + (int64_t)first * tok_stride;
+            int l = lane;
+            asm volatile("" : "+v"(l));   // opaque: keeps this rarely used arithmetic from being hoisted out of the caller's loop
 #pragma unroll
             for (int j = 0; j < COUNT; ++j) {
-                const int r = min(row[j], last_tok - first);
-                issue_one((uint32_t)(r * (int)tok_stride * 2 + unit_off[j]), tile_base, dst + 1024 * j);
+                int row, unit_off;
+                src_of(n0 + j, l, row, unit_off);
+                const int r = min(row, last_tok - first);
+                issue_one((uint32_t)(r * (int)tok_stride * 2 + unit_off), tile_base, dst + 1024 * j);
             }
         }
     }
