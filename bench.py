@@ -33,9 +33,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, vendor figure
 # (KiB per dispatch, one counter per run), scaled by what the same counters read for a plain 1 GiB device copy
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Summary and commands: profiles/attention_fwd_bwd_gqa32x8_d128_s8192_hbm_traffic.md
 MEASURED_TRAFFIC_KIB = {
-    "attn_fwd_kernel": 2.0 * 72047 + 66562,
-    "attn_bwd_dkdv_kernel": 2.0 * 705646 + 32820,
-    "attn_bwd_dq_kernel": 2.0 * 106418 + 65537,
+    "attn_fwd_kernel": 2.0 * 72101 + 66560,
+    "attn_bwd_dkdv_kernel": 2.0 * 703245 + 32788,
+    "attn_bwd_dq_kernel": 2.0 * 106432 + 65536,
 }
 
 
