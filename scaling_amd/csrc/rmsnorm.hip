@@ -175,6 +175,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
 // One barrier per row step (both row sums travel through a double-buffered LDS slot).
 constexpr int kWideBlock = 512;     // two blocks per compute unit: one loads while the other computes
 constexpr int kWideMaxBlocks = 512;
+constexpr int kLnMaxBlocks = 512;     // partial dweight / dbias rows of the LayerNorm backward
 
 template <typename T, int TPR, int CH>
 __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T* __restrict__ x, const T* __restrict__ w,
@@ -305,7 +306,12 @@ __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T
 // dw[col] = sum_p partial[p][col]; 16 columns x 16 row groups per block, fixed summation order.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw,
-                                                                    int n_partial, int hidden) {
+                                                                    int n_partial, int hidden, T* __restrict__ dw2 = nullptr) {
+    // blockIdx.y == 1 (LayerNorm): the second set of partial rows, stored after the first, goes to dw2
+    if (blockIdx.y == 1) {
+        partial += (int64_t)n_partial * hidden;
+        dw = dw2;
+    }
     __shared__ float lds[16][17];
     const int cl = threadIdx.x % 16, pg = threadIdx.x / 16;
     const int col = blockIdx.x * 16 + cl;
@@ -603,6 +609,154 @@ __global__ __launch_bounds__(kBlock) void layernorm_bwd_kernel(const T* __restri
     for (int i = threadIdx.x; i < hidden; i += kBlock) { out_w[i] = comb_lds[i]; out_b[i] = comb_lds[hidden + i]; }
 }
 
+// Backward for wide rows, laid out like rmsnorm_bwd_wide_kernel: 512 threads per block, TPR (256 or 512)
+// threads per row, the fp32 weight in LDS, the rows of the next step in flight while this step is reduced.
+// A row step takes two block-wide reductions (the mean, then the centred sums), each through its own
+// double-buffered LDS slot, so two barriers per step.
+template <typename T, int TPR, int CH>
+__global__ __launch_bounds__(kWideBlock, 4) void layernorm_bwd_wide_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                            const T* __restrict__ dy, T* __restrict__ dx,
+                                                                            float* __restrict__ partial, int64_t n_rows,
+                                                                            int hidden, float eps) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int RPB = kWideBlock / TPR;
+    constexpr int WPR = TPR / 64;
+    extern __shared__ float comb_lds[];   // [hidden] dweight, [hidden] dbias, then [hidden] fp32 copy of the weight
+    __shared__ float part_mean[2][8];
+    __shared__ float part_sq[2][8], part_s1[2][8], part_s2[2][8];
+    float* w_lds = comb_lds + 2 * hidden;
+    const int tr = threadIdx.x % TPR;
+    const int rg = threadIdx.x / TPR;
+    const int wave = threadIdx.x >> 6;
+    const int vecs = hidden / V;
+    const float inv_h = 1.0f / (float)hidden;
+
+    float acc_w[CH][V], acc_b[CH][V];
+    for (int i = threadIdx.x; i < hidden; i += kWideBlock) w_lds[i] = Elem<T>::load1(w + i);
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < V; ++i) { acc_w[c][i] = 0.f; acc_b[c][i] = 0.f; }
+    __syncthreads();
+    const int64_t row_step = (int64_t)gridDim.x * RPB;
+    const int64_t iters = (n_rows + row_step - 1) / row_step;
+    uint4 xraw[CH], graw[CH], xnext[CH], gnext[CH];
+    auto fetch = [&](int64_t it, uint4 (&xv)[CH], uint4 (&gv)[CH]) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
+        const uint4* gr = reinterpret_cast<const uint4*>(dy + (row_ok ? row : 0) * hidden);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int v = c * TPR + tr;
+            const bool ok = row_ok && v < vecs;
+            xv[c] = ok ? xr[v] : make_uint4(0, 0, 0, 0);
+            gv[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
+        }
+    };
+    if (iters > 0) fetch(0, xraw, graw);
+    for (int64_t it = 0; it < iters; ++it) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        if (it + 1 < iters) fetch(it + 1, xnext, gnext);
+        const int par = (int)(it & 1);
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float xf[V];
+            Elem<T>::unpack(xraw[c], xf);
+#pragma unroll
+            for (int i = 0; i < V; ++i) sum += xf[i];
+        }
+        sum = group_sum<64>(sum);
+        if ((threadIdx.x & 63) == 0) part_mean[par][wave] = sum;
+        __syncthreads();
+        sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < WPR; ++j) sum += part_mean[par][WPR * rg + j];
+        const float mean = sum * inv_h;
+        float sq = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float xf[V], gf[V], wf[V];
+            Elem<T>::unpack(xraw[c], xf);
+            Elem<T>::unpack(graw[c], gf);
+            const bool live = c * TPR + tr < vecs;
+            const int v0 = (live ? c * TPR + tr : 0) * V;
+#pragma unroll
+            for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v0 + i);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const float xc = live ? xf[i] - mean : 0.f;
+                const float gw = gf[i] * wf[i];       // zero where the row or the vector is out of range
+                sq += xc * xc;
+                s1 += gw;
+                s2 += gw * xc;
+            }
+        }
+        sq = group_sum<64>(sq);
+        s1 = group_sum<64>(s1);
+        s2 = group_sum<64>(s2);
+        if ((threadIdx.x & 63) == 0) { part_sq[par][wave] = sq; part_s1[par][wave] = s1; part_s2[par][wave] = s2; }
+        __syncthreads();
+        sq = 0.f; s1 = 0.f; s2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < WPR; ++j) {
+            sq += part_sq[par][WPR * rg + j];
+            s1 += part_s1[par][WPR * rg + j];
+            s2 += part_s2[par][WPR * rg + j];
+        }
+        const float rstd = rsqrtf(sq * inv_h + eps);
+        s1 *= inv_h;
+        s2 *= inv_h * rstd;                           // mean(gw * xhat)
+        if (row_ok) {
+            uint4* dxr = reinterpret_cast<uint4*>(dx + row * hidden);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+                    float xf[V], gf[V], wf[V], o[V];
+                    Elem<T>::unpack(xraw[c], xf);
+                    Elem<T>::unpack(graw[c], gf);
+#pragma unroll
+                    for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v * V + i);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        const float xhat = (xf[i] - mean) * rstd;
+                        o[i] = rstd * (gf[i] * wf[i] - s1 - xhat * s2);
+                        acc_w[c][i] += gf[i] * xhat;
+                        acc_b[c][i] += gf[i];
+                    }
+                    dxr[v] = Elem<T>::pack(o);
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c) { xraw[c] = xnext[c]; graw[c] = gnext[c]; }
+    }
+    for (int i = threadIdx.x; i < 2 * hidden; i += kWideBlock) comb_lds[i] = 0.f;
+    __syncthreads();
+    for (int g = 0; g < RPB; ++g) {
+        if (rg == g) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        comb_lds[v * V + i] += acc_w[c][i];
+                        comb_lds[hidden + v * V + i] += acc_b[c][i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out_w = partial + (int64_t)blockIdx.x * hidden;
+    float* out_b = partial + ((int64_t)gridDim.x + blockIdx.x) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kWideBlock) { out_w[i] = comb_lds[i]; out_b[i] = comb_lds[hidden + i]; }
+}
+
 template <typename T>
 int launch_ln_fwd(const void* x, const void* w, const void* b, void* y, int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
     Plan plan;
@@ -626,27 +780,41 @@ int launch_ln_bwd(const void* x, const void* w, const void* dy, void* dx, void* 
                   int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
     Plan plan;
     if (!make_plan<T>(hidden, &plan)) return mi_fail(MI_E_SHAPE, "layernorm: hidden=%lld unsupported", (long long)hidden);
-    int blocks = bwd_blocks(n_rows, plan.tpr);
-    if (blocks > 256) blocks = 256;
+    const int64_t vecs = hidden / Elem<T>::kVec;
+    const bool wide = vecs >= 256 && vecs <= 1024 && (size_t)3 * hidden * sizeof(float) <= 159 * 1024;
+    const int wide_tpr = vecs <= 512 ? 256 : 512;
+    const int wide_rpb = kWideBlock / wide_tpr;
+    const int64_t wide_blocks = (n_rows + wide_rpb - 1) / wide_rpb;
+    int blocks = wide ? (int)(wide_blocks > kLnMaxBlocks ? kLnMaxBlocks : (wide_blocks < 1 ? 1 : wide_blocks))
+                      : bwd_blocks(n_rows, plan.tpr);
+    if (blocks > kLnMaxBlocks) blocks = kLnMaxBlocks;
     if (ws == nullptr || ws_bytes < (size_t)2 * blocks * hidden * sizeof(float))
         return mi_fail(MI_E_WORKSPACE, "layernorm_bwd: workspace needs %zu bytes, got %zu",
                        (size_t)2 * blocks * hidden * sizeof(float), ws_bytes);
-    const bool launched = dispatch_plan(plan, [&](auto tag) {
-        constexpr int TPR = decltype(tag)::TPR;
-        constexpr int CH = decltype(tag)::CH;
-        layernorm_bwd_kernel<T, TPR, CH><<<dim3(blocks), dim3(kBlock), 2 * hidden * sizeof(float), st>>>(
-            (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps);
-    });
+    bool launched = true;
+    if (wide) {
+        const int ch = (int)((vecs + wide_tpr - 1) / wide_tpr);
+        const size_t lds = 3 * hidden * sizeof(float);
+#define LN_WIDE(TPRV, CHV) layernorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kWideBlock), lds, st>>>( \
+            (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps)
+        if (wide_tpr == 256) { if (ch <= 1) LN_WIDE(256, 1); else LN_WIDE(256, 2); }
+        else LN_WIDE(512, 2);
+#undef LN_WIDE
+    } else {
+        launched = dispatch_plan(plan, [&](auto tag) {
+            constexpr int TPR = decltype(tag)::TPR;
+            constexpr int CH = decltype(tag)::CH;
+            layernorm_bwd_kernel<T, TPR, CH><<<dim3(blocks), dim3(kBlock), 2 * hidden * sizeof(float), st>>>(
+                (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps);
+        });
+    }
     if (!launched) return mi_fail(MI_E_SHAPE, "layernorm: no kernel for hidden=%lld", (long long)hidden);
     int rc = mi_check_launch("layernorm_bwd");
     if (rc != MI_OK) return rc;
     const unsigned rgrid = (unsigned)((hidden + 15) / 16);
-    rmsnorm_dw_reduce_kernel<T><<<dim3(rgrid), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw, blocks, (int)hidden);
-    rc = mi_check_launch("layernorm_dw_reduce");
-    if (rc != MI_OK || db == nullptr) return rc;
-    rmsnorm_dw_reduce_kernel<T><<<dim3(rgrid), dim3(kBlock), 0, st>>>((const float*)ws + (size_t)blocks * hidden, (T*)db, blocks,
-                                                                      (int)hidden);
-    return mi_check_launch("layernorm_db_reduce");
+    rmsnorm_dw_reduce_kernel<T><<<dim3(rgrid, db != nullptr ? 2 : 1), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw, blocks,
+                                                                                             (int)hidden, (T*)db);
+    return mi_check_launch("layernorm_dw_reduce");
 }
 
 }  // namespace
@@ -693,7 +861,7 @@ int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* 
 
 size_t mi_layernorm_bwd_workspace_bytes(int64_t n_rows, int64_t hidden) {
     (void)n_rows;
-    return (size_t)2 * 256 * (size_t)(hidden > 0 ? hidden : 0) * sizeof(float);
+    return (size_t)2 * kLnMaxBlocks * (size_t)(hidden > 0 ? hidden : 0) * sizeof(float);
 }
 
 int mi_layernorm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dweight, void* dbias,

@@ -87,17 +87,49 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const T* __restrict_
     }
 }
 
-// exact (erf) GELU, the reference's default activation (torch.nn.functional.gelu with approximate='none')
-__device__ __forceinline__ float gelu_f(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
-__device__ __forceinline__ float gelu_grad_f(float x) {
-    return 0.5f * (1.0f + erff(x * 0.7071067811865476f)) + x * 0.3989422804014327f * __expf(-0.5f * x * x);
-}
+// exact (erf) GELU, the reference's default activation (torch.nn.functional.gelu with approximate='none').
+// fp32 tensors use erff.  16-bit tensors use a branch-free form: with z = |x| / sqrt(2),
+//   0.5 * erfc(z) = 0.5 * t * (a1 + t * (a2 + t * (a3 + t * (a4 + t * a5)))) * exp(-z * z),  t = 1 / (1 + p * z)
+// (Abramowitz & Stegun 7.1.26, absolute error <= 1.5e-7 on erfc, far below half a bf16 / fp16 ulp of the
+// result), so Phi(x) = x >= 0 ? 1 - h : h needs one reciprocal and one exponential, and the same
+// exponential is the Gaussian density of the derivative.
+template <bool FAST> struct GeluMath {
+    // cdf = Phi(x), pdf_e = exp(-x * x / 2)
+    static __device__ __forceinline__ void parts(float x, float& cdf, float& pdf_e) {
+        if constexpr (FAST) {
+            const float z = fabsf(x) * 0.7071067811865476f;
+            const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+            pdf_e = __builtin_amdgcn_exp2f(x * x * -0.7213475204444817f);
+            float poly = 1.061405429f;
+            poly = poly * t - 1.453152027f;
+            poly = poly * t + 1.421413741f;
+            poly = poly * t - 0.284496736f;
+            poly = poly * t + 0.254829592f;
+            const float h = 0.5f * poly * t * pdf_e;
+            cdf = x >= 0.f ? 1.0f - h : h;
+        } else {
+            cdf = 0.5f * (1.0f + erff(x * 0.7071067811865476f));
+            pdf_e = __expf(-0.5f * x * x);
+        }
+    }
+    static __device__ __forceinline__ float value(float x) {
+        float cdf, e;
+        parts(x, cdf, e);
+        return x * cdf;
+    }
+    static __device__ __forceinline__ float grad(float x) {
+        float cdf, e;
+        parts(x, cdf, e);
+        return cdf + x * 0.3989422804014327f * e;
+    }
+};
 
 // BWD = false: y = gelu(x) (dy unused);  BWD = true: y = dy * gelu'(x)
 template <typename T, bool BWD>
 __global__ __launch_bounds__(kBlock) void gelu_kernel(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ y,
                                                        int64_t n_vec, int64_t n_elem) {
     constexpr int V = Elem<T>::kVec;
+    using G = GeluMath<sizeof(T) == 2>;
     const int64_t base = ((int64_t)blockIdx.x * kBlock) * kUnroll + threadIdx.x;
     uint4 rx[kUnroll], rd[kUnroll];
 #pragma unroll
@@ -116,14 +148,14 @@ __global__ __launch_bounds__(kBlock) void gelu_kernel(const T* __restrict__ x, c
             Elem<T>::unpack(rx[u], fx);
             if (BWD) Elem<T>::unpack(rd[u], fd);
 #pragma unroll
-            for (int i = 0; i < V; ++i) fx[i] = BWD ? fd[i] * gelu_grad_f(fx[i]) : gelu_f(fx[i]);
+            for (int i = 0; i < V; ++i) fx[i] = BWD ? fd[i] * G::grad(fx[i]) : G::value(fx[i]);
             reinterpret_cast<uint4*>(y)[v] = Elem<T>::pack(fx);
         }
     }
     if (blockIdx.x == gridDim.x - 1) {
         for (int64_t i = n_vec * V + threadIdx.x; i < n_elem; i += kBlock) {
             const float a = Elem<T>::load1(x + i);
-            Elem<T>::store1(y + i, BWD ? Elem<T>::load1(dy + i) * gelu_grad_f(a) : gelu_f(a));
+            Elem<T>::store1(y + i, BWD ? Elem<T>::load1(dy + i) * G::grad(a) : G::value(a));
         }
     }
 }
