@@ -162,6 +162,16 @@ def bandwidth_cases(steps, warmup):
     ms = time_gpu(lambda: ops.gelu_backward(a, dout), steps, warmup)
     out["gelu_bwd"] = {"ms": ms, "GBs": 3 * N * I * 2 / ms / 1e6}
     del a, gate, dout
+    rows, vocab = 4096, 128256                      # config-5 vocabulary
+    logits = (torch.randn(rows, vocab, generator=torch.Generator(device=dev).manual_seed(2), device=dev) * 2).bfloat16()
+    targets = torch.randint(0, vocab, (rows,), device=dev)
+    row_scale = torch.full((rows,), 1.0 / rows, device=dev)
+    dlogits = torch.empty_like(logits)
+    ms = time_gpu(lambda: ops.cross_entropy_forward(logits, targets), steps, warmup)
+    out["cross_entropy_fwd"] = {"ms": ms, "GBs": rows * vocab * 2 / ms / 1e6}
+    ms = time_gpu(lambda: ops.cross_entropy_forward(logits, targets, row_scale, dlogits), steps, warmup)
+    out["cross_entropy_fwd_bwd"] = {"ms": ms, "GBs": 2 * rows * vocab * 2 / ms / 1e6}
+    del logits, dlogits
     nq, nkv, d = 32, 8, 128
     qk = torch.randn(N, nq + nkv, d, generator=g).bfloat16().to(dev)
     tabs = oracle.rotary_tables(d, 8192, 500000, torch.bfloat16)

@@ -95,6 +95,22 @@ int mi_gelu_fwd(const void* x, void* y, int64_t n_elem, int dtype, void* stream)
 int mi_gelu_bwd(const void* x, const void* dy, void* dx, int64_t n_elem, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Token-level cross entropy over vocabulary rows.  Replaces transformer/model/losses/cross_entropy.py:18-32
+ * (torch.nn.functional.cross_entropy(logits.float(), target, reduction="none")) and the argmax of :84, and
+ * produces what autograd derives from them.  Per row r with target t (fp32 arithmetic on `dtype` logits):
+ *   lse = log sum_i exp(x_i),  losses[r] = lse - x_t,  argmax[r] = first index of max_i x_i,
+ *   dlogits[r][i] = row_scale[r] * (exp(x_i - lse) - [i == t])        (only when dlogits != NULL)
+ * row_scale (fp32, NULL = 1) carries loss_weight[r] / sum(loss_weights) times the upstream gradient
+ * (cross_entropy.py:30).  A target outside [0, vocab) marks an ignored row (loss 0, zero gradient; -100 is
+ * torch's ignore_index).  losses / lse / argmax / dlogits may each be NULL; dlogits may alias logits
+ * (in-place gradient for a chunked LM head).  Row strides are in elements.
+ * Algorithmic HBM bytes: n_rows*vocab*e read, plus the same written when dlogits is given.
+ * ------------------------------------------------------------------------------------------ */
+int mi_cross_entropy(const void* logits, const int64_t* targets, const float* row_scale, float* losses, float* lse,
+                     int32_t* argmax, void* dlogits, int64_t n_rows, int64_t vocab, int64_t logits_row_stride,
+                     int64_t dlogits_row_stride, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * SwiGLU activation.  Replaces core/nn/mlp.py:248-249:  out = silu(a) * gate, elementwise over
  * n_elem contiguous elements.  Backward: da = dout*gate*sig(a)*(1 + a*(1 - sig(a))), dgate = dout*silu(a).
  * Algorithmic HBM bytes: fwd 3*n_elem*e, bwd 5*n_elem*e.

@@ -30,6 +30,8 @@ Pinning status (what fixes each function independently of this file):
   swiglu (+ closed-form gradient)   F.silu; autograd vs closed form
   transformer layer, final norm     the layer golden (all 8 intermediate activations)
   cached decode                     cached == uncached invariant
+  token_losses, cross_entropy_loss  F.cross_entropy (library routine), closed forms (uniform logits -> log V,
+                                    gradient = softmax - onehot, rows of the gradient sum to 0), fp64 gradcheck
 No function is "parity unpinned".
 """
 
@@ -48,6 +50,7 @@ from .attention import (  # noqa: F401
 )
 from .rotary import RotaryTables, apply_rotary, apply_rotary_complex, rotary_tables  # noqa: F401
 from .norm import layer_norm, rms_norm  # noqa: F401
+from .loss import cross_entropy_loss, lm_head, token_losses  # noqa: F401
 from .mlp import gelu_mlp, swiglu, swiglu_grad, swiglu_mlp  # noqa: F401
 from .layer import (  # noqa: F401
     LayerSpec,

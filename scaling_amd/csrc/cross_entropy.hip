@@ -1,0 +1,410 @@
+// Token-level cross entropy over vocabulary rows for gfx950: loss, log-sum-exp, argmax and (optionally) the
+// gradient with respect to the logits in one launch.  HBM-bound: a row is read once and, when the gradient is
+// asked for, written once.
+//
+// Fast path: one 1024-thread workgroup per row keeps the whole row in registers (up to 16 x 128-bit vectors per
+// thread, i.e. 131072 16-bit or 65536 fp32 logits), so max, sum of exponentials and the gradient all come from
+// the single read.  Anything else (rows that do not fit, unaligned rows, vocab not a multiple of the vector
+// width) takes the streaming kernel, which re-reads the row for each of its three passes.
+#include "common.h"
+
+namespace {
+
+constexpr int kCeBlock = 1024;
+constexpr int kCeWaves = kCeBlock / 64;
+constexpr int kCeResident = 256;   // compute units
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct RowStats {
+    float mx;       // row maximum
+    float sum;      // sum exp(x - mx)
+    int arg;        // first index of the maximum
+};
+
+// Block-wide (max, first index of max); every thread receives the result.
+__device__ __forceinline__ void block_argmax(float& v, int& idx, float* lds_v, int* lds_i) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, MI_WAVE);
+        const int oi = __shfl_xor(idx, off, MI_WAVE);
+        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { lds_v[wave] = v; lds_i[wave] = idx; }
+    __syncthreads();
+    v = lds_v[0];
+    idx = lds_i[0];
+#pragma unroll
+    for (int w = 1; w < kCeWaves; ++w) {
+        const float ov = lds_v[w];
+        const int oi = lds_i[w];
+        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+}
+
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+    v = group_sum<64>(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds[wave] = v;
+    __syncthreads();
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kCeWaves; ++w) s += lds[w];
+    return s;
+}
+
+// 128 bits of -inf in the logits' type: a register that holds no part of the row
+template <typename T> __device__ __forceinline__ uint4 neg_inf_vec();
+template <> __device__ __forceinline__ uint4 neg_inf_vec<__bf16>() { return make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u); }
+template <> __device__ __forceinline__ uint4 neg_inf_vec<_Float16>() { return make_uint4(0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u); }
+template <> __device__ __forceinline__ uint4 neg_inf_vec<float>() { return make_uint4(0xff800000u, 0xff800000u, 0xff800000u, 0xff800000u); }
+
+// Keeps the three passes from sharing one unpacked fp32 copy of the row (it would need eight times the registers):
+// after this the compiler knows nothing about the value.
+__device__ __forceinline__ void forget(uint4& u) { asm volatile("" : "+v"(u.x), "+v"(u.y), "+v"(u.z), "+v"(u.w)); }
+
+struct CeArgs {
+    const void* logits;
+    const int64_t* targets;
+    const float* row_scale;    // nullable: gradient scale per row (loss weight / sum of weights), 1 when null
+    float* losses;             // nullable
+    float* lse;                // nullable
+    int32_t* argmax;           // nullable
+    void* dlogits;             // nullable, may alias logits
+    int64_t logits_stride, dlogits_stride;
+    int vocab;
+};
+
+// Finishes a row once max / sum are known: scalar outputs by thread 0, returns (lse, scale) for the gradient.
+template <typename T>
+__device__ __forceinline__ void row_outputs(const CeArgs& a, int64_t row, const RowStats& st, int64_t target, bool ignored,
+                                            float x_target, float& lse, float& scale) {
+    lse = st.mx + __builtin_amdgcn_logf(st.sum) * kLn2;
+    scale = ignored ? 0.f : (a.row_scale != nullptr ? a.row_scale[row] : 1.0f);
+    if (threadIdx.x == 0) {
+        if (a.losses != nullptr) a.losses[row] = ignored ? 0.f : lse - x_target;
+        if (a.lse != nullptr) a.lse[row] = lse;
+        if (a.argmax != nullptr) a.argmax[row] = st.arg;
+    }
+    (void)target;
+}
+
+template <typename T, int NV>
+__global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_rows) {
+    constexpr int V = Elem<T>::kVec;
+    // reduction slots, double-buffered by row parity so that one barrier per row is enough
+    __shared__ float lds_m[2][kCeWaves], lds_s[2][kCeWaves];
+    __shared__ int lds_i[2][kCeWaves];
+    const int vecs = a.vocab / V;
+    const int wave = threadIdx.x >> 6;
+    const bool lane0 = (threadIdx.x & 63) == 0;
+
+    // A workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ...  The vectors of the next row are requested
+    // as soon as the gradient pass over the current row has consumed the register they land in, so the read of
+    // row r + 1 (and the write of row r) overlap the arithmetic of row r.  Registers past the end of the row are
+    // never loaded and stay at -inf, which every pass treats as "no element" (max ignores it, exp gives 0).
+    uint4 raw[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) raw[j] = neg_inf_vec<T>();
+    auto row_ptr = [&](int64_t r) { return reinterpret_cast<const T*>(a.logits) + r * a.logits_stride; };
+    auto load_vec = [&](int64_t r, int j) {
+        const int v = j * kCeBlock + threadIdx.x;
+        if (v < vecs) raw[j] = reinterpret_cast<const uint4*>(row_ptr(r))[v];
+    };
+    auto load_target = [&](int64_t r, int64_t& target, bool& ignored, float& x_target) {
+        target = a.targets[r];
+        ignored = target < 0 || target >= a.vocab;
+        x_target = ignored ? 0.f : Elem<T>::load1(row_ptr(r) + target);   // read before an in-place gradient overwrites it
+    };
+    auto emit_argmax = [&](int64_t r, int par) {      // thread 0, after a barrier that follows the slot writes
+        if (a.argmax == nullptr) return;
+        int best = lds_i[par][0];
+#pragma unroll
+        for (int w = 1; w < kCeWaves; ++w) best = min(best, lds_i[par][w]);
+        a.argmax[r] = best;
+    };
+
+    int64_t row = blockIdx.x;
+    if (row >= n_rows) return;
+    int64_t target, target_next = 0;
+    bool ignored, ignored_next = true;
+    float x_target, x_target_next = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) load_vec(row, j);
+    load_target(row, target, ignored, x_target);
+
+    int par = 0;
+    int64_t prev_row = -1;
+    for (; row < n_rows; row += gridDim.x, par ^= 1) {
+        const int64_t next = row + gridDim.x;
+        const bool has_next = next < n_rows;
+        if (has_next) load_target(next, target_next, ignored_next, x_target_next);
+        // pass 1: this thread's maximum
+        float mt = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            float f[V];
+            forget(raw[j]);
+            Elem<T>::unpack(raw[j], f);
+#pragma unroll
+            for (int i = 0; i < V; ++i) mt = fmaxf(mt, f[i]);
+            __builtin_amdgcn_sched_barrier(0);    // one vector at a time: unpacking ahead only costs registers
+        }
+        // pass 2: this thread's sum of exponentials relative to its own maximum
+        const float mt2 = (mt == -INFINITY ? 0.f : mt) * kLog2e;
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            float f[V];
+            forget(raw[j]);
+            Elem<T>::unpack(raw[j], f);
+#pragma unroll
+            for (int i = 0; i < V; i += 2) {
+                s0 += __builtin_amdgcn_exp2f(f[i] * kLog2e - mt2);
+                s1 += __builtin_amdgcn_exp2f(f[i + 1] * kLog2e - mt2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // merge (maximum, sum) pairs: wavefront, then block
+        float wm = mt;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) wm = fmaxf(wm, __shfl_xor(wm, off, MI_WAVE));
+        float ws = (mt == -INFINITY) ? 0.f : (s0 + s1) * __builtin_amdgcn_exp2f((mt - wm) * kLog2e);
+        ws = group_sum<64>(ws);
+        if (lane0) { lds_m[par][wave] = wm; lds_s[par][wave] = ws; }
+        __syncthreads();
+        if (threadIdx.x == 0 && prev_row >= 0) emit_argmax(prev_row, par ^ 1);   // slots of the previous row are complete
+        float mx = lds_m[par][0];
+#pragma unroll
+        for (int w = 1; w < kCeWaves; ++w) mx = fmaxf(mx, lds_m[par][w]);
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < kCeWaves; ++w) {
+            const float m_w = lds_m[par][w];
+            sum += (m_w == -INFINITY) ? 0.f : lds_s[par][w] * __builtin_amdgcn_exp2f((m_w - mx) * kLog2e);
+        }
+        // first position of the maximum: only the few threads that hold it look, and they re-read their vectors
+        // from memory (cache-hot, not yet overwritten) instead of walking the register copy a fourth time
+        int arg = 0x7fffffff;
+        if (mt == mx) {
+            const uint4* xr = reinterpret_cast<const uint4*>(row_ptr(row));
+#pragma unroll 1
+            for (int v = threadIdx.x; v < vecs && arg == 0x7fffffff; v += kCeBlock) {
+                float f[V];
+                Elem<T>::unpack(xr[v], f);
+#pragma unroll
+                for (int i = V - 1; i >= 0; --i)
+                    if (f[i] == mx) arg = v * V + i;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) arg = min(arg, __shfl_xor(arg, off, MI_WAVE));
+        if (lane0) lds_i[par][wave] = arg;
+
+        const float lse = mx + __builtin_amdgcn_logf(sum) * kLn2;
+        const float scale = ignored ? 0.f : (a.row_scale != nullptr ? a.row_scale[row] : 1.0f);
+        if (threadIdx.x == 0) {
+            if (a.losses != nullptr) a.losses[row] = ignored ? 0.f : lse - x_target;
+            if (a.lse != nullptr) a.lse[row] = lse;
+        }
+        // pass 3: gradient; the thread that stores the vector holding the target patches that element right
+        // after (two stores of one thread to one address keep their order)
+        T* dx = reinterpret_cast<T*>(a.dlogits) + row * a.dlogits_stride;
+        const float l2 = lse * kLog2e;
+        const int v_target = ignored ? -1 : (int)(target / V);
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int v = j * kCeBlock + threadIdx.x;
+            if (v < vecs) {
+                float f[V];
+                forget(raw[j]);
+                Elem<T>::unpack(raw[j], f);
+#pragma unroll
+                for (int i = 0; i < V; ++i) f[i] = __builtin_amdgcn_exp2f(f[i] * kLog2e - l2) * scale;
+                reinterpret_cast<uint4*>(dx)[v] = Elem<T>::pack(f);
+                if (v == v_target)
+                    Elem<T>::store1(dx + target, (__builtin_amdgcn_exp2f(x_target * kLog2e - l2) - 1.0f) * scale);
+            }
+            if (has_next) load_vec(next, j);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        prev_row = row;
+        target = target_next;
+        ignored = ignored_next;
+        x_target = x_target_next;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) emit_argmax(prev_row, par ^ 1);
+}
+
+// Forward only (no gradient asked for): nothing of the row has to be kept, so each thread streams its vectors
+// once with a running (max, sum) pair and the pairs are merged at the end.  256 threads per row and several
+// rows per compute unit keep loads in flight under the arithmetic.
+constexpr int kFwdBlock = 256;
+constexpr int kFwdDepth = 4;        // vectors in flight per thread
+
+template <typename T>
+__global__ __launch_bounds__(kFwdBlock) void ce_fwd_kernel(const CeArgs a) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int NW = kFwdBlock / 64;
+    __shared__ float lds_m[NW], lds_s[NW];
+    __shared__ int lds_i[NW];
+    const int64_t row = blockIdx.x;
+    const T* x = reinterpret_cast<const T*>(a.logits) + row * a.logits_stride;
+    const uint4* xr = reinterpret_cast<const uint4*>(x);
+    const int vecs = a.vocab / V;
+    const int64_t target = a.targets[row];
+    const bool ignored = target < 0 || target >= a.vocab;
+    const float x_target = ignored ? 0.f : Elem<T>::load1(x + target);
+
+    float m = -INFINITY, s = 0.f;     // running maximum (natural units) and sum of exp(x - m)
+    uint4 buf[kFwdDepth];
+#pragma unroll
+    for (int d = 0; d < kFwdDepth; ++d) {
+        const int v = threadIdx.x + d * kFwdBlock;
+        buf[d] = v < vecs ? xr[v] : neg_inf_vec<T>();
+    }
+    for (int v0 = threadIdx.x; v0 < vecs; v0 += kFwdDepth * kFwdBlock) {
+#pragma unroll
+        for (int d = 0; d < kFwdDepth; ++d) {
+            float f[V];
+            Elem<T>::unpack(buf[d], f);
+            const int vn = v0 + (d + kFwdDepth) * kFwdBlock;
+            buf[d] = vn < vecs ? xr[vn] : neg_inf_vec<T>();
+            float vm = f[0];
+#pragma unroll
+            for (int i = 1; i < V; ++i) vm = fmaxf(vm, f[i]);
+            if (vm > m) {             // rare after the first vectors
+                s *= __builtin_amdgcn_exp2f((m - vm) * kLog2e);
+                m = vm;
+            }
+            const float m2 = m * kLog2e;
+            if (m > -INFINITY) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) s += __builtin_amdgcn_exp2f(f[i] * kLog2e - m2);
+            }
+        }
+    }
+    // merge the (m, s) pairs of the block
+    float bm = m;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) bm = fmaxf(bm, __shfl_xor(bm, off, MI_WAVE));
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds_m[wave] = bm;
+    __syncthreads();
+    bm = lds_m[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) bm = fmaxf(bm, lds_m[w]);
+    float part = (m > -INFINITY) ? s * __builtin_amdgcn_exp2f((m - bm) * kLog2e) : 0.f;
+    part = group_sum<64>(part);
+    if ((threadIdx.x & 63) == 0) lds_s[wave] = part;
+    // first position of the maximum: the threads whose running maximum equals it re-read their vectors
+    int arg = 0x7fffffff;
+    if (m == bm) {
+#pragma unroll 1
+        for (int v = threadIdx.x; v < vecs && arg == 0x7fffffff; v += kFwdBlock) {
+            float f[V];
+            Elem<T>::unpack(xr[v], f);
+#pragma unroll
+            for (int i = V - 1; i >= 0; --i)
+                if (f[i] == bm) arg = v * V + i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) arg = min(arg, __shfl_xor(arg, off, MI_WAVE));
+    if ((threadIdx.x & 63) == 0) lds_i[wave] = arg;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float sum = 0.f;
+        int best = 0x7fffffff;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) { sum += lds_s[w]; best = min(best, lds_i[w]); }
+        const float lse = bm + __builtin_amdgcn_logf(sum) * kLn2;
+        if (a.losses != nullptr) a.losses[row] = ignored ? 0.f : lse - x_target;
+        if (a.lse != nullptr) a.lse[row] = lse;
+        if (a.argmax != nullptr) a.argmax[row] = best;
+    }
+}
+
+// Any vocabulary size, stride and alignment: three passes over the row with scalar accesses.
+template <typename T>
+__global__ __launch_bounds__(kCeBlock) void ce_stream_kernel(const CeArgs a) {
+    __shared__ float lds_v[kCeWaves];
+    __shared__ int lds_i[kCeWaves];
+    __shared__ float lds_s[kCeWaves];
+    const int64_t row = blockIdx.x;
+    const T* x = reinterpret_cast<const T*>(a.logits) + row * a.logits_stride;
+    const int64_t target = a.targets[row];
+    const bool ignored = target < 0 || target >= a.vocab;
+    const float x_target = ignored ? 0.f : Elem<T>::load1(x + target);
+    float mx = -INFINITY;
+    int arg = 0x7fffffff;
+    for (int i = threadIdx.x; i < a.vocab; i += kCeBlock) {
+        const float f = Elem<T>::load1(x + i);
+        if (f > mx) { mx = f; arg = i; }
+    }
+    block_argmax(mx, arg, lds_v, lds_i);
+    const float m2 = mx * kLog2e;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < a.vocab; i += kCeBlock) sum += __builtin_amdgcn_exp2f(Elem<T>::load1(x + i) * kLog2e - m2);
+    sum = block_sum(sum, lds_s);
+    RowStats st{mx, sum, arg};
+    float lse, scale;
+    row_outputs<T>(a, row, st, target, ignored, x_target, lse, scale);
+    if (a.dlogits == nullptr) return;
+    T* dx = reinterpret_cast<T*>(a.dlogits) + row * a.dlogits_stride;
+    const float l2 = lse * kLog2e;
+    for (int i = threadIdx.x; i < a.vocab; i += kCeBlock) {
+        const float p = __builtin_amdgcn_exp2f(Elem<T>::load1(x + i) * kLog2e - l2);
+        Elem<T>::store1(dx + i, (p - ((int64_t)i == target ? 1.0f : 0.f)) * scale);
+    }
+}
+
+template <typename T>
+int launch_ce(const CeArgs& a, int64_t n_rows, hipStream_t st) {
+    constexpr int V = Elem<T>::kVec;
+    const bool vec_ok = a.vocab % V == 0 && a.logits_stride % V == 0 && mi_aligned16(a.logits) &&
+                        (a.dlogits == nullptr || (a.dlogits_stride % V == 0 && mi_aligned16(a.dlogits)));
+    const int64_t vecs = a.vocab / V;
+    const int nv = (int)((vecs + kCeBlock - 1) / kCeBlock);
+    const dim3 grid((unsigned)n_rows), block(kCeBlock);
+    if (vec_ok && a.dlogits == nullptr) {
+        ce_fwd_kernel<T><<<grid, dim3(kFwdBlock), 0, st>>>(a);
+    } else if (vec_ok && nv <= 16) {
+        // one resident workgroup per compute unit, each walking its share of the rows
+        const dim3 pgrid((unsigned)(n_rows < kCeResident ? n_rows : kCeResident));
+        const int nr = (int)n_rows;
+        if (nv <= 1) ce_row_kernel<T, 1><<<pgrid, block, 0, st>>>(a, nr);
+        else if (nv <= 2) ce_row_kernel<T, 2><<<pgrid, block, 0, st>>>(a, nr);
+        else if (nv <= 4) ce_row_kernel<T, 4><<<pgrid, block, 0, st>>>(a, nr);
+        else if (nv <= 8) ce_row_kernel<T, 8><<<pgrid, block, 0, st>>>(a, nr);
+        else ce_row_kernel<T, 16><<<pgrid, block, 0, st>>>(a, nr);
+    } else {
+        ce_stream_kernel<T><<<grid, block, 0, st>>>(a);
+    }
+    return mi_check_launch("cross_entropy");
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi_cross_entropy(const void* logits, const int64_t* targets, const float* row_scale, float* losses, float* lse,
+                     int32_t* argmax, void* dlogits, int64_t n_rows, int64_t vocab, int64_t logits_row_stride,
+                     int64_t dlogits_row_stride, int dtype, void* stream) {
+    if (!logits || !targets) return mi_fail(MI_E_NULL, "cross_entropy: null pointer");
+    if (n_rows < 0 || vocab <= 0 || vocab > 0x7fffffffLL)
+        return mi_fail(MI_E_SHAPE, "cross_entropy: bad shape [%lld, %lld]", (long long)n_rows, (long long)vocab);
+    if (n_rows > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "cross_entropy: too many rows");
+    if (logits_row_stride < vocab || (dlogits != nullptr && dlogits_row_stride < vocab))
+        return mi_fail(MI_E_SHAPE, "cross_entropy: row stride smaller than the vocabulary");
+    if (n_rows == 0) return MI_OK;
+    CeArgs a;
+    a.logits = logits; a.targets = targets; a.row_scale = row_scale; a.losses = losses; a.lse = lse; a.argmax = argmax;
+    a.dlogits = dlogits; a.logits_stride = logits_row_stride; a.dlogits_stride = dlogits_row_stride; a.vocab = (int)vocab;
+    MI_DISPATCH_DTYPE(dtype, return launch_ce<T>(a, n_rows, (hipStream_t)stream));
+    return MI_OK;
+}
+
+}  // extern "C"

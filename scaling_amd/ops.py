@@ -18,6 +18,7 @@ from ._lib import MiAttnArgs, MiAttnBwdArgs, MiDecodeArgs, check, dtype_code, pt
 __all__ = [
     "rms_norm", "swiglu", "rotary_embedding", "rotary_embedding_complex", "attention", "attention_forward", "attention_backward",
     "decode_attention", "rms_norm_forward", "rms_norm_backward", "swiglu_forward", "swiglu_backward",
+    "cross_entropy", "cross_entropy_forward", "linear_cross_entropy",
 ]
 
 
@@ -278,6 +279,105 @@ def rotary_embedding_complex(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tens
                              position_ids: Optional[torch.Tensor] = None, seq_len_for_null_ids: int = 0) -> torch.Tensor:
     """Interleaved-pair rotary on x [tokens, heads, head_dim]; cos / sin fp32 [rows, head_dim/2]."""
     return _RotaryComplex.apply(x, cos, sin, position_ids, seq_len_for_null_ids)
+
+
+# ------------------------------------------------------------------------------------------------
+# cross entropy over vocabulary rows
+# ------------------------------------------------------------------------------------------------
+def cross_entropy_forward(logits: torch.Tensor, targets: torch.Tensor, row_scale: Optional[torch.Tensor] = None,
+                          dlogits: Optional[torch.Tensor] = None, want_lse: bool = False):
+    """One launch over logits [rows, vocab]: returns (losses fp32 [rows], argmax int32 [rows]) (+ lse if asked).
+
+    With ``dlogits`` (same shape and dtype, may be ``logits`` itself) the gradient
+    ``row_scale[r] * (softmax(x_r) - onehot(t_r))`` is written in the same pass."""
+    _need_cuda(logits, targets, row_scale, dlogits)
+    assert logits.dim() == 2 and logits.stride(1) == 1, "logits must be [rows, vocab] with contiguous vocab"
+    assert targets.dtype == torch.int64 and targets.is_contiguous() and targets.numel() == logits.shape[0]
+    if row_scale is not None:
+        assert row_scale.dtype == torch.float32 and row_scale.is_contiguous() and row_scale.numel() == logits.shape[0]
+    if dlogits is not None:
+        assert dlogits.shape == logits.shape and dlogits.dtype == logits.dtype and dlogits.stride(1) == 1
+    n, v = logits.shape
+    losses = torch.empty(n, dtype=torch.float32, device=logits.device)
+    argmax = torch.empty(n, dtype=torch.int32, device=logits.device)
+    lse = torch.empty(n, dtype=torch.float32, device=logits.device) if want_lse else None
+    check(_lib.load().mi_cross_entropy(ptr(logits), ptr(targets), ptr(row_scale), ptr(losses), ptr(lse), ptr(argmax), ptr(dlogits),
+                                       n, v, logits.stride(0), dlogits.stride(0) if dlogits is not None else 0,
+                                       dtype_code(logits.dtype), stream_ptr()), "mi_cross_entropy")
+    return (losses, argmax, lse) if want_lse else (losses, argmax)
+
+
+class _CrossEntropy(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, targets):
+        losses, argmax = cross_entropy_forward(logits, targets)
+        ctx.save_for_backward(logits, targets)
+        ctx.mark_non_differentiable(argmax)
+        return losses, argmax
+
+    @staticmethod
+    def backward(ctx, dlosses, _dargmax):
+        logits, targets = ctx.saved_tensors
+        dlogits = torch.empty_like(logits)
+        cross_entropy_forward(logits, targets, row_scale=dlosses.float().contiguous(), dlogits=dlogits)
+        return dlogits, None
+
+
+def cross_entropy(logits: torch.Tensor, targets: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Differentiable per-row losses (fp32) and the row argmax (int32) of logits [rows, vocab]."""
+    if logits.stride(1) != 1:
+        logits = logits.contiguous()
+    return _CrossEntropy.apply(logits, targets.contiguous())
+
+
+class _LinearCrossEntropy(torch.autograd.Function):
+    """loss = sum_r w_r * CE(h_r W^T, t_r) / sum_r w_r without ever holding the [rows, vocab] logits: rows are
+    processed in chunks, each chunk's logits become its gradient in place and are folded into dh / dW at once."""
+
+    @staticmethod
+    def forward(ctx, h, weight, targets, loss_weights, chunk_rows):
+        n = h.shape[0]
+        w32 = loss_weights.float().contiguous()
+        total = w32.sum()
+        row_scale = (w32 / total).contiguous()
+        need_dh, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        dh = torch.empty_like(h) if need_dh else None
+        dw = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device) if need_dw else None
+        losses = torch.empty(n, dtype=torch.float32, device=h.device)
+        argmax = torch.empty(n, dtype=torch.int32, device=h.device)
+        for r0 in range(0, n, chunk_rows):
+            r1 = min(n, r0 + chunk_rows)
+            logits = torch.matmul(h[r0:r1], weight.t())                       # PyTorch GEMM, [chunk, vocab]
+            grad_buf = logits if (need_dh or need_dw) else None
+            lc, ac = cross_entropy_forward(logits, targets[r0:r1], row_scale=row_scale[r0:r1], dlogits=grad_buf)
+            losses[r0:r1] = lc
+            argmax[r0:r1] = ac
+            if need_dh:
+                torch.matmul(logits, weight, out=dh[r0:r1])
+            if need_dw:
+                dw.add_(torch.matmul(logits.t(), h[r0:r1]))                   # chunk product, accumulated in fp32
+        loss = (losses * w32).sum() / total
+        ctx.save_for_backward(dh if need_dh else torch.empty(0), dw if need_dw else torch.empty(0))
+        ctx.flags = (need_dh, need_dw, weight.dtype)
+        ctx.mark_non_differentiable(argmax)
+        return loss, argmax
+
+    @staticmethod
+    def backward(ctx, dloss, _dargmax):
+        dh, dw = ctx.saved_tensors
+        need_dh, need_dw, wdtype = ctx.flags
+        return (dh * dloss.to(dh.dtype) if need_dh else None, (dw * dloss).to(wdtype) if need_dw else None, None, None, None)
+
+
+def linear_cross_entropy(h: torch.Tensor, weight: torch.Tensor, targets: torch.Tensor, loss_weights: torch.Tensor,
+                         chunk_rows: int = 2048) -> Tuple[torch.Tensor, torch.Tensor]:
+    """LM head + weighted cross entropy, chunked over rows.  h [rows, hidden], weight [vocab, hidden].
+
+    Returns (loss, argmax int32 [rows]); the gradients of h and weight are computed in the forward pass."""
+    _need_cuda(h, weight, targets, loss_weights)
+    assert h.dim() == 2 and weight.dim() == 2 and h.shape[1] == weight.shape[1] and h.dtype == weight.dtype
+    return _LinearCrossEntropy.apply(h.contiguous(), weight, targets.contiguous().view(-1), loss_weights.contiguous().view(-1),
+                                     int(chunk_rows))
 
 
 # ------------------------------------------------------------------------------------------------

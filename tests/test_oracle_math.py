@@ -223,3 +223,39 @@ def test_cached_generation_equals_uncached():
     tok_c, log_c = oracle.generate_cached(spec, model, prompt, 6)
     assert tok_u == tok_c
     assert torch.allclose(log_u, log_c, atol=1e-5)
+
+
+# ---- LM head + cross entropy (losses/cross_entropy.py:18-32, 58-88) -----------------------------------------
+def test_cross_entropy_oracle_against_library_and_closed_forms():
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn(3, 17, 50, generator=g, dtype=torch.float64)
+    targets = torch.randint(0, 50, (3, 17), generator=g)
+    weights = torch.rand(3, 17, generator=g, dtype=torch.float64)
+    weights[0, :5] = 0
+    loss, m = oracle.cross_entropy_loss(logits, targets, weights)
+    lib = torch.nn.functional.cross_entropy(logits.reshape(-1, 50), targets.flatten(), reduction="none")
+    assert torch.allclose(oracle.token_losses(logits.reshape(-1, 50), targets.flatten()), lib, rtol=1e-12)
+    assert torch.allclose(loss, (lib * weights.flatten()).sum() / weights.sum(), rtol=1e-12)
+    hits = (logits.reshape(-1, 50).argmax(-1) == targets.flatten()).double()
+    mask = (weights.flatten() > 0).double()
+    assert torch.allclose(m["accuracy"], (hits * mask).sum() / mask.sum())
+    # uniform logits -> log V; a dominant target logit -> 0; ignore_index rows -> 0
+    assert torch.allclose(oracle.token_losses(torch.zeros(2, 1000, dtype=torch.float64), torch.tensor([3, 9])),
+                          torch.full((2,), math.log(1000.0), dtype=torch.float64))
+    peaked = torch.zeros(1, 10, dtype=torch.float64)
+    peaked[0, 4] = 100.0
+    assert float(oracle.token_losses(peaked, torch.tensor([4]))) < 1e-12
+    assert float(oracle.token_losses(torch.randn(1, 10, dtype=torch.float64), torch.tensor([-100]))) == 0.0
+    # gradient closed form: d loss / d logits = w / sum(w) * (softmax - onehot); every row sums to zero
+    x = logits.clone().requires_grad_()
+    oracle.cross_entropy_loss(x, targets, weights)[0].backward()
+    p = torch.softmax(logits.reshape(-1, 50), -1)
+    p[torch.arange(51), targets.flatten()] -= 1.0
+    want = (p * (weights.flatten() / weights.sum()).unsqueeze(-1)).reshape(3, 17, 50)
+    assert torch.allclose(x.grad, want, rtol=1e-10, atol=1e-14)
+    assert float(x.grad.sum(-1).abs().max()) < 1e-15
+    small = torch.randn(4, 6, dtype=torch.float64, generator=g).requires_grad_()
+    assert torch.autograd.gradcheck(lambda z: oracle.cross_entropy_loss(z, torch.tensor([0, 5, 2, 2]), torch.tensor([1.0, 0.5, 0.0, 2.0]))[0], (small,))
+    # the head is a bias-free projection with weight [vocab, hidden]
+    h, w = torch.randn(5, 8, dtype=torch.float64, generator=g), torch.randn(11, 8, dtype=torch.float64, generator=g)
+    assert torch.allclose(oracle.lm_head(h, w), h @ w.t())
