@@ -9,8 +9,9 @@
 //   3. dQ: a workgroup owns 256 queries of one head (32 per wavefront, Q and dO fragments in registers),
 //      loops over 64-key tiles:  S^T = K Q^T, dP^T = V dO^T, dS^T, dQ^T += K^T dS^T.
 // Tiles whose rows are needed both as row operands and transposed (Q / dO in kernel 2, K in kernel 3) are
-// staged once, token-major, in a layout that serves plain 128-bit reads and LDS transpose reads without
-// bank conflicts (TokTile in attn_common.h); score tiles are consumed in their accumulator layout.
+// loaded once, global -> LDS directly, token-major, in a swizzled layout that serves plain 128-bit reads and
+// LDS transpose reads without bank conflicts (LdsTile in attn_common.h); score tiles are consumed in their
+// accumulator layout.
 #include "attn_common.h"
 
 namespace {

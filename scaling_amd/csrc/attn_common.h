@@ -103,52 +103,6 @@ __device__ __forceinline__ bf16x8_t tr_pair(const char* lo_addr, const char* hi_
     return __builtin_bit_cast(bf16x8_t, both);
 }
 
-// Plain token-major tile (stride = 64 mod 256 bytes) that is only read transposed.
-// lane_base = tr_lane_base(lane, stride); chunk m, feature tile dt: see tr_operand.
-__device__ __forceinline__ int tr_lane_base(int lane, int stride_bytes) {
-    const int g = lane >> 5, i = lane & 15, blk = (lane >> 4) & 1;
-    return (4 * g + (i >> 2)) * stride_bytes + (16 * blk + 4 * (i & 3)) * 2;
-}
-
-__device__ __forceinline__ bf16x8_t tr_operand(const char* tile, int lane_base, int stride_bytes, int m, int dt) {
-    return tr_pair(tile + lane_base + (16 * m) * stride_bytes + 64 * dt,
-                   tile + lane_base + (16 * m + 8) * stride_bytes + 64 * dt);
-}
-
-// Token-major tile that is read both ways without bank conflicts: as a row operand (lane = token,
-// 16 bytes of features per k-step) and transposed (lane = feature, k-slots = tokens).  The row stride is
-// 4 or 12 (mod 16) 16-byte units and the unit index of a row is XORed with ((row >> 2) & 3):
-//   row operand   16 consecutive rows at one k-step land on 16 different units (mod 16),
-//   transposed    the 4 rows x 2 x 32 bytes touched by 32 lanes land on 16 different units (mod 16),
-//   loader        the units of one row are permuted inside aligned groups of four.
-// Rows of a tile start at a multiple of 16, so the XOR term of a lane is fixed per operand.
-template <int D> struct TokTile {
-    static constexpr int kStride = (D == 128) ? 320 : (D == 32 ? 64 : 192);   // bytes per token
-    static_assert(D == 32 || D == 64 || D == 96 || D == 128, "head_dim");
-
-    // byte offset of 16-byte unit c of row r (loader side)
-    static __device__ __forceinline__ int unit_offset(int r, int c) {
-        return r * kStride + ((c ^ ((r >> 2) & 3)) << 4);
-    }
-    // row operand of lane (row, g): k-step ks is at (ks even ? even : odd) + 32 * ks
-    static __device__ __forceinline__ void row_bases(int row, int g, int& even, int& odd) {
-        const int a = (row >> 2) & 3;
-        const int rb = row * kStride + ((g ^ (a & 1)) << 4);
-        even = rb + 32 * (a >> 1);
-        odd = rb - 32 * (a >> 1);
-    }
-    // transposed operand: chunk m (16 tokens, chunk order), feature tile dt (32 features):
-    //   tr_pair(tile + h0 + 16*m*kStride + 64*dt, tile + h1 + 16*m*kStride + 64*dt)
-    static __device__ __forceinline__ void tr_bases(int lane, int& h0, int& h1) {
-        const int g = lane >> 5, i = lane & 15, blk = (lane >> 4) & 1;
-        const int row = 4 * g + (i >> 2);
-        const int u = 2 * blk + ((i >> 1) & 1);
-        const int byte = (i & 1) * 8;
-        h0 = row * kStride + ((u ^ g) << 4) + byte;
-        h1 = (row + 8) * kStride + ((u ^ (2 + g)) << 4) + byte;
-    }
-};
-
 // ---- token-major LDS tile filled by direct global -> LDS loads ------------------------------------------
 // 64 tokens, unpadded rows of UPR 16-byte units (head_dim 96 uses rows of 16 units, 12 of them live).
 // A direct load instruction writes 64 x 16 bytes to consecutive LDS addresses (lane i -> base + 16 i), so
@@ -273,17 +227,6 @@ __device__ __forceinline__ void wait_vmcnt_dyn(int n) {
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt");
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
-}
-
-// 4 tokens x 8 features held as 4 row vectors -> for feature dd the 4 token values as one 8-byte group
-__device__ __forceinline__ uint2 transpose_quad(const uint4 (&raw)[4], int dd) {
-    const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&raw[0]);
-    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&raw[1]);
-    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&raw[2]);
-    const uint32_t* w3 = reinterpret_cast<const uint32_t*>(&raw[3]);
-    const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of the two words
-    return make_uint2(__builtin_amdgcn_perm(w1[dd >> 1], w0[dd >> 1], sel),
-                      __builtin_amdgcn_perm(w3[dd >> 1], w2[dd >> 1], sel));
 }
 
 // 128-bit load / store through a native vector type.  Copying a uint4 (a struct) between address spaces

@@ -22,6 +22,7 @@ import torch.nn.functional as F
 from .config import TransformerArchitectureConfig, architecture_from_config_file
 from .data import get_cumulative_seq_lengths, get_position_ids
 from .layer import InferenceSettings, LayerNormWrapper, TransformerLayer, TransformerLayerIO
+from .loss import TransformerLMHead
 
 # class names written by older versions of the reference (partitioned_module.py:25-32)
 LEGACY_CLASS_NAMES = {"LuminousEmbeddingInput": "EmbeddingInput", "LuminousLayer": "TransformerLayer",
@@ -40,15 +41,6 @@ class EmbeddingInput(torch.nn.Module):
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         return self.embedding(token_ids)
-
-
-class TransformerLMHead(torch.nn.Module):
-    def __init__(self, cfg: TransformerArchitectureConfig, device=None):
-        super().__init__()
-        self.linear = torch.nn.Linear(cfg.hidden_size, cfg.vocab_size, bias=False, device=device, dtype=cfg.precision.dtype)
-
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.linear(x)
 
 
 class TransformerInferenceModule(torch.nn.Module):
@@ -74,7 +66,7 @@ class TransformerInferenceModule(torch.nn.Module):
         for i in range(cfg.num_layers):
             layers.append(TransformerLayer(cfg, layer_index=i, init_method=init, device=self.device))
         layers.append(LayerNormWrapper(cfg, layer_index=cfg.num_layers, device=self.device))
-        layers.append(TransformerLMHead(cfg, self.device))
+        layers.append(TransformerLMHead(cfg, device=self.device))
         self._layers = torch.nn.ModuleList(layers)
         init(self._layers[0].embedding.weight)
         if cfg.weight_tying:
@@ -138,7 +130,7 @@ class TransformerInferenceModule(torch.nn.Module):
         if last_token_only:
             x.activations = x.activations[:, -1:, :].contiguous()
         x = self._layers[-2](x)
-        return self._layers[-1](x.activations)
+        return self._layers[-1].linear(x.activations)
 
     def logits(self, input_tokens: Sequence[int]) -> torch.Tensor:
         return self.forward(torch.tensor([list(input_tokens)])).squeeze(0)
@@ -176,7 +168,7 @@ class TransformerInferenceModule(torch.nn.Module):
             h = self._layers[0](tok)
             for layer in layers:
                 h = layer.decode_step(h, pos)
-            lg = self._layers[-1](self._layers[-2].norm(h))
+            lg = self._layers[-1].linear(self._layers[-2].norm(h))
             nxt = torch.argmax(lg, dim=-1)                                # [b, 1]
             out.index_copy_(1, step, nxt)
             tok.copy_(nxt)
