@@ -202,6 +202,15 @@ typedef struct mi_attn_args {
     const int64_t* position_ids_k;
     int64_t rotary_table_rows;
     void* stream;
+    /* dropout on the attention probabilities (attention.py:204-207): 0 = off.  Element (head, query, key) is
+     * dropped iff byte(lowbias32(head_base + (query >> 1) * 0x9E3779B1 + (key >> 1) * 0x85EBCA77)
+     *                  >> (16 * (query & 1) + 8 * (key & 1))) < T,  T = round(256 * dropout_p) clamped to 1..255,
+     * head_base = lowbias32(seed32 ^ lowbias32(head * 0x9E3779B9 + 0x7F4A7C15)), seed32 = low ^ high word of
+     * dropout_seed; query / key are token indices on the flattened axes.  The effective drop probability is
+     * T / 256 and kept probabilities are scaled by 256 / (256 - T).  The backward call must pass the same values.
+     * Not available together with the fused rotary of the forward. */
+    float dropout_p;
+    uint64_t dropout_seed;
 } mi_attn_args;
 
 int mi_attn_fwd(const mi_attn_args* args);

@@ -73,17 +73,20 @@ def multi_head_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Te
                          cumulative_seq_lengths: torch.Tensor, causal: bool,
                          query_key_scaling_factor: float, softmax_in_fp32: bool = False,
                          softmax_scale: float = 1.0, dropout_p: float = 0.0,
-                         mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+                         mask: Optional[torch.Tensor] = None,
+                         dropout_keep: Optional[torch.Tensor] = None) -> torch.Tensor:
     """core/nn/attention/attention.py:108-213 with `MaskedSoftmaxTorch` as softmax_fn.
 
     query [s_q, b, n, d]; key, value [s_k, b, n, d] (kv heads already repeated).
     Returns [(b n), s_q, d].  Scores are alpha * Q K^T *in the input dtype*
     (`baddbmm`, lines 154-160), the mask comes from the query-side cumulative
     lengths with s_q as the per-item length (lines 166-168), probabilities are
-    cast to the value dtype before P V (line 211).  Attention-score
-    manipulation and dropout p > 0 are outside the restated path.
+    cast to the value dtype before P V (line 211).  Dropout (lines 204-207, torch.nn.Dropout on the
+    probabilities) is restated with an explicit keep mask `dropout_keep` [b, n, s_q, s_k] (bool) so that a
+    test can supply the mask the kernels generate: probs * keep / (1 - dropout_p).  Attention-score
+    manipulation is outside the restated path.
     """
-    assert dropout_p == 0.0, "oracle restates the deterministic path only"
+    assert (dropout_p == 0.0) == (dropout_keep is None), "dropout needs both the rate and the keep mask"
     s_q, b, n, d = query.shape
     q = query.permute(1, 2, 0, 3).reshape(b * n, s_q, d)
     k = key.permute(1, 2, 0, 3).reshape(b * n, key.shape[0], d)
@@ -96,5 +99,7 @@ def multi_head_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Te
     if mask is None:
         mask = cumulative_seq_lengths_to_dense_attention_mask(cumulative_seq_lengths, s_q, causal)
     probs = masked_softmax(scores, mask, softmax_in_fp32=softmax_in_fp32, scale=softmax_scale)
+    if dropout_keep is not None:
+        probs = probs * dropout_keep.to(probs.dtype) * (1.0 / (1.0 - dropout_p))
     probs = probs.reshape(b * n, s_q, k.shape[1])
     return torch.bmm(probs.to(v.dtype), v)

@@ -6,7 +6,7 @@ been built, or a kernel returns an error status, a RuntimeError is raised.
 
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
+from ctypes import c_uint64, POINTER, Structure, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_void_p
 
 import torch
 
@@ -42,6 +42,7 @@ class MiAttnArgs(Structure):
         ("position_ids_q", c_void_p), ("position_ids_k", c_void_p),
         ("rotary_table_rows", c_int64),
         ("stream", c_void_p),
+        ("dropout_p", c_float), ("dropout_seed", c_uint64),
     ]
 
 

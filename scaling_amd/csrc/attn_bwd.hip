@@ -52,7 +52,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_delta_kernel(const AttnPara
 // (32 of the 64 queries staged per iteration), so the pair (w, w + 4) accumulates the same dK / dV
 // rows and is summed once at the end.  The first four wavefronts stage Q, the last four dO; the staged
 // tiles are double buffered (one barrier per iteration).
-template <int D>
+template <int D, bool DROP>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
     constexpr int BNK = 128;              // keys per workgroup
     constexpr int BQ = 64;                // queries per tile
@@ -170,6 +170,12 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     const int a_row = Tile::row_base(32 * sub + l32, g);                       // Q / dO rows of this wavefront's sub-tile
     const int b_row = (kgp >> 1) * TILE + Tile::row_base(32 * (kgp & 1) + l32, g);   // its K / V rows
     const float c2 = p.scale_log2;
+    // dropout: hash input of this lane's key column at query pair 2 g, bit offset of its column of a 2 x 2 block
+    uint32_t drop_xc = 0, drop_sel = 0;
+    if constexpr (DROP) {
+        drop_xc = (uint32_t)(key >> 1) * kDropC2 + (uint32_t)(2 * g) * kDropC1;
+        drop_sel = 8u * (uint32_t)(key & 1);
+    }
 
     for (int iter = 0; iter < total_iters; ++iter) {
         const int buf = iter & 1;
@@ -204,16 +210,32 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                 }
             }
             bf16x8_t pf[2], dsf[2];
+            uint32_t drop_xb = 0;
+            if constexpr (DROP) {
+                const int head_i = kvh * p.n_rep + iter / n_tiles;
+                drop_xb = drop_head_base(p.drop_seed, head_i) + drop_xc + (uint32_t)(qs >> 1) * kDropC1;
+            }
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(&lse_lds[buf][32 * sub + 8 * a + 4 * g]);
                 const f32x4_t d4 = *reinterpret_cast<const f32x4_t*>(&delta_lds[buf][32 * sub + 8 * a + 4 * g]);
+                bool keep[4] = {true, true, true, true};
+                if constexpr (DROP) {
+                    // register 4 a + c holds query qs + 8 a + 4 g + c: two query pairs per a
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const uint32_t h = lowbias32(drop_xb + (uint32_t)(4 * a + j) * kDropC1);
+                        keep[2 * j] = drop_byte(h, drop_sel) >= p.drop_thr;
+                        keep[2 * j + 1] = drop_byte(h, drop_sel + 16) >= p.drop_thr;
+                    }
+                }
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const int r = 4 * a + c;
                     const float pv = fast_exp2(s_acc[r] * c2 - l4[c]);
-                    const float ds = pv * (dp_acc[r] - d4[c]);
-                    pf[a >> 1][4 * (a & 1) + c] = (__bf16)pv;
+                    const float dpv = DROP ? (keep[c] ? dp_acc[r] * p.drop_rscale : 0.f) : dp_acc[r];
+                    const float ds = pv * (dpv - d4[c]);
+                    pf[a >> 1][4 * (a & 1) + c] = (__bf16)((DROP && !keep[c]) ? 0.f : pv);
                     dsf[a >> 1][4 * (a & 1) + c] = (__bf16)ds;
                 }
             }
@@ -265,8 +287,9 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                 const uint32_t k0 = pack_bf16x2(dk_acc[dt][4 * a] * p.scale, dk_acc[dt][4 * a + 1] * p.scale);
                 const uint32_t k1 = pack_bf16x2(dk_acc[dt][4 * a + 2] * p.scale, dk_acc[dt][4 * a + 3] * p.scale);
                 *reinterpret_cast<uint2*>(dkr + 32 * dt + 8 * a) = make_uint2(k0, k1);
-                const uint32_t v0 = pack_bf16x2(dv_acc[dt][4 * a], dv_acc[dt][4 * a + 1]);
-                const uint32_t v1 = pack_bf16x2(dv_acc[dt][4 * a + 2], dv_acc[dt][4 * a + 3]);
+                const float vs = DROP ? p.drop_rscale : 1.0f;   // dV = (P * mask / (1 - p))^T dO
+                const uint32_t v0 = pack_bf16x2(dv_acc[dt][4 * a] * vs, dv_acc[dt][4 * a + 1] * vs);
+                const uint32_t v1 = pack_bf16x2(dv_acc[dt][4 * a + 2] * vs, dv_acc[dt][4 * a + 3] * vs);
                 *reinterpret_cast<uint2*>(dvr + 32 * dt + 8 * a) = make_uint2(v0, v1);
             }
     }
@@ -278,7 +301,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 // 8 wavefronts, two per SIMD, 32 queries each (256 per workgroup); the first four stage K (one
 // token-major tile read both as row operand and transposed), the last four stage V.  Double-buffered
 // LDS, one barrier per 64-key tile.
-template <int D>
+template <int D, bool DROP>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p) {
     constexpr int BM = 256;
     constexpr int BN = 64;
@@ -372,6 +395,12 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     int tr_h0, tr_h1;
     Tile::tr_bases(lane, tr_h0, tr_h1);
     const int a_row = Tile::row_base(l32, g);
+    // dropout: hash input of this lane's query row at key pair 2 g, bit offset of its row of a 2 x 2 block
+    uint32_t drop_xr = 0, drop_sel = 0;
+    if constexpr (DROP) {
+        drop_xr = drop_head_base(p.drop_seed, head) + (uint32_t)(tq >> 1) * kDropC1 + (uint32_t)(2 * g) * kDropC2;
+        drop_sel = 16u * (uint32_t)(tq & 1);
+    }
     for (int it = 0; it < n_tiles; ++it) {
         const int kt = kt0 + it * BN;
         issue_tile(it + 2);
@@ -411,6 +440,18 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
             for (int m = 0; m < 4; ++m) {
                 const int t = m >> 1, r0 = 8 * (m & 1);
                 bf16x8_t dsf;
+                if constexpr (DROP) {
+                    // dP of a dropped probability is zero, that of a kept one carries the 1 / (1 - p) scale
+                    const uint32_t drop_xt = drop_xr + (uint32_t)(kt >> 1) * kDropC2;
+#pragma unroll
+                    for (int pi = 0; pi < 4; ++pi) {
+                        const int a = 2 * (m & 1) + (pi >> 1), j = pi & 1;
+                        const uint32_t h = lowbias32(drop_xt + (uint32_t)(16 * t + 4 * a + j) * kDropC2);
+                        const bool keep0 = drop_byte(h, drop_sel) >= p.drop_thr, keep1 = drop_byte(h, drop_sel + 8) >= p.drop_thr;
+                        dp_acc[t][r0 + 2 * pi] = keep0 ? dp_acc[t][r0 + 2 * pi] * p.drop_rscale : 0.f;
+                        dp_acc[t][r0 + 2 * pi + 1] = keep1 ? dp_acc[t][r0 + 2 * pi + 1] * p.drop_rscale : 0.f;
+                    }
+                }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float pv = fast_exp2(s_acc[t][r0 + e] * c2 - lse2);
@@ -455,13 +496,15 @@ template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) 
     }
     if (all || (stages & MI_ATTN_BWD_DKDV)) {
         const int64_t grid = (((int64_t)p.total_k + 127) / 128) * p.nkv;
-        attn_bwd_dkdv_kernel<D><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        if (p.drop_thr != 0) attn_bwd_dkdv_kernel<D, true><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        else attn_bwd_dkdv_kernel<D, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         int rc = mi_check_launch("attn_bwd_dkdv");
         if (rc != MI_OK) return rc;
     }
     if (all || (stages & MI_ATTN_BWD_DQ)) {
         const int64_t grid = (((int64_t)p.total_q + 255) / 256) * p.nq;
-        attn_bwd_dq_kernel<D><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        if (p.drop_thr != 0) attn_bwd_dq_kernel<D, true><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        else attn_bwd_dq_kernel<D, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         return mi_check_launch("attn_bwd_dq");
     }
     return MI_OK;

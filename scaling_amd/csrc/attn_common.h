@@ -26,7 +26,33 @@ struct AttnParams {
     const __bf16* d_o; __bf16* dq; __bf16* dk; __bf16* dv; float* delta;
     int64_t dk_st, dk_sh, dv_st, dv_sh;
     float scale;        // softmax_scale
+    // dropout on the attention probabilities (0 = off): an element is dropped iff its random byte < drop_thr,
+    // kept probabilities are scaled by drop_rscale = 256 / (256 - drop_thr)
+    uint32_t drop_thr; float drop_rscale; uint32_t drop_seed;
 };
+
+// ---- dropout mask ---------------------------------------------------------------------------------------
+// The random byte of element (query q, key k) of a head is a pure function of (seed, head, q, k), so the
+// forward and both backward kernels regenerate the same mask whatever their tiling:
+//   x = head_base + (q >> 1) * C1 + (k >> 1) * C2          (mod 2^32)
+//   h = lowbias32(x)                                       (two multiply / xor-shift rounds)
+//   byte = (h >> (16 * (q & 1) + 8 * (k & 1))) & 0xff
+// One hash serves a 2 x 2 block of elements, two of which any lane of either score-tile layout holds.
+constexpr uint32_t kDropC1 = 0x9E3779B1u, kDropC2 = 0x85EBCA77u;
+
+__host__ __device__ __forceinline__ uint32_t lowbias32(uint32_t x) {
+    x ^= x >> 16; x *= 0x7FEB352Du;
+    x ^= x >> 15; x *= 0x846CA68Bu;
+    x ^= x >> 16;
+    return x;
+}
+
+__device__ __forceinline__ uint32_t drop_head_base(uint32_t seed, int head) {
+    return lowbias32(seed ^ lowbias32((uint32_t)head * 0x9E3779B9u + 0x7F4A7C15u));
+}
+
+// byte `field` (0..3) of the block hash
+__device__ __forceinline__ uint32_t drop_byte(uint32_t h, uint32_t shift) { return __builtin_amdgcn_ubfe(h, shift, 8); }
 
 __device__ __forceinline__ f32x16_t mfma_32x32x16(bf16x8_t a, bf16x8_t b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);

@@ -24,7 +24,7 @@ namespace {
 constexpr int BN = 64;               // keys per tile
 constexpr float kRescaleGap = 8.0f;  // log2 units by which a row max may lag before O is rescaled
 
-template <int D, int NW, bool ROT>
+template <int D, int NW, bool ROT, bool DROP>
 __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p) {
     constexpr int BM = 32 * NW;
     constexpr int KS = D / 16;            // contraction steps of Q K^T
@@ -215,6 +215,12 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     int v_h0, v_h1;
     Tile::tr_bases(lane, v_h0, v_h1);
     const int k_row = Tile::row_base(l32, g);
+    // dropout: hash input of this lane's query row at key pair 2 g, and the bit offset of its row of a 2 x 2 block
+    uint32_t drop_xr = 0, drop_sel = 0;
+    if constexpr (DROP) {
+        drop_xr = drop_head_base(p.drop_seed, head) + (uint32_t)(tq >> 1) * kDropC1 + (uint32_t)(2 * g) * kDropC2;
+        drop_sel = 16u * (uint32_t)(tq & 1);
+    }
     f32x16_t s_acc[2];
     bf16x8_t pf[4];
     bool pending = false;                 // pf holds the probabilities of the previous tile
@@ -323,6 +329,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
             }
             const float m_use = (m_i == -INFINITY) ? 0.f : m_i;
             float rs0 = 0.f, rs1 = 0.f;
+            const uint32_t drop_xt = drop_xr + (uint32_t)(kt >> 1) * kDropC2;   // used with DROP only
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
                 const int t = m >> 1, r0 = 8 * (m & 1);
@@ -331,6 +338,17 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                     const float ev = fast_exp2(s_acc[t][r0 + e] * c2 - m_use);
                     if (e & 1) rs1 += ev; else rs0 += ev;
                     pf[m][e] = (__bf16)ev;
+                }
+                if constexpr (DROP) {
+                    // the row sum above stays that of the full softmax; only the P that multiplies V is masked
+                    // (register r0 + e holds key kt + 32 t + 8 a + 4 g + c with 4 a + c = r0 + e)
+#pragma unroll
+                    for (int pi = 0; pi < 4; ++pi) {
+                        const int a = 2 * (m & 1) + (pi >> 1), j = pi & 1;
+                        const uint32_t h = lowbias32(drop_xt + (uint32_t)(16 * t + 4 * a + j) * kDropC2);
+                        if (drop_byte(h, drop_sel) < p.drop_thr) pf[m][2 * pi] = (__bf16)0.f;
+                        if (drop_byte(h, drop_sel + 8) < p.drop_thr) pf[m][2 * pi + 1] = (__bf16)0.f;
+                    }
                 }
             }
             l_i += rs0 + rs1;
@@ -352,7 +370,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
 
     // ---- epilogue ------------------------------------------------------------------------------
     const float l_tot = l_i + __shfl_xor(l_i, 32, 64);
-    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    const float inv = (l_tot > 0.f ? 1.0f / l_tot : 0.f) * (DROP ? p.drop_rscale : 1.0f);
     if (tq < p.total_q) {
         __bf16* orow = p.o + (int64_t)tq * p.o_st + (int64_t)head * p.o_sh + 4 * g;
 #pragma unroll
@@ -370,24 +388,28 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     }
 }
 
-template <int D, int NW, bool ROT> int launch(const AttnParams& p, hipStream_t st) {
+template <int D, int NW, bool ROT, bool DROP> int launch(const AttnParams& p, hipStream_t st) {
     constexpr int BM = 32 * NW;
     const int64_t nqb = ((int64_t)p.total_q + BM - 1) / BM;
     const int64_t grid = nqb * p.nq;
     if (grid > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_fwd: grid too large");
-    attn_fwd_kernel<D, NW, ROT><<<dim3((unsigned)grid), dim3(64 * NW), 0, st>>>(p);
+    attn_fwd_kernel<D, NW, ROT, DROP><<<dim3((unsigned)grid), dim3(64 * NW), 0, st>>>(p);
     return mi_check_launch("attn_fwd");
 }
 
 template <int D> int launch_d(const AttnParams& p, bool rot, int nw, hipStream_t st) {
+    if (p.drop_thr != 0) {               // dropout: one tiling per head_dim (256-query workgroups), no fused rotary
+        if (rot) return mi_fail(MI_E_SHAPE, "attn_fwd: dropout and fused rotary cannot be combined");
+        return launch<D, 8, false, true>(p, st);
+    }
     if (rot) {
         if constexpr (D == 64 || D == 128) {
-            return nw == 8 ? launch<D, 8, true>(p, st) : launch<D, 4, true>(p, st);
+            return nw == 8 ? launch<D, 8, true, false>(p, st) : launch<D, 4, true, false>(p, st);
         } else {
             return mi_fail(MI_E_SHAPE, "attn_fwd: fused rotary needs head_dim 64 or 128");
         }
     }
-    return nw == 8 ? launch<D, 8, false>(p, st) : launch<D, 4, false>(p, st);
+    return nw == 8 ? launch<D, 8, false, false>(p, st) : launch<D, 4, false, false>(p, st);
 }
 
 }  // namespace

@@ -26,6 +26,8 @@ int mi_attn_validate(const mi_attn_args* a, const char* who) {
         if (a->rotary_table_rows <= 0 || a->rotary_table_rows > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "%s: bad rotary table size", who);
         if (!mi_aligned16(a->rotary_cos) || !mi_aligned16(a->rotary_sin)) return mi_fail(MI_E_ALIGN, "%s: rotary tables must be 16-byte aligned", who);
     }
+    if (!(a->dropout_p >= 0.f) || a->dropout_p >= 1.f) return mi_fail(MI_E_SHAPE, "%s: dropout_p must be in [0, 1)", who);
+    if (a->dropout_p > 0.f && a->rotary_cos) return mi_fail(MI_E_SHAPE, "%s: dropout and fused rotary cannot be combined", who);
     return MI_OK;
 }
 
@@ -45,4 +47,11 @@ void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p) {
     p->scale_log2 = a->softmax_scale * 1.4426950408889634f;
     p->cos = (const __bf16*)a->rotary_cos; p->sin = (const __bf16*)a->rotary_sin;
     p->pos_q = a->position_ids_q; p->pos_k = a->position_ids_k; p->table_rows = (int)a->rotary_table_rows;
+    if (a->dropout_p > 0.f) {
+        int t = (int)(a->dropout_p * 256.0f + 0.5f);
+        t = t < 1 ? 1 : (t > 255 ? 255 : t);
+        p->drop_thr = (uint32_t)t;
+        p->drop_rscale = 256.0f / (float)(256 - t);
+        p->drop_seed = (uint32_t)(a->dropout_seed & 0xffffffffu) ^ (uint32_t)(a->dropout_seed >> 32);
+    }
 }

@@ -234,8 +234,9 @@ class ParallelSelfAttention(torch.nn.Module):
     """Mirror of core/nn/attention/attention.py:509-969 for `masked_softmax.kernel = hip`.
 
     Same constructor arguments and forward signature.  Differences, all documented errors rather than
-    silent fall-backs: attention-probability dropout, attention-score manipulation, LoRA, local
-    attention windows, u-muP and fp8 are not available;
+    silent fall-backs: attention-score manipulation, LoRA, local attention windows, u-muP and fp8 are not
+    available; attention-probability dropout is applied inside the kernels in training mode (its mask comes
+    from a counter-based hash, not from torch's generator stream, and its rate is quantised to 1/256);
     the dtype must be bfloat16.  The KV cache is pre-allocated (see `KVCache`), supports batches of
     single-document rows and is filled/extended in place.
     """
@@ -261,8 +262,8 @@ class ParallelSelfAttention(torch.nn.Module):
             raise NotImplementedError(
                 f"this module implements masked_softmax.kernel = 'hip' only (got '{masked_softmax_config.kernel.value}'); "
                 "the other kernels live in the reference implementation")
-        if dropout_attention_probs != 0.0:
-            raise NotImplementedError("dropout on attention probabilities is not available with the hip kernel")
+        assert 0.0 <= dropout_attention_probs < 1.0, "dropout_attention_probs must be in [0, 1)"
+        self.dropout_attention_probs = float(dropout_attention_probs)   # applied in training mode only
         if num_local_attention_heads > 0 or lora_config is not None or fp8_config is not None or \
                 fp8_config_dense_out is not None or bitfit_bias_name is not None:
             raise NotImplementedError("local attention, LoRA, fp8 and bitfit are outside the hip kernel's scope")
@@ -379,7 +380,8 @@ class ParallelSelfAttention(torch.nn.Module):
         if use_cache:  # prefill: keep post-rotary K and V (attention.py:861-862)
             self._fill_cache(k, v, b, s, cache_index)
         ctx = ops.attention(q, k, v, cu, None if cumulative_seq_lengths_key is None else cumulative_seq_lengths_key.to(torch.int32),
-                            self.causal, self.softmax_scale)
+                            self.causal, self.softmax_scale,
+                            dropout_p=self.dropout_attention_probs if self.training else 0.0)
         return self.dense(ctx.view(b, s, nq * d))
 
     # ---- KV cache ----------------------------------------------------------------------------------

@@ -383,7 +383,7 @@ def linear_cross_entropy(h: torch.Tensor, weight: torch.Tensor, targets: torch.T
 # ------------------------------------------------------------------------------------------------
 # attention core
 # ------------------------------------------------------------------------------------------------
-def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, flags=0) -> MiAttnArgs:
+def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, flags=0, dropout=None) -> MiAttnArgs:
     a = MiAttnArgs()
     a.flags = int(flags)
     a.q, a.k, a.v, a.o, a.lse = ptr(q), ptr(k), ptr(v), ptr(o), ptr(lse)
@@ -403,6 +403,8 @@ def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, fla
         a.rotary_cos, a.rotary_sin = ptr(cos), ptr(sin)
         a.position_ids_q, a.position_ids_k = ptr(pos_q), ptr(pos_k)
         a.rotary_table_rows = cos.shape[0]
+    if dropout is not None and dropout[0] > 0.0:
+        a.dropout_p, a.dropout_seed = float(dropout[0]), int(dropout[1]) & 0xFFFFFFFFFFFFFFFF
     a.stream = stream_ptr()
     return a
 
@@ -417,8 +419,11 @@ def _check_qkv(q, k, v, cu_q, cu_k):
         assert cu_k.dtype == torch.int32 and cu_k.is_contiguous() and cu_k.numel() == cu_q.numel()
 
 
-def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None, rotary=None, flags=0):
+def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None, rotary=None, flags=0,
+                      dropout=None):
     """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens]).
+
+    dropout: optional (p, seed) for dropout on the attention probabilities; the backward needs the same pair.
 
     flags: 0 lets the library pick the tiling; 1 / 2 pin one / two query groups per wavefront."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
@@ -431,13 +436,13 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
         assert pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0]
     o = torch.empty((q.shape[0], q.shape[1], q.shape[2]), dtype=q.dtype, device=q.device)
     lse = torch.empty((q.shape[1], q.shape[0]), dtype=torch.float32, device=q.device)
-    a = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary, flags)
+    a = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary, flags, dropout)
     check(_lib.load().mi_attn_fwd(ctypes.byref(a)), "mi_attn_fwd")
     return o, lse
 
 
 def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None,
-                       flags=0, buffers=None):
+                       flags=0, buffers=None, dropout=None):
     """Returns (dq, dk, dv) for already rotated q/k.
 
     flags: 0 runs the whole backward; 16 / 32 / 64 run only the delta / dK-dV / dQ kernel (timing aid).
@@ -461,7 +466,7 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
         nbytes = lib.mi_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], q.shape[2])
         ws = torch.empty(max(nbytes // 4, 4), dtype=torch.float32, device=q.device)
     b = MiAttnBwdArgs()
-    b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, None, flags)
+    b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, None, flags, dropout)
     b.d_o, b.dq, b.dk, b.dv = ptr(do), ptr(dq), ptr(dk), ptr(dv)
     b.dk_stride_token, b.dk_stride_head = dk.stride(0), dk.stride(1)
     b.dv_stride_token, b.dv_stride_head = dv.stride(0), dv.stride(1)
@@ -472,30 +477,47 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
 
 class _Attention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, cu_q, cu_k, causal, scale):
-        o, lse = attention_forward(q, k, v, cu_q, cu_k, causal, scale)
+    def forward(ctx, q, k, v, cu_q, cu_k, causal, scale, dropout_p, dropout_seed):
+        dropout = (dropout_p, dropout_seed) if dropout_p > 0.0 else None
+        o, lse = attention_forward(q, k, v, cu_q, cu_k, causal, scale, dropout=dropout)
         ctx.save_for_backward(q, k, v, o, lse, cu_q, cu_k if cu_k is not None else cu_q)
-        ctx.causal, ctx.scale = causal, scale
+        ctx.causal, ctx.scale, ctx.dropout = causal, scale, dropout
         return o
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, o, lse, cu_q, cu_k = ctx.saved_tensors
-        dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale)
-        return dq, dk, dv, None, None, None, None
+        dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale, dropout=ctx.dropout)
+        return dq, dk, dv, None, None, None, None, None, None
+
+
+def next_dropout_seed(device: torch.device) -> int:
+    """A fresh 64-bit seed from the device's default generator without touching the GPU: (seed, offset) of the
+    Philox state, with the offset advanced as torch's own random kernels do.  The state is part of what
+    torch.utils.checkpoint saves and restores, so a recomputed forward draws the same seed."""
+    gen = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+    seed, offset = gen.initial_seed(), gen.get_offset()
+    gen.set_offset(offset + 4)
+    return (seed * 0x9E3779B97F4A7C15 + offset * 0xD1B54A32D192ED03 + 0x2545F4914F6CDD1D) & 0xFFFFFFFFFFFFFFFF
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
               cu_seqlens_k: Optional[torch.Tensor] = None, causal: bool = True,
-              softmax_scale: Optional[float] = None) -> torch.Tensor:
+              softmax_scale: Optional[float] = None, dropout_p: float = 0.0,
+              dropout_seed: Optional[int] = None) -> torch.Tensor:
     """Differentiable attention core on q [tokens, n_q, d], k/v [tokens_k, n_kv, d] (bf16).
 
     Tokens are the flattened (batch seq) axis; cu_seqlens are int32 offsets on it.  Returns
-    o [tokens, n_q, d].
+    o [tokens, n_q, d].  dropout_p > 0 drops attention probabilities (attention.py:204-207) with a mask that
+    is a function of (dropout_seed, head, query, key); without a seed one is drawn from the device generator.
+    The drop probability is quantised to round(256 p) / 256.
     """
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
-    return _Attention.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, float(softmax_scale))
+    if dropout_p > 0.0 and dropout_seed is None:
+        dropout_seed = next_dropout_seed(q.device)
+    return _Attention.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, float(softmax_scale), float(dropout_p),
+                            int(dropout_seed) if dropout_seed is not None else 0)
 
 
 # ------------------------------------------------------------------------------------------------

@@ -235,3 +235,64 @@ def test_attention_full_size_properties(name, b, s, nq, nkv, docs):
     o1, _ = ops.attention_forward(qd, kd, ones, cud, None, True, scale)
     assert float((o1.float() - 1).abs().max()) <= 2 ** -7
     assert bool(torch.isfinite(lse).all())
+
+
+# ---- dropout on the attention probabilities (attention.py:204-207) --------------------------------------------
+@pytest.mark.parametrize("b,s,nq,nkv,d,causal,cuts,p", [
+    (1, 256, 4, 4, 128, True, (), 0.1),
+    (2, 192, 4, 2, 64, True, (100, 250), 0.25),
+    (1, 320, 8, 2, 128, False, (77,), 0.1),
+    (1, 200, 2, 1, 32, True, (), 0.5),
+    (1, 136, 3, 3, 96, True, (9,), 0.05),
+])
+def test_attention_dropout_matches_oracle_with_the_same_mask(b, s, nq, nkv, d, causal, cuts, p):
+    """The kernels' mask is a documented integer function of (seed, head, query, key); the test rebuilds it in
+    numpy and hands it to the oracle, so forward and all three gradients are compared element for element."""
+    print(f"case attn dropout b={b} s={s} nq={nq} nkv={nkv} d={d} causal={causal} cuts={cuts} p={p}", flush=True)
+    seed = 0x1234_5678_9ABC_DEF0 + s
+    q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=s + nq)
+    cu = U.make_cu(b, s, cuts)
+    scale = 1.0 / math.sqrt(d)
+    keep, p_eff = U.dropout_keep_mask(seed, nq, b * s, b * s, p)
+    assert abs(p_eff - p) <= 1.0 / 512
+    ref = U.oracle_attention(q, k, v, cu, b, s, causal, scale, torch.float32, do, dropout=(keep, p_eff))
+    ref_o = U.oracle_attention(q, k, v, cu, b, s, causal, scale, torch.bfloat16, do, dropout=(keep, p_eff))
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o = ops.attention(qg, kg, vg, cu.to(DEV), None, causal, scale, dropout_p=p, dropout_seed=seed)
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    for name, got, r, ro in (("o", o, ref[0], ref_o[0]), ("dq", qg.grad, ref[1], ref_o[1]),
+                             ("dk", kg.grad, ref[2], ref_o[2]), ("dv", vg.grad, ref[3], ref_o[3])):
+        check(f"attn.dropout.{name}", got, r, ro)
+    # the mask really dropped something, the same seed reproduces the result, another seed does not
+    plain = ops.attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), None, causal, scale)
+    assert not torch.equal(plain, o.detach())
+    again = ops.attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), None, causal, scale, dropout_p=p, dropout_seed=seed)
+    other = ops.attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), None, causal, scale, dropout_p=p, dropout_seed=seed + 1)
+    assert torch.equal(again, o.detach()) and not torch.equal(other, o.detach())
+
+
+def test_attention_dropout_statistics_and_generator_seed():
+    """With V = identity-like one-hot rows the output of a non-causal single document is the dropped probability
+    matrix itself, which exposes the keep rate; seeds drawn from the device generator follow torch.manual_seed."""
+    print("case attn dropout statistics", flush=True)
+    s, d, p = 128, 128, 0.1
+    q = torch.zeros(s, 8, d, dtype=torch.bfloat16, device=DEV)      # uniform probabilities 1 / s
+    k = torch.zeros(s, 8, d, dtype=torch.bfloat16, device=DEV)
+    v = torch.eye(s, d, dtype=torch.bfloat16, device=DEV).unsqueeze(1).expand(s, 8, d).contiguous()
+    cu = torch.tensor([0, s], dtype=torch.int32, device=DEV)
+    seed = 99
+    o = ops.attention(q, k, v, cu, None, False, 1.0, dropout_p=p, dropout_seed=seed)   # o[q, h, k] = keep / (1 - p) / s
+    keep, p_eff = U.dropout_keep_mask(seed, 8, s, s, p)
+    got_keep = (o.float().cpu() > 0).permute(1, 0, 2)
+    assert torch.equal(got_keep, keep)
+    kept_value = o.float().max().item()
+    assert abs(kept_value - 1.0 / (1.0 - p_eff) / s) < 1e-4
+    rate = got_keep.float().mean().item()
+    assert abs(rate - (1.0 - p_eff)) < 4 * math.sqrt(p_eff * (1 - p_eff) / got_keep.numel())
+    torch.manual_seed(7)
+    a = ops.attention(q, k, v, cu, None, False, 1.0, dropout_p=p)
+    b2 = ops.attention(q, k, v, cu, None, False, 1.0, dropout_p=p)
+    torch.manual_seed(7)
+    a2 = ops.attention(q, k, v, cu, None, False, 1.0, dropout_p=p)
+    assert torch.equal(a, a2) and not torch.equal(a, b2)

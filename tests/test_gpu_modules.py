@@ -179,3 +179,44 @@ def test_graph_captured_decode_equals_eager_decode(max_tokens):
     assert graphed == eager
     # a second capture on the same module (fresh prefill) gives the same tokens again
     assert model.generate_graph(max_tokens, prompts) == eager
+
+
+def test_layer_with_attention_dropout_train_eval_and_recompute():
+    """dropout_attention_probs: off in eval mode, on in training mode, reproducible from torch.manual_seed, and
+    identical when the layer is recomputed under activation checkpointing (the seed comes from the generator
+    state that torch.utils.checkpoint restores)."""
+    print("case layer attention dropout", flush=True)
+    from torch.utils.checkpoint import checkpoint
+    cfg_drop = _arch(dropout_attention_probs=0.2, attention_num_kv_heads=2)
+    cfg_none = _arch(attention_num_kv_heads=2)
+    layer = _seeded_layer(cfg_drop, 3)
+    plain = _seeded_layer(cfg_none, 3)
+    b, s = 2, 96
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(b, s, cfg_drop.hidden_size, generator=g).bfloat16().to(DEV)
+    ids = torch.ones(b, s, dtype=torch.int64)
+    cu = D.get_cumulative_seq_lengths(ids).to(DEV)
+    pos = D.get_position_ids(ids).to(DEV)
+
+    def run(mod, inp):
+        return mod(TransformerLayerIO(activations=inp, position_ids=pos, cumulative_seq_lengths=cu)).activations
+
+    layer.eval(); plain.eval()
+    assert torch.equal(run(layer, x), run(plain, x))
+    layer.train()
+    torch.manual_seed(5)
+    y1 = run(layer, x)
+    y2 = run(layer, x)
+    torch.manual_seed(5)
+    y3 = run(layer, x)
+    assert torch.equal(y1, y3) and not torch.equal(y1, y2) and not torch.equal(y1, run(plain, x))
+    # gradients with and without recomputation agree bit for bit
+    grads = []
+    for use_ckpt in (False, True):
+        torch.manual_seed(11)
+        xin = x.clone().requires_grad_()
+        layer.zero_grad()
+        out = checkpoint(lambda t: run(layer, t), xin, use_reentrant=False) if use_ckpt else run(layer, xin)
+        out.float().square().mean().backward()
+        grads.append((xin.grad.clone(), layer.self_attention.dense.weight.grad.clone()))
+    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])

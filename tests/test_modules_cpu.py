@@ -129,8 +129,8 @@ def test_unsupported_options_raise():
     hip = C.MaskedSoftmaxConfig(kernel="hip")
     with pytest.raises(NotImplementedError, match="hip"):
         ParallelSelfAttention(256, 4, C.MaskedSoftmaxConfig(kernel="torch"), dtype=torch.bfloat16, device=CPU)
-    with pytest.raises(NotImplementedError, match="dropout"):
-        ParallelSelfAttention(256, 4, hip, dropout_attention_probs=0.1, dtype=torch.bfloat16, device=CPU)
+    assert ParallelSelfAttention(256, 4, hip, dropout_attention_probs=0.1, dtype=torch.bfloat16, device=CPU,
+                                 rotary_config=C.RotaryConfig(dimensions=64)).dropout_attention_probs == 0.1
     with pytest.raises(NotImplementedError, match="bfloat16"):
         ParallelSelfAttention(256, 4, hip, dtype=torch.float32, device=CPU)
     cplx = ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, rotary_config=C.RotaryConfig(dimensions=64, max_seq_length=16),
