@@ -244,7 +244,7 @@ int mi_attn_bwd(const mi_attn_bwd_args* args);
  *
  * If k_new/v_new != NULL the kernel first appends them at position ctx_len[b]-1 (in-place append
  * instead of torch.cat); with rotary_cos != NULL it rotates q and k_new by position_ids[b] before
- * use/append (fused rotary).  q, o: [batch, n_q_heads, head_dim] contiguous.
+ * use/append (fused rotary).  o: [batch, n_q_heads, head_dim] contiguous; q likewise unless q_stride_batch is set.
  * The key axis is split into n_splits chunks processed by different workgroups and merged by a
  * second kernel; workspace = mi_attn_decode_workspace_bytes() bytes of fp32 scratch.
  * Algorithmic HBM bytes: 2 * sum_b ctx_len[b] * n_kv_heads * head_dim * e  (K and V read once).
@@ -273,6 +273,9 @@ typedef struct mi_decode_args {
     void* workspace;
     size_t workspace_bytes;
     void* stream;
+    /* element strides between the sequences of q / k_new / v_new (their [heads, head_dim] part stays contiguous);
+     * 0 = packed ([batch, heads, head_dim] contiguous).  Lets q, k and v be column slices of one fused projection. */
+    int64_t q_stride_batch, k_new_stride_batch, v_new_stride_batch;
 } mi_decode_args;
 
 size_t mi_attn_decode_workspace_bytes(int32_t batch, int32_t n_q_heads, int32_t head_dim, int32_t max_ctx);

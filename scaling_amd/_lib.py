@@ -68,6 +68,7 @@ class MiDecodeArgs(Structure):
         ("softmax_scale", c_float), ("n_splits", c_int32),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("stream", c_void_p),
+        ("q_stride_batch", c_int64), ("k_new_stride_batch", c_int64), ("v_new_stride_batch", c_int64),
     ]
 
 

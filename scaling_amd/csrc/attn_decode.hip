@@ -26,6 +26,7 @@ struct DecodeParams {
     const __bf16* cos; const __bf16* sin; const int64_t* pos; int table_rows;
     int batch, max_ctx, nq, nkv, n_rep, n_splits;
     int64_t c_sb, c_st, c_sh;
+    int64_t q_sb, kn_sb, vn_sb;   // element strides between sequences of q / k_new / v_new
     float scale_log2;
     float* ws_o;   // [batch][nq][n_splits][D]
     float* ws_ml;  // [batch][nq][n_splits][2]
@@ -45,7 +46,8 @@ __global__ void decode_append_kernel(const DecodeParams p) {
     const int c = idx % HV, kvh = (idx / HV) % p.nkv, b = idx / (HV * p.nkv);
     const int ctx = p.ctx_len[b];
     if (ctx < 1 || ctx > p.max_ctx) return;
-    const int64_t src = ((int64_t)b * p.nkv + kvh) * D + 8 * c;
+    const int64_t src = (int64_t)b * p.kn_sb + (int64_t)kvh * D + 8 * c;
+    const int64_t src_v = (int64_t)b * p.vn_sb + (int64_t)kvh * D + 8 * c;
     const int64_t dst = (int64_t)b * p.c_sb + (int64_t)(ctx - 1) * p.c_st + (int64_t)kvh * p.c_sh + 8 * c;
     uint4 lo = *reinterpret_cast<const uint4*>(p.k_new + src);
     uint4 hi = *reinterpret_cast<const uint4*>(p.k_new + src + D / 2);
@@ -58,8 +60,8 @@ __global__ void decode_append_kernel(const DecodeParams p) {
     }
     *reinterpret_cast<uint4*>(p.kc + dst) = lo;
     *reinterpret_cast<uint4*>(p.kc + dst + D / 2) = hi;
-    *reinterpret_cast<uint4*>(p.vc + dst) = *reinterpret_cast<const uint4*>(p.v_new + src);
-    *reinterpret_cast<uint4*>(p.vc + dst + D / 2) = *reinterpret_cast<const uint4*>(p.v_new + src + D / 2);
+    *reinterpret_cast<uint4*>(p.vc + dst) = *reinterpret_cast<const uint4*>(p.v_new + src_v);
+    *reinterpret_cast<uint4*>(p.vc + dst + D / 2) = *reinterpret_cast<const uint4*>(p.v_new + src_v + D / 2);
 }
 
 // ---- split kernel ----------------------------------------------------------------------------------
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     bf16x8_t qf[KS];
     {
         const int hs = l16 < p.n_rep ? l16 : 0;
-        const __bf16* qr = p.q + ((int64_t)b * p.nq + kvh * p.n_rep + hs) * D + 8 * G;
+        const __bf16* qr = p.q + (int64_t)b * p.q_sb + (int64_t)(kvh * p.n_rep + hs) * D + 8 * G;
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qr + 32 * ks);
@@ -353,8 +355,13 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
         (a->k_new && (!mi_aligned16(a->k_new) || !mi_aligned16(a->v_new))) ||
         (rot && (!mi_aligned16(a->rotary_cos) || !mi_aligned16(a->rotary_sin))))
         return mi_fail(MI_E_ALIGN, "attn_decode: tensors must be 16-byte aligned");
-    if (a->cache_stride_batch % 8 || a->cache_stride_token % 8 || a->cache_stride_head % 8)
-        return mi_fail(MI_E_ALIGN, "attn_decode: cache strides must be multiples of 8 elements");
+    if (a->cache_stride_batch % 8 || a->cache_stride_token % 8 || a->cache_stride_head % 8 || a->q_stride_batch % 8 ||
+        a->k_new_stride_batch % 8 || a->v_new_stride_batch % 8)
+        return mi_fail(MI_E_ALIGN, "attn_decode: strides must be multiples of 8 elements");
+    if ((a->q_stride_batch && a->q_stride_batch < (int64_t)a->n_q_heads * a->head_dim) ||
+        (a->k_new_stride_batch && a->k_new_stride_batch < (int64_t)a->n_kv_heads * a->head_dim) ||
+        (a->v_new_stride_batch && a->v_new_stride_batch < (int64_t)a->n_kv_heads * a->head_dim))
+        return mi_fail(MI_E_SHAPE, "attn_decode: a sequence stride is smaller than heads * head_dim");
     if (!(a->softmax_scale > 0.f)) return mi_fail(MI_E_SHAPE, "attn_decode: softmax_scale must be positive");
     int splits = a->n_splits > 0 ? a->n_splits : choose_splits(a->batch, a->n_kv_heads, a->max_ctx);
     if (splits > kMaxSplits) splits = kMaxSplits;
@@ -369,6 +376,9 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     p.batch = a->batch; p.max_ctx = a->max_ctx; p.nq = a->n_q_heads; p.nkv = a->n_kv_heads;
     p.n_rep = a->n_q_heads / a->n_kv_heads; p.n_splits = splits;
     p.c_sb = a->cache_stride_batch; p.c_st = a->cache_stride_token; p.c_sh = a->cache_stride_head;
+    p.q_sb = a->q_stride_batch ? a->q_stride_batch : (int64_t)a->n_q_heads * a->head_dim;
+    p.kn_sb = a->k_new_stride_batch ? a->k_new_stride_batch : (int64_t)a->n_kv_heads * a->head_dim;
+    p.vn_sb = a->v_new_stride_batch ? a->v_new_stride_batch : (int64_t)a->n_kv_heads * a->head_dim;
     p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
     p.ws_o = (float*)a->workspace;
     p.ws_ml = p.ws_o + (size_t)a->batch * a->n_q_heads * splits * a->head_dim;

@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
             Elem<T>::unpack(raw[j], f);
 #pragma unroll
             for (int i = 0; i < V; ++i) mt = fmaxf(mt, f[i]);
-            __builtin_amdgcn_sched_barrier(0);    // one vector at a time: unpacking ahead only costs registers
+            if (j & 1) __builtin_amdgcn_sched_barrier(0);    // two vectors at a time: unpacking further ahead only costs registers
         }
         // pass 2: this thread's sum of exponentials relative to its own maximum
         const float mt2 = (mt == -INFINITY ? 0.f : mt) * kLog2e;
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
                 s0 += __builtin_amdgcn_exp2f(f[i] * kLog2e - mt2);
                 s1 += __builtin_amdgcn_exp2f(f[i + 1] * kLog2e - mt2);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            if (j & 1) __builtin_amdgcn_sched_barrier(0);
         }
         // merge (maximum, sum) pairs: wavefront, then block
         float wm = mt;
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
                     Elem<T>::store1(dx + target, (__builtin_amdgcn_exp2f(x_target * kLog2e - l2) - 1.0f) * scale);
             }
             if (has_next) load_vec(next, j);
-            __builtin_amdgcn_sched_barrier(0);
+            if (j & 1) __builtin_amdgcn_sched_barrier(0);
         }
         prev_row = row;
         target = target_next;

@@ -164,10 +164,17 @@ class TransformerInferenceModule(torch.nn.Module):
                 cache.workspace = ops.decode_workspace(b, att.num_attention_heads, att.hidden_size_per_attention_head,
                                                        cache.max_ctx, self.device)
 
+        # every layer has seen the same tokens: one device-side context-length vector serves all caches and is
+        # advanced once per step instead of once per layer
+        shared_ctx = layers[0].self_attention.cache[0].ctx_len
+        for layer in layers[1:]:
+            layer.self_attention.cache[0].ctx_len = shared_ctx
+
         def one_step():
             h = self._layers[0](tok)
+            shared_ctx.add_(1)
             for layer in layers:
-                h = layer.decode_step(h, pos)
+                h = layer.decode_step(h, pos, advance=False)
             lg = self._layers[-1].linear(self._layers[-2].norm(h))
             nxt = torch.argmax(lg, dim=-1)                                # [b, 1]
             out.index_copy_(1, step, nxt)
@@ -189,8 +196,11 @@ class TransformerInferenceModule(torch.nn.Module):
                 one_step()
             for _ in range(remaining):   # capture only records; every remaining token is one replay
                 graph.replay()
-        for layer in layers:
-            layer.self_attention.cache[0].length = n_prompt + max_tokens - 1
+        for i, layer in enumerate(layers):
+            cache = layer.self_attention.cache[0]
+            cache.length = n_prompt + max_tokens - 1
+            if i > 0:
+                cache.ctx_len = shared_ctx.clone()      # each cache owns its lengths again
         return out.tolist()
 
     @torch.no_grad()

@@ -103,9 +103,11 @@ class TransformerLayer(torch.nn.Module):
         residual = self.mlp(self.post_attention_layernorm(hidden_state))
         return self.dropout_mlp(residual) + hidden_state
 
-    def decode_step(self, hidden_state: torch.Tensor, position_ids: torch.Tensor, cache_index: int = 0) -> torch.Tensor:
+    def decode_step(self, hidden_state: torch.Tensor, position_ids: torch.Tensor, cache_index: int = 0,
+                    advance: bool = True) -> torch.Tensor:
         """Cached single-token step on plain tensors, free of host synchronisation (HIP-graph capturable)."""
-        h = hidden_state + self.self_attention.decode_forward(self.input_layernorm(hidden_state), position_ids, cache_index)
+        h = hidden_state + self.self_attention.decode_forward(self.input_layernorm(hidden_state), position_ids, cache_index,
+                                                              advance=advance)
         return h + self.mlp(self.post_attention_layernorm(h))
 
     def forward(self, x: TransformerLayerIO) -> TransformerLayerIO:

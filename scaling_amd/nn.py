@@ -335,10 +335,47 @@ class ParallelSelfAttention(torch.nn.Module):
         if self.qkv_in_one:
             qkv = self.query_key_value(x).view(b * s, nq, 3 * d)       # per head: q then k then v (attention.py:790-796)
             return qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:]
+        if not torch.is_grad_enabled():
+            # inference: one projection GEMM over the row-stacked weights; q, k, v are column slices of its output
+            w, bias = self._fused_qkv()
+            out = F.linear(x, w, bias).view(b * s, (nq + 2 * nkv) * d)
+            return (out[:, :nq * d].view(b * s, nq, d), out[:, nq * d:(nq + nkv) * d].view(b * s, nkv, d),
+                    out[:, (nq + nkv) * d:].view(b * s, nkv, d))
         q = self.query(x).view(b * s, nq, d)
         k = self.key(x).view(b * s, nkv, d)
         v = self.value(x).view(b * s, nkv, d)
         return q, k, v
+
+    def _fused_qkv(self):
+        """The weights (and biases) of `query`, `key`, `value` as row blocks of one tensor.  Built on first use: the
+        three parameters are re-pointed at views of the stacked copy, so values, names and the state dict stay as
+        they are while a single GEMM can read all of them.  Rebuilt if a parameter was moved or replaced."""
+        mods = (self.query, self.key, self.value)
+        rows = [m.weight.shape[0] for m in mods]
+        offs = [0, rows[0], rows[0] + rows[1]]
+        fused = self.__dict__.get("_qkv_fused")
+
+        def aliased(t, name):
+            return t is not None and all(getattr(m, name).data_ptr() == t[o:o + r].data_ptr() and getattr(m, name).device == t.device
+                                         for m, o, r in zip(mods, offs, rows))
+
+        has_bias = mods[0].bias is not None
+        if fused is None or not aliased(fused[0], "weight") or (has_bias and not aliased(fused[1], "bias")):
+            w = torch.cat([m.weight.data for m in mods], dim=0)
+            bias = torch.cat([m.bias.data for m in mods], dim=0) if has_bias else None
+            for m, o, r in zip(mods, offs, rows):
+                m.weight.data = w[o:o + r]
+                if has_bias:
+                    m.bias.data = bias[o:o + r]
+            fused = (w, bias)
+            self.__dict__["_qkv_fused"] = fused
+        return fused
+
+    @staticmethod
+    def _decode_operand(t: torch.Tensor) -> torch.Tensor:
+        """q / k / v of one token per sequence as the decode kernel takes them: [heads, d] contiguous per sequence."""
+        ok = t.stride(2) == 1 and t.stride(1) == t.shape[2] and t.stride(0) % 8 == 0
+        return t if ok else t.contiguous()
 
     @staticmethod
     def _rows_are_single_documents(cu: torch.Tensor, b: int, s: int) -> bool:
@@ -404,17 +441,20 @@ class ParallelSelfAttention(torch.nn.Module):
         cache.length = s
         cache.ctx_len.fill_(s)
 
-    def decode_forward(self, x: torch.Tensor, position_ids: torch.Tensor, cache_index: int = 0) -> torch.Tensor:
+    def decode_forward(self, x: torch.Tensor, position_ids: torch.Tensor, cache_index: int = 0,
+                       advance: bool = True) -> torch.Tensor:
         """One cached decode step without any host synchronisation (usable under HIP graph capture):
         x [b, 1, H], position_ids int64 [b].  The caller guarantees a prefilled cache with room for one
-        more token per sequence; only the device-side context lengths are advanced here."""
+        more token per sequence; only the device-side context lengths are advanced here (advance=False when
+        the caller shares one context-length tensor between layers and has advanced it already)."""
         b = x.shape[0]
         nq, d = self.num_attention_heads, self.hidden_size_per_attention_head
         q, k, v = self._project(x)
         if self.key_query_norm:
             q, k = self.norm_query(q), self.norm_key(k)
         cache = self.cache[cache_index]
-        cache.ctx_len.add_(1)
+        if advance:
+            cache.ctx_len.add_(1)
         rotary = None
         if self.rotary_embedding is not None:
             if self._fusable_rotary:
@@ -423,8 +463,8 @@ class ParallelSelfAttention(torch.nn.Module):
             else:
                 q = self.rotary_embedding.rotate_tokens(q, position_ids, 1)
                 k = self.rotary_embedding.rotate_tokens(k, position_ids, 1)
-        ctx = ops.decode_attention(q.contiguous(), cache.k, cache.v, cache.ctx_len, k.contiguous(), v.contiguous(),
-                                   rotary=rotary, softmax_scale=self.softmax_scale, workspace=cache.workspace)
+        ctx = ops.decode_attention(self._decode_operand(q), cache.k, cache.v, cache.ctx_len, self._decode_operand(k),
+                                   self._decode_operand(v), rotary=rotary, softmax_scale=self.softmax_scale, workspace=cache.workspace)
         return self.dense(ctx.view(b, 1, nq * d))
 
     def _decode_step(self, q, k, v, pos, b: int, s: int, cache_index: int) -> torch.Tensor:
@@ -448,5 +488,5 @@ class ParallelSelfAttention(torch.nn.Module):
                 k = self.rotary_embedding.rotate_tokens(k, pos, 1)
         if cache.workspace is None:
             cache.workspace = ops.decode_workspace(b, nq, d, cache.max_ctx, q.device)
-        return ops.decode_attention(q.contiguous(), cache.k, cache.v, cache.ctx_len, k.contiguous(), v.contiguous(),
-                                    rotary=rotary, softmax_scale=self.softmax_scale, workspace=cache.workspace)
+        return ops.decode_attention(self._decode_operand(q), cache.k, cache.v, cache.ctx_len, self._decode_operand(k),
+                                    self._decode_operand(v), rotary=rotary, softmax_scale=self.softmax_scale, workspace=cache.workspace)

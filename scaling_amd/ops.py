@@ -535,10 +535,16 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      n_splits: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One decode step.  q [B, n_q, d]; caches [B, max_ctx, n_kv, d]; ctx_len int32 [B] counts the valid
     keys INCLUDING the token appended by this call (k_new/v_new [B, n_kv, d], written at ctx_len-1).
-    rotary = (cos, sin, position_ids[B]) rotates q and k_new inside the kernels."""
+    rotary = (cos, sin, position_ids[B]) rotates q and k_new inside the kernels.  q, k_new and v_new may be
+    column slices of one projection output: only their [heads, d] part has to be contiguous."""
     _need_cuda(q, k_cache, v_cache, ctx_len)
     B, nq, d = q.shape
-    assert q.is_contiguous() and k_cache.dim() == 4 and k_cache.shape == v_cache.shape
+
+    def _rows(t):
+        assert t.stride(2) == 1 and t.stride(1) == d and t.stride(0) % 8 == 0, "each sequence's [heads, d] block must be contiguous"
+        return t.stride(0)
+
+    assert k_cache.dim() == 4 and k_cache.shape == v_cache.shape
     assert k_cache.stride() == v_cache.stride() and k_cache.stride(3) == 1
     assert ctx_len.dtype == torch.int32 and ctx_len.numel() == B
     if softmax_scale is None:
@@ -546,12 +552,14 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     if workspace is None:
         workspace = decode_workspace(B, nq, d, k_cache.shape[1], q.device)
     if out is None:
-        out = torch.empty_like(q)
+        out = torch.empty((B, nq, d), dtype=q.dtype, device=q.device)
     a = MiDecodeArgs()
     a.q, a.k_cache, a.v_cache, a.o, a.ctx_len = ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), ptr(ctx_len)
+    a.q_stride_batch = _rows(q)
     if k_new is not None:
-        assert k_new.is_contiguous() and v_new.is_contiguous() and k_new.shape == (B, k_cache.shape[2], d)
+        assert k_new.shape == (B, k_cache.shape[2], d) and v_new.shape == k_new.shape
         a.k_new, a.v_new = ptr(k_new), ptr(v_new)
+        a.k_new_stride_batch, a.v_new_stride_batch = _rows(k_new), _rows(v_new)
     if rotary is not None:
         cos, sin, pos = rotary
         assert cos.dtype == q.dtype and cos.is_contiguous() and sin.is_contiguous() and cos.shape[1] == d
