@@ -60,6 +60,13 @@ int mi_check_device(void);
 int mi_rmsnorm_fwd(const void* x, const void* weight, void* y, float* rstd,
                    int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
 
+/* Residual add fused into the norm that follows it (transformer/model/layers/layer.py:252-293 with
+ * core/nn/residual.py:49-65 at inference): sum_out = x + residual rounded to `dtype`, y = rmsnorm(sum_out) * weight
+ * exactly as mi_rmsnorm_fwd computes it from the stored sum.  sum_out may alias x or residual; y may not alias.
+ * Forward only.  Algorithmic HBM bytes: 4 * n_rows * hidden * e. */
+int mi_add_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* sum_out, void* y,
+                       int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
+
 /* Backward of the above (what autograd derives from rms_norm.py:47-50):
  *   dx = rstd * (dy*w) - x * rstd^3 * mean(dy*w*x),   dweight = sum_rows dy * x * rstd.
  * rstd is recomputed from x.  `workspace` holds per-block fp32 partial sums of dweight and must be

@@ -18,7 +18,7 @@ _DTYPE_CODE = {torch.bfloat16: MI_BF16, torch.float16: MI_F16, torch.float32: MI
 
 EXPORTS = (
     "mi_version", "mi_last_error", "mi_status_string", "mi_check_device",
-    "mi_rmsnorm_fwd", "mi_rmsnorm_bwd_workspace_bytes", "mi_rmsnorm_bwd",
+    "mi_rmsnorm_fwd", "mi_add_rmsnorm_fwd", "mi_rmsnorm_bwd_workspace_bytes", "mi_rmsnorm_bwd",
     "mi_layernorm_fwd", "mi_layernorm_bwd_workspace_bytes", "mi_layernorm_bwd", "mi_gelu_fwd", "mi_gelu_bwd", "mi_cross_entropy",
     "mi_swiglu_fwd", "mi_swiglu_bwd", "mi_rotary", "mi_rotary_complex",
     "mi_attn_fwd", "mi_attn_bwd_workspace_bytes", "mi_attn_bwd",
@@ -85,6 +85,8 @@ def _declare(lib):
     lib.mi_rmsnorm_fwd.restype = c_int
     lib.mi_rmsnorm_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_int, c_void_p]
     lib.mi_rmsnorm_bwd_workspace_bytes.restype = c_size_t
+    lib.mi_add_rmsnorm_fwd.restype = c_int
+    lib.mi_add_rmsnorm_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_int, c_void_p]
     lib.mi_rmsnorm_bwd_workspace_bytes.argtypes = [c_int64, c_int64]
     lib.mi_rmsnorm_bwd.restype = c_int
     lib.mi_rmsnorm_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int64,

@@ -25,10 +25,13 @@ template <int TPR> __device__ __forceinline__ float row_sum(float v, float* lds)
     }
 }
 
-template <typename T, int TPR, int CH>
+// ADD: the row that is normalised is x + residual, rounded to T and also stored to sum_out (which may alias x or
+// residual): the residual add of the layer fused into the norm that follows it.
+template <typename T, int TPR, int CH, bool ADD = false>
 __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                               T* __restrict__ y, float* __restrict__ rstd_out,
-                                                              int64_t n_rows, int hidden, float eps) {
+                                                              int64_t n_rows, int hidden, float eps,
+                                                              const T* residual = nullptr, T* sum_out = nullptr) {
     constexpr int V = Elem<T>::kVec;
     constexpr int RPB = kBlock / TPR;
     __shared__ float lds[4];
@@ -42,6 +45,17 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
     for (int c = 0; c < CH; ++c) {
         const int v = c * TPR + tr;
         raw[c] = (row_ok && v < vecs) ? xr[v] : make_uint4(0, 0, 0, 0);
+        if constexpr (ADD) {
+            if (row_ok && v < vecs) {
+                float a[V], r[V];
+                Elem<T>::unpack(raw[c], a);
+                Elem<T>::unpack(reinterpret_cast<const uint4*>(residual + row * hidden)[v], r);
+#pragma unroll
+                for (int i = 0; i < V; ++i) a[i] += r[i];
+                raw[c] = Elem<T>::pack(a);            // the norm sees the sum as it is stored
+                reinterpret_cast<uint4*>(sum_out + row * hidden)[v] = raw[c];
+            }
+        }
     }
     float ss = 0.f;
 #pragma unroll
@@ -377,7 +391,7 @@ template <typename F> bool dispatch_plan(const Plan& plan, F&& f) {
 
 template <typename T>
 int launch_fwd(const void* x, const void* w, void* y, float* rstd, int64_t n_rows, int64_t hidden, float eps,
-               hipStream_t st) {
+               hipStream_t st, const void* residual = nullptr, void* sum_out = nullptr) {
     Plan plan;
     if (!make_plan<T>(hidden, &plan))
         return mi_fail(MI_E_SHAPE, "rmsnorm: hidden=%lld unsupported (must be a multiple of %d and <= %d)",
@@ -387,8 +401,12 @@ int launch_fwd(const void* x, const void* w, void* y, float* rstd, int64_t n_row
         constexpr int CH = decltype(tag)::CH;
         const int rpb = kBlock / TPR;
         const unsigned grid = (unsigned)((n_rows + rpb - 1) / rpb);
-        rmsnorm_fwd_kernel<T, TPR, CH><<<dim3(grid), dim3(kBlock), 0, st>>>((const T*)x, (const T*)w, (T*)y, rstd, n_rows,
-                                                                            (int)hidden, eps);
+        if (residual != nullptr)
+            rmsnorm_fwd_kernel<T, TPR, CH, true><<<dim3(grid), dim3(kBlock), 0, st>>>((const T*)x, (const T*)w, (T*)y, rstd, n_rows,
+                                                                                      (int)hidden, eps, (const T*)residual, (T*)sum_out);
+        else
+            rmsnorm_fwd_kernel<T, TPR, CH><<<dim3(grid), dim3(kBlock), 0, st>>>((const T*)x, (const T*)w, (T*)y, rstd, n_rows,
+                                                                                (int)hidden, eps);
     });
     if (!launched) return mi_fail(MI_E_SHAPE, "rmsnorm: no kernel for hidden=%lld", (long long)hidden);
     return mi_check_launch("rmsnorm_fwd");
@@ -828,6 +846,18 @@ int mi_rmsnorm_fwd(const void* x, const void* weight, void* y, float* rstd, int6
     if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(y)) return mi_fail(MI_E_ALIGN, "rmsnorm_fwd: pointers must be 16-byte aligned");
     if (n_rows == 0) return MI_OK;
     MI_DISPATCH_DTYPE(dtype, return launch_fwd<T>(x, weight, y, rstd, n_rows, hidden, eps, (hipStream_t)stream));
+    return MI_OK;
+}
+
+int mi_add_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* sum_out, void* y, int64_t n_rows,
+                       int64_t hidden, float eps, int dtype, void* stream) {
+    if (!x || !residual || !weight || !sum_out || !y) return mi_fail(MI_E_NULL, "add_rmsnorm_fwd: null pointer");
+    if (n_rows < 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "add_rmsnorm_fwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
+    if (!mi_aligned16(x) || !mi_aligned16(residual) || !mi_aligned16(weight) || !mi_aligned16(sum_out) || !mi_aligned16(y))
+        return mi_fail(MI_E_ALIGN, "add_rmsnorm_fwd: pointers must be 16-byte aligned");
+    if (y == sum_out || y == x || y == residual) return mi_fail(MI_E_SHAPE, "add_rmsnorm_fwd: y must not alias the other tensors");
+    if (n_rows == 0) return MI_OK;
+    MI_DISPATCH_DTYPE(dtype, return launch_fwd<T>(x, weight, y, nullptr, n_rows, hidden, eps, (hipStream_t)stream, residual, sum_out));
     return MI_OK;
 }
 

@@ -170,12 +170,29 @@ class TransformerInferenceModule(torch.nn.Module):
         for layer in layers[1:]:
             layer.self_attention.cache[0].ctx_len = shared_ctx
 
+        from .nn import RMSNorm
+        from . import ops
+        final_norm = self._layers[-2].norm
+        fuse_add_norm = all(isinstance(n, RMSNorm) for layer in layers for n in (layer.input_layernorm, layer.post_attention_layernorm)) \
+            and isinstance(final_norm, RMSNorm)
+
         def one_step():
             h = self._layers[0](tok)
             shared_ctx.add_(1)
-            for layer in layers:
-                h = layer.decode_step(h, pos, advance=False)
-            lg = self._layers[-1].linear(self._layers[-2].norm(h))
+            if fuse_add_norm:
+                # every residual add is folded into the RMSNorm that follows it (same rounding points as the
+                # separate add and norm of layer.decode_step)
+                n = layers[0].input_layernorm(h)
+                for i, layer in enumerate(layers):
+                    a = layer.self_attention.decode_forward(n, pos, advance=False)
+                    h, n = ops.add_rms_norm(h, a, layer.post_attention_layernorm.weight, layer.post_attention_layernorm.eps)
+                    nxt_norm = layers[i + 1].input_layernorm if i + 1 < len(layers) else final_norm
+                    h, n = ops.add_rms_norm(h, layer.mlp(n), nxt_norm.weight, nxt_norm.eps)
+                lg = self._layers[-1].linear(n)
+            else:
+                for layer in layers:
+                    h = layer.decode_step(h, pos, advance=False)
+                lg = self._layers[-1].linear(final_norm(h))
             nxt = torch.argmax(lg, dim=-1)                                # [b, 1]
             out.index_copy_(1, step, nxt)
             tok.copy_(nxt)

@@ -18,7 +18,7 @@ from ._lib import MiAttnArgs, MiAttnBwdArgs, MiDecodeArgs, check, dtype_code, pt
 __all__ = [
     "rms_norm", "swiglu", "rotary_embedding", "rotary_embedding_complex", "attention", "attention_forward", "attention_backward",
     "decode_attention", "rms_norm_forward", "rms_norm_backward", "swiglu_forward", "swiglu_backward",
-    "cross_entropy", "cross_entropy_forward", "linear_cross_entropy",
+    "cross_entropy", "cross_entropy_forward", "linear_cross_entropy", "add_rms_norm",
 ]
 
 
@@ -32,6 +32,18 @@ def _need_cuda(*tensors):
 # ------------------------------------------------------------------------------------------------
 # RMSNorm
 # ------------------------------------------------------------------------------------------------
+def add_rms_norm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(x + residual, rms_norm(x + residual) * weight) in one launch (inference; no autograd).  The sum is rounded
+    to the tensor dtype before it is normalised, as the separate add and norm would do."""
+    _need_cuda(x, residual, weight)
+    assert x.shape == residual.shape and x.dtype == residual.dtype == weight.dtype and x.shape[-1] == weight.shape[0]
+    x2, r2 = x.contiguous().view(-1, x.shape[-1]), residual.contiguous().view(-1, x.shape[-1])
+    total, y = torch.empty_like(x2), torch.empty_like(x2)
+    check(_lib.load().mi_add_rmsnorm_fwd(ptr(x2), ptr(r2), ptr(weight.contiguous()), ptr(total), ptr(y), x2.shape[0], x2.shape[1],
+                                         float(eps), dtype_code(x.dtype), stream_ptr()), "mi_add_rmsnorm_fwd")
+    return total.view(x.shape), y.view(x.shape)
+
+
 def rms_norm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     _need_cuda(x, weight)
     assert x.shape[-1] == weight.shape[0] and weight.dtype == x.dtype

@@ -249,3 +249,21 @@ def test_layernorm_and_gelu_mlp_reproduce_the_reference_golden(golden_dir):
     assert float(((att + h).cpu() - gt["hidden_states_mlp"]).abs().max()) < 1e-4
     fin = ops.layer_norm(gt["hidden_states_layer0"].to(DEV), dev("transformer.norm.weight"), dev("transformer.norm.bias"), 1e-5)
     assert float((fin.cpu() - gt["hidden_states_norm"]).abs().max()) < 1e-3
+
+
+@pytest.mark.parametrize("rows,hidden", [(32, 4096), (5, 256), (33, 8192)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_add_rmsnorm_equals_separate_add_and_norm(rows, hidden, dtype):
+    """The fused residual add + RMSNorm of the decode loop is bit-identical to the tensor add followed by the norm
+    kernel (the sum is rounded to the tensor dtype before it is normalised), and in-place sums are allowed."""
+    print(f"case add_rmsnorm rows={rows} hidden={hidden} dtype={dtype}", flush=True)
+    g = torch.Generator().manual_seed(rows + hidden)
+    x, r = _rand(g, rows, hidden, dtype=dtype).to(DEV), _rand(g, rows, hidden, dtype=dtype).to(DEV)
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype).to(DEV)
+    total, y = ops.add_rms_norm(x, r, w, 1e-5)
+    want_total = x + r
+    assert torch.equal(total, want_total)
+    assert torch.equal(y, ops.rms_norm_forward(want_total, w, 1e-5))
+    ref = oracle.rms_norm((x.float() + r.float()).to(dtype).float().cpu(), w.float().cpu(), 1e-5)
+    check("add_rmsnorm.y", y, ref, max_abs_tol=1e-5 if dtype == torch.float32 else 2e-2,
+          mean_rel_tol=1e-5 if dtype == torch.float32 else 1e-3)
