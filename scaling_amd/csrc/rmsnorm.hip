@@ -384,7 +384,7 @@ template <typename F> bool dispatch_plan(const Plan& plan, F&& f) {
 #define RMS_CASE(TPRV, CHV) if (plan.tpr == TPRV && plan.ch == CHV) { f(PlanTag<TPRV, CHV>{}); return true; }
     RMS_CASE(16, 1)
     RMS_CASE(64, 1) RMS_CASE(64, 2) RMS_CASE(64, 4) RMS_CASE(64, 8)
-    RMS_CASE(256, 4) RMS_CASE(256, 8)
+    RMS_CASE(256, 1) RMS_CASE(256, 2) RMS_CASE(256, 4) RMS_CASE(256, 8)
 #undef RMS_CASE
     return false;
 }
@@ -396,6 +396,12 @@ int launch_fwd(const void* x, const void* w, void* y, float* rstd, int64_t n_row
     if (!make_plan<T>(hidden, &plan))
         return mi_fail(MI_E_SHAPE, "rmsnorm: hidden=%lld unsupported (must be a multiple of %d and <= %d)",
                        (long long)hidden, Elem<T>::kVec, 256 * 8 * Elem<T>::kVec);
+    // few rows (a decode step): a whole block per row, so that the launch is not eight blocks of long serial threads
+    const int64_t vecs = hidden / Elem<T>::kVec;
+    if (plan.tpr == 64 && plan.ch >= 2 && n_rows <= 1024) {
+        plan.tpr = 256;
+        plan.ch = vecs <= 256 ? 1 : 2;
+    }
     const bool launched = dispatch_plan(plan, [&](auto tag) {
         constexpr int TPR = decltype(tag)::TPR;
         constexpr int CH = decltype(tag)::CH;
