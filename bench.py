@@ -279,6 +279,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--decode-steps", type=int, default=256, help="greedy decode steps of the config-5 workload")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="only run the config-5 decode workload (for a kernel trace of the decode step)")
+    ap.add_argument("--decode-layers", type=int, default=32, help="layers of the config-5 model")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -298,6 +301,10 @@ def main():
         ms = time_gpu(lambda: dst.copy_(src), args.steps, args.warmup)
         print(json.dumps({"calibration": "device copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "ms": ms,
                           "GBs": 2 * (1 << 30) / ms / 1e6}))
+        return
+
+    if args.decode_only:
+        print(json.dumps({"config5_decode": decode_case(args.decode_steps, layers=args.decode_layers)}))
         return
 
     b, s, nq, nkv, d = 1, 8192, 32, 8, 128
@@ -322,7 +329,7 @@ def main():
         extra["config3_gqa_packed_rotary_s8192"] = attention_case(1, 8192, 32, 8, 128, cu3, args.steps, args.warmup, seed=3, rotary=True)
         extra["config3_gqa_packed_rotary_s8192"]["n_docs"] = len(cu3) - 1
         extra.update(bandwidth_cases(args.steps, args.warmup))
-        extra["config5_decode_8b_b32_ctx4096"] = decode_case(args.decode_steps)
+        extra["config5_decode_8b_b32_ctx4096"] = decode_case(args.decode_steps, layers=args.decode_layers)
 
     line = {
         "metric": "attn fwd+bwd TFLOP/s (% bf16 MFMA peak); decode tok/s; norm GB/s (% HBM)",
