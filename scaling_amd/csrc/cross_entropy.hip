@@ -393,13 +393,13 @@ extern "C" {
 int mi_cross_entropy(const void* logits, const int64_t* targets, const float* row_scale, float* losses, float* lse,
                      int32_t* argmax, void* dlogits, int64_t n_rows, int64_t vocab, int64_t logits_row_stride,
                      int64_t dlogits_row_stride, int dtype, void* stream) {
-    if (!logits || !targets) return mi_fail(MI_E_NULL, "cross_entropy: null pointer");
     if (n_rows < 0 || vocab <= 0 || vocab > 0x7fffffffLL)
         return mi_fail(MI_E_SHAPE, "cross_entropy: bad shape [%lld, %lld]", (long long)n_rows, (long long)vocab);
+    if (n_rows == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
+    if (!logits || !targets) return mi_fail(MI_E_NULL, "cross_entropy: null pointer");
     if (n_rows > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "cross_entropy: too many rows");
     if (logits_row_stride < vocab || (dlogits != nullptr && dlogits_row_stride < vocab))
         return mi_fail(MI_E_SHAPE, "cross_entropy: row stride smaller than the vocabulary");
-    if (n_rows == 0) return MI_OK;
     CeArgs a;
     a.logits = logits; a.targets = targets; a.row_scale = row_scale; a.losses = losses; a.lse = lse; a.argmax = argmax;
     a.dlogits = dlogits; a.logits_stride = logits_row_stride; a.dlogits_stride = dlogits_row_stride; a.vocab = (int)vocab;

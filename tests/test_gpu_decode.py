@@ -108,3 +108,31 @@ def test_decode_equals_last_row_of_prefill_kernel():
     torch.cuda.synchronize()
     diff = (out[0].float() - full[n - 1].float()).abs()
     assert float(diff.max()) <= 1.6e-2
+
+
+def test_decode_takes_column_slices_of_a_fused_projection():
+    """q, k_new and v_new as strided column slices of one [B, (nq + 2 nkv) d] tensor (what a single q/k/v GEMM
+    produces) give bit-identical outputs and cache contents to packed copies of the same values."""
+    print("case decode strided operands", flush=True)
+    B, nq, nkv, d, max_ctx = 5, 8, 2, 128, 200
+    g = torch.Generator().manual_seed(5)
+    fused = torch.randn(B, (nq + 2 * nkv) * d, generator=g).bfloat16().to(DEV)
+    q = fused[:, :nq * d].view(B, nq, d)
+    k = fused[:, nq * d:(nq + nkv) * d].view(B, nkv, d)
+    v = fused[:, (nq + nkv) * d:].view(B, nkv, d)
+    assert not q.is_contiguous() and q.stride(0) == (nq + 2 * nkv) * d
+    ctx = torch.tensor([200, 1, 77, 128, 129], dtype=torch.int32, device=DEV)
+    outs, caches = [], []
+    for packed in (False, True):
+        kc = torch.randn(B, max_ctx, nkv, d, generator=torch.Generator().manual_seed(6)).bfloat16().to(DEV)
+        vc = torch.randn(B, max_ctx, nkv, d, generator=torch.Generator().manual_seed(7)).bfloat16().to(DEV)
+        args = (q.contiguous(), kc, vc, ctx, k.contiguous(), v.contiguous()) if packed else (q, kc, vc, ctx, k, v)
+        outs.append(ops.decode_attention(*args))
+        caches.append((kc, vc))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
+    for b in range(B):     # the appended rows landed at ctx - 1
+        assert torch.equal(caches[0][0][b, int(ctx[b]) - 1], k[b]) and torch.equal(caches[0][1][b, int(ctx[b]) - 1], v[b])
+    with pytest.raises(AssertionError):
+        ops.decode_attention(fused.view(B, nq + 2 * nkv, d)[:, ::2], caches[0][0], caches[0][1], ctx)   # heads not contiguous

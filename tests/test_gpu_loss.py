@@ -171,7 +171,7 @@ def test_lm_head_module_loss_equals_head_then_loss():
     io = TransformerLayerIO(activations=x, position_ids=None)
     fused, m_fused = head.loss(io, batch, chunk_rows=32)
     unfused, m_unfused = CrossEntropyLoss()(head(io), batch)
-    assert abs(float(fused) - float(unfused)) < 1e-5 * abs(float(unfused))
+    assert abs(fused.item() - unfused.item()) < 1e-5 * abs(unfused.item())
     assert float(m_fused["accuracy"]) == float(m_unfused["accuracy"])
 
 
@@ -200,3 +200,32 @@ def test_cross_entropy_full_size_properties():
         check(f"cross_entropy.full.row{r}", dl[r].cpu(), ref)
         assert abs(float(losses[r]) - float(torch.logsumexp(x, -1) - x[int(targets[r])])) < 1e-4
         assert int(argmax[r]) == int(x.argmax())
+
+
+def test_cross_entropy_edge_shapes_and_errors():
+    print("case cross_entropy edges", flush=True)
+    # a vocabulary of one: probability 1, loss 0, zero gradient
+    one = torch.randn(4, 1, device=DEV)
+    g = torch.empty_like(one)
+    losses, argmax = ops.cross_entropy_forward(one, torch.zeros(4, dtype=torch.int64, device=DEV), None, g)
+    assert float(losses.abs().max()) == 0.0 and argmax.tolist() == [0] * 4 and float(g.abs().max()) == 0.0
+    # no rows
+    empty = torch.empty(0, 128, device=DEV, dtype=torch.bfloat16)
+    losses, argmax = ops.cross_entropy_forward(empty, torch.empty(0, dtype=torch.int64, device=DEV))
+    assert losses.numel() == 0 and argmax.numel() == 0
+    # fp16 logits through the register-resident kernel
+    gen = torch.Generator().manual_seed(4)
+    x = (torch.randn(9, 4096, generator=gen) * 3).half()
+    t = torch.randint(0, 4096, (9,), generator=gen)
+    dl = torch.empty(9, 4096, dtype=torch.float16, device=DEV)
+    losses, argmax = ops.cross_entropy_forward(x.to(DEV), t.to(DEV), None, dl)
+    ref = torch.nn.functional.cross_entropy(x.float(), t, reduction="none")
+    assert torch.allclose(losses.cpu(), ref, rtol=1e-5, atol=1e-5) and torch.equal(argmax.cpu().long(), x.float().argmax(-1))
+    p = torch.softmax(x.float(), -1)
+    p[torch.arange(9), t] -= 1.0
+    assert torch.allclose(dl.float().cpu(), p, atol=1e-3)
+    # host-side checks
+    with pytest.raises(AssertionError):
+        ops.cross_entropy_forward(x.to(DEV).t(), t.to(DEV))                 # vocabulary dimension not contiguous
+    with pytest.raises(RuntimeError):
+        ops.cross_entropy_forward(x, t)                                       # CPU tensors: there is no CPU path
