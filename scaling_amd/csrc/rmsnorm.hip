@@ -183,21 +183,22 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
     for (int i = threadIdx.x; i < hidden; i += kBlock) out[i] = dw_lds[i];
 }
 
-// Backward for wide rows: 1024 threads per block, TPR (128 or 256) threads per row, so 8 or 4 rows are in
-// flight per block and the per-thread slices (raw row vectors, packed weight, fp32 dweight) are small
-// enough for 16 wavefronts per compute unit; the number of per-block dweight partial rows stays <= 512.
+// Backward for wide rows: 1024 threads per block, TPR (256 or 512) threads per row, so 4 or 2 rows are in
+// flight per block and the per-thread slices (raw row vectors, fp32 dweight) are small enough for 16
+// wavefronts per compute unit; one block per compute unit keeps the number of dweight partial rows <= 256.
 // One barrier per row step (both row sums travel through a double-buffered LDS slot).
-constexpr int kWideBlock = 512;     // two blocks per compute unit: one loads while the other computes
-constexpr int kWideMaxBlocks = 512;
+constexpr int kWideBlock = 512;     // LayerNorm backward: two blocks per compute unit (two barriers per row step)
+constexpr int kRmsWideBlock = 1024; // RMSNorm backward: one block per compute unit, half as many partial dweight rows
+constexpr int kWideMaxBlocks = 256;
 constexpr int kLnMaxBlocks = 512;     // partial dweight / dbias rows of the LayerNorm backward
 
 template <typename T, int TPR, int CH>
-__global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T* __restrict__ x, const T* __restrict__ w,
+__global__ __launch_bounds__(kRmsWideBlock) void rmsnorm_bwd_wide_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                                           const T* __restrict__ dy, T* __restrict__ dx,
                                                                           float* __restrict__ dw_partial, int64_t n_rows,
                                                                           int hidden, float eps) {
     constexpr int V = Elem<T>::kVec;
-    constexpr int RPB = kWideBlock / TPR;
+    constexpr int RPB = kRmsWideBlock / TPR;
     constexpr int WPR = TPR / 64;      // wavefronts per row
     extern __shared__ float dw_lds[];  // [hidden] dweight combine buffer, then [hidden] fp32 copy of the weight
     __shared__ float2 part[2][16];     // [parity][wavefront]
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T
     // the weight is read from LDS where it is used: keeping it in registers would cost as many registers
     // as the dweight accumulator and halve the number of resident wavefronts
     float acc[CH][V];
-    for (int i = threadIdx.x; i < hidden; i += kWideBlock) w_lds[i] = Elem<T>::load1(w + i);
+    for (int i = threadIdx.x; i < hidden; i += kRmsWideBlock) w_lds[i] = Elem<T>::load1(w + i);
 #pragma unroll
     for (int c = 0; c < CH; ++c)
 #pragma unroll
@@ -298,7 +299,7 @@ __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T
             fetch(it + 1, xraw, graw);
         }
     }
-    for (int i = threadIdx.x; i < hidden; i += kWideBlock) dw_lds[i] = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += kRmsWideBlock) dw_lds[i] = 0.f;
     __syncthreads();
     for (int g = 0; g < RPB; ++g) {
         if (rg == g) {
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(kWideBlock, 4) void rmsnorm_bwd_wide_kernel(const T
         __syncthreads();
     }
     float* out = dw_partial + (int64_t)blockIdx.x * hidden;
-    for (int i = threadIdx.x; i < hidden; i += kWideBlock) out[i] = dw_lds[i];
+    for (int i = threadIdx.x; i < hidden; i += kRmsWideBlock) out[i] = dw_lds[i];
 }
 
 // dw[col] = sum_p partial[p][col]; 16 columns x 16 row groups per block, fixed summation order.
@@ -429,7 +430,7 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
     // wide rows: 256 threads per row up to 512 vectors (2 rows per block), the whole block per row beyond
     const int wide_tpr = vecs <= 512 ? 256 : 512;
     // wide rows: a single round of blocks (two per compute unit), each amortising its epilogue over many rows
-    const int wide_rpb = kWideBlock / wide_tpr;
+    const int wide_rpb = kRmsWideBlock / wide_tpr;
     const int64_t wide_blocks = (n_rows + wide_rpb - 1) / wide_rpb;
     const int blocks = wide ? (int)(wide_blocks > kWideMaxBlocks ? kWideMaxBlocks : (wide_blocks < 1 ? 1 : wide_blocks))
                             : bwd_blocks(n_rows, plan.tpr);
@@ -439,7 +440,7 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
     if (wide) {
         const int ch = (int)((vecs + wide_tpr - 1) / wide_tpr);
         const size_t lds = 2 * hidden * sizeof(float);
-#define RMS_WIDE(TPRV, CHV) rmsnorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kWideBlock), lds, st>>>( \
+#define RMS_WIDE(TPRV, CHV) rmsnorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kRmsWideBlock), lds, st>>>( \
             (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps)
         if (wide_tpr == 256) { if (ch <= 1) RMS_WIDE(256, 1); else RMS_WIDE(256, 2); }
         else { if (ch <= 2) RMS_WIDE(512, 2); else RMS_WIDE(512, 4); }
