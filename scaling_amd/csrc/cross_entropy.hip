@@ -239,9 +239,9 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
 }
 
 // Forward only (no gradient asked for): nothing of the row has to be kept, so each thread streams its vectors
-// once with a running (max, sum) pair and the pairs are merged at the end.  256 threads per row and several
+// once with a running (max, sum) pair and the pairs are merged at the end.  512 threads per row and several
 // rows per compute unit keep loads in flight under the arithmetic.
-constexpr int kFwdBlock = 256;
+constexpr int kFwdBlock = 512;
 constexpr int kFwdDepth = 4;        // vectors in flight per thread
 
 template <typename T>
