@@ -2,10 +2,13 @@
 // gradient with respect to the logits in one launch.  HBM-bound: a row is read once and, when the gradient is
 // asked for, written once.
 //
-// Fast path: one 1024-thread workgroup per row keeps the whole row in registers (up to 16 x 128-bit vectors per
-// thread, i.e. 131072 16-bit or 65536 fp32 logits), so max, sum of exponentials and the gradient all come from
-// the single read.  Anything else (rows that do not fit, unaligned rows, vocab not a multiple of the vector
-// width) takes the streaming kernel, which re-reads the row for each of its three passes.
+// Three kernels:
+//   ce_row_kernel     gradient asked for: 1024-thread workgroups (one per compute unit) walk the rows; a row stays in
+//                     registers (up to 16 x 128-bit vectors per thread, i.e. 131072 16-bit or 65536 fp32 logits), so
+//                     max, sum of exponentials and the gradient all come from the single read
+//   ce_fwd_kernel     no gradient: 512-thread workgroups stream a row once with a running (max, sum)
+//   ce_stream_kernel  anything else (rows that do not fit, unaligned rows, vocab not a multiple of the vector width):
+//                     scalar accesses, the row is re-read for each of three passes
 #include "common.h"
 
 namespace {
