@@ -80,16 +80,19 @@ int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, 
 /* ------------------------------------------------------------------------------------------
  * LayerNorm.  Replaces core/nn/norm/layernorm.py:75-86 (torch.nn.functional.layer_norm over the last
  * dimension):  y = (x - mean) * rsqrt(var + eps) * weight + bias, biased variance, fp32 arithmetic, one
- * rounding to `dtype` on store.  bias may be NULL.  Backward recomputes mean / rstd from x:
+ * rounding to `dtype` on store.  bias may be NULL.  `mean` / `rstd` (fp32 [n_rows], both or neither; may be
+ * NULL) receive the row statistics, the two tensors torch.native_layer_norm saves for its backward.
  *   dx = rstd * (dy*w - mean(dy*w) - xhat * mean(dy*w*xhat)),  dweight = sum_rows dy*xhat,  dbias = sum_rows dy
- * (dbias may be NULL).  `workspace`: fp32, at least mi_layernorm_bwd_workspace_bytes(n_rows, hidden) bytes;
- * partial sums are reduced in a fixed order.  Algorithmic HBM bytes as for RMSNorm.
+ * (dbias may be NULL).  The backward takes the saved `mean` / `rstd` (then a row needs one reduction instead
+ * of two) or, when both are NULL, recomputes them from x.  `workspace`: fp32, at least
+ * mi_layernorm_bwd_workspace_bytes(n_rows, hidden) bytes; partial sums are reduced in a fixed order.
+ * Algorithmic HBM bytes as for RMSNorm.
  * ------------------------------------------------------------------------------------------ */
-int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* y,
+int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* y, float* mean, float* rstd,
                      int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
 size_t mi_layernorm_bwd_workspace_bytes(int64_t n_rows, int64_t hidden);
-int mi_layernorm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dweight, void* dbias,
-                     void* workspace, size_t workspace_bytes,
+int mi_layernorm_bwd(const void* x, const void* weight, const void* dy, const float* mean, const float* rstd,
+                     void* dx, void* dweight, void* dbias, void* workspace, size_t workspace_bytes,
                      int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------

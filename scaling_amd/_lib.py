@@ -92,12 +92,13 @@ def _declare(lib):
     lib.mi_rmsnorm_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int64,
                                    c_int64, c_float, c_int, c_void_p]
     lib.mi_layernorm_fwd.restype = c_int
-    lib.mi_layernorm_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_int, c_void_p]
+    lib.mi_layernorm_fwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float,
+                                     c_int, c_void_p]
     lib.mi_layernorm_bwd_workspace_bytes.restype = c_size_t
     lib.mi_layernorm_bwd_workspace_bytes.argtypes = [c_int64, c_int64]
     lib.mi_layernorm_bwd.restype = c_int
-    lib.mi_layernorm_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
-                                     c_int64, c_int64, c_float, c_int, c_void_p]
+    lib.mi_layernorm_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_void_p, c_size_t, c_int64, c_int64, c_float, c_int, c_void_p]
     lib.mi_gelu_fwd.restype = c_int
     lib.mi_gelu_fwd.argtypes = [c_void_p, c_void_p, c_int64, c_int, c_void_p]
     lib.mi_gelu_bwd.restype = c_int

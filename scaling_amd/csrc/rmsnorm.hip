@@ -471,6 +471,7 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
 template <typename T, int TPR, int CH>
 __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                                 const T* __restrict__ b, T* __restrict__ y,
+                                                                float* __restrict__ mean_out, float* __restrict__ rstd_out,
                                                                 int64_t n_rows, int hidden, float eps) {
     constexpr int V = Elem<T>::kVec;
     constexpr int RPB = kBlock / TPR;
@@ -504,6 +505,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(const T* __restri
     }
     const float rstd = rsqrtf(row_sum<TPR>(sq, lds) * inv_h + eps);
     if (!row_ok) return;
+    if (mean_out != nullptr && tr == 0) { mean_out[row] = mean; rstd_out[row] = rstd; }
     const uint4* wr = reinterpret_cast<const uint4*>(w);
     const uint4* br = reinterpret_cast<const uint4*>(b);
     uint4* yr = reinterpret_cast<uint4*>(y + row * hidden);
@@ -782,8 +784,143 @@ __global__ __launch_bounds__(kWideBlock, 4) void layernorm_bwd_wide_kernel(const
     for (int i = threadIdx.x; i < hidden; i += kWideBlock) { out_w[i] = comb_lds[i]; out_b[i] = comb_lds[hidden + i]; }
 }
 
+// Backward for wide rows when the forward pass saved mean and rstd: the two row sums (g*w and g*w*xhat) no
+// longer wait for the statistics, so a row step takes one block-wide reduction, as in rmsnorm_bwd_wide_kernel
+// (same block shape: kRmsWideBlock threads, one block per compute unit, one barrier per row step).
+template <typename T, int TPR, int CH>
+__global__ __launch_bounds__(kRmsWideBlock) void layernorm_bwd_stats_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                             const T* __restrict__ dy,
+                                                                             const float* __restrict__ mean_in,
+                                                                             const float* __restrict__ rstd_in, T* __restrict__ dx,
+                                                                             float* __restrict__ partial, int64_t n_rows,
+                                                                             int hidden) {
+    constexpr int V = Elem<T>::kVec;
+    constexpr int RPB = kRmsWideBlock / TPR;
+    constexpr int WPR = TPR / 64;
+    extern __shared__ float comb_lds[];   // [hidden] dweight, [hidden] dbias, then [hidden] fp32 copy of the weight
+    __shared__ float2 part[2][16];        // [parity][wavefront]: sum g*w, sum g*w*xhat
+    float* w_lds = comb_lds + 2 * hidden;
+    const int tr = threadIdx.x % TPR;
+    const int rg = threadIdx.x / TPR;
+    const int wave = threadIdx.x >> 6;
+    const int vecs = hidden / V;
+    const float inv_h = 1.0f / (float)hidden;
+
+    float acc_w[CH][V], acc_b[CH][V];
+    for (int i = threadIdx.x; i < hidden; i += kRmsWideBlock) w_lds[i] = Elem<T>::load1(w + i);
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int i = 0; i < V; ++i) { acc_w[c][i] = 0.f; acc_b[c][i] = 0.f; }
+    __syncthreads();
+    const int64_t row_step = (int64_t)gridDim.x * RPB;
+    const int64_t iters = (n_rows + row_step - 1) / row_step;
+    uint4 xraw[CH], graw[CH], xnext[CH], gnext[CH];
+    float mean = 0.f, rstd = 0.f, mean_next = 0.f, rstd_next = 0.f;
+    auto fetch = [&](int64_t it, uint4 (&xv)[CH], uint4 (&gv)[CH], float& mu, float& rs) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        const uint4* xr = reinterpret_cast<const uint4*>(x + (row_ok ? row : 0) * hidden);
+        const uint4* gr = reinterpret_cast<const uint4*>(dy + (row_ok ? row : 0) * hidden);
+        mu = mean_in[row_ok ? row : 0];
+        rs = rstd_in[row_ok ? row : 0];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int v = c * TPR + tr;
+            const bool ok = row_ok && v < vecs;
+            xv[c] = ok ? xr[v] : make_uint4(0, 0, 0, 0);
+            gv[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
+        }
+    };
+    if (iters > 0) fetch(0, xraw, graw, mean, rstd);
+    for (int64_t it = 0; it < iters; ++it) {
+        const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
+        const bool row_ok = row < n_rows;
+        if (it + 1 < iters) fetch(it + 1, xnext, gnext, mean_next, rstd_next);
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float xf[V], gf[V], wf[V];
+            Elem<T>::unpack(xraw[c], xf);
+            Elem<T>::unpack(graw[c], gf);
+            const int v0 = (c * TPR + tr < vecs ? c * TPR + tr : 0) * V;
+#pragma unroll
+            for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v0 + i);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const float gw = gf[i] * wf[i];       // zero where the row or the vector is out of range
+                s1 += gw;
+                s2 += gw * ((xf[i] - mean) * rstd);
+            }
+        }
+        s1 = group_sum<64>(s1);
+        s2 = group_sum<64>(s2);
+        const int par = (int)(it & 1);
+        if ((threadIdx.x & 63) == 0) part[par][wave] = make_float2(s1, s2);
+        __syncthreads();
+        s1 = 0.f;
+        s2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < WPR; ++j) {
+            const float2 pj = part[par][WPR * rg + j];
+            s1 += pj.x;
+            s2 += pj.y;
+        }
+        s1 *= inv_h;
+        s2 *= inv_h;
+        if (row_ok) {
+            uint4* dxr = reinterpret_cast<uint4*>(dx + row * hidden);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+                    float xf[V], gf[V], wf[V], o[V];
+                    Elem<T>::unpack(xraw[c], xf);
+                    Elem<T>::unpack(graw[c], gf);
+#pragma unroll
+                    for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v * V + i);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        const float xhat = (xf[i] - mean) * rstd;
+                        o[i] = rstd * (gf[i] * wf[i] - s1 - xhat * s2);
+                        acc_w[c][i] += gf[i] * xhat;
+                        acc_b[c][i] += gf[i];
+                    }
+                    dxr[v] = Elem<T>::pack(o);
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c) { xraw[c] = xnext[c]; graw[c] = gnext[c]; }
+        mean = mean_next;
+        rstd = rstd_next;
+    }
+    for (int i = threadIdx.x; i < 2 * hidden; i += kRmsWideBlock) comb_lds[i] = 0.f;
+    __syncthreads();
+    for (int g = 0; g < RPB; ++g) {
+        if (rg == g) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int v = c * TPR + tr;
+                if (v < vecs) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        comb_lds[v * V + i] += acc_w[c][i];
+                        comb_lds[hidden + v * V + i] += acc_b[c][i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out_w = partial + (int64_t)blockIdx.x * hidden;
+    float* out_b = partial + ((int64_t)gridDim.x + blockIdx.x) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += kRmsWideBlock) { out_w[i] = comb_lds[i]; out_b[i] = comb_lds[hidden + i]; }
+}
+
 template <typename T>
-int launch_ln_fwd(const void* x, const void* w, const void* b, void* y, int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
+int launch_ln_fwd(const void* x, const void* w, const void* b, void* y, float* mean, float* rstd, int64_t n_rows,
+                  int64_t hidden, float eps, hipStream_t st) {
     Plan plan;
     if (!make_plan<T>(hidden, &plan))
         return mi_fail(MI_E_SHAPE, "layernorm: hidden=%lld unsupported (must be a multiple of %d and <= %d)",
@@ -794,30 +931,41 @@ int launch_ln_fwd(const void* x, const void* w, const void* b, void* y, int64_t 
         const int rpb = kBlock / TPR;
         const unsigned grid = (unsigned)((n_rows + rpb - 1) / rpb);
         layernorm_fwd_kernel<T, TPR, CH><<<dim3(grid), dim3(kBlock), 0, st>>>((const T*)x, (const T*)w, (const T*)b, (T*)y,
-                                                                              n_rows, (int)hidden, eps);
+                                                                              mean, rstd, n_rows, (int)hidden, eps);
     });
     if (!launched) return mi_fail(MI_E_SHAPE, "layernorm: no kernel for hidden=%lld", (long long)hidden);
     return mi_check_launch("layernorm_fwd");
 }
 
 template <typename T>
-int launch_ln_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw, void* db, void* ws, size_t ws_bytes,
-                  int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
+int launch_ln_bwd(const void* x, const void* w, const void* dy, const float* mean, const float* rstd, void* dx, void* dw,
+                  void* db, void* ws, size_t ws_bytes, int64_t n_rows, int64_t hidden, float eps, hipStream_t st) {
     Plan plan;
     if (!make_plan<T>(hidden, &plan)) return mi_fail(MI_E_SHAPE, "layernorm: hidden=%lld unsupported", (long long)hidden);
     const int64_t vecs = hidden / Elem<T>::kVec;
     const bool wide = vecs >= 256 && vecs <= 1024 && (size_t)3 * hidden * sizeof(float) <= 159 * 1024;
     const int wide_tpr = vecs <= 512 ? 256 : 512;
-    const int wide_rpb = kWideBlock / wide_tpr;
+    // saved statistics (wide rows only; narrower rows recompute them, which costs them nothing measurable)
+    const bool stats = wide && mean != nullptr;
+    const int wide_rpb = (stats ? kRmsWideBlock : kWideBlock) / wide_tpr;
+    const int wide_max = stats ? kWideMaxBlocks : kLnMaxBlocks;
     const int64_t wide_blocks = (n_rows + wide_rpb - 1) / wide_rpb;
-    int blocks = wide ? (int)(wide_blocks > kLnMaxBlocks ? kLnMaxBlocks : (wide_blocks < 1 ? 1 : wide_blocks))
+    int blocks = wide ? (int)(wide_blocks > wide_max ? wide_max : (wide_blocks < 1 ? 1 : wide_blocks))
                       : bwd_blocks(n_rows, plan.tpr);
     if (blocks > kLnMaxBlocks) blocks = kLnMaxBlocks;
     if (ws == nullptr || ws_bytes < (size_t)2 * blocks * hidden * sizeof(float))
         return mi_fail(MI_E_WORKSPACE, "layernorm_bwd: workspace needs %zu bytes, got %zu",
                        (size_t)2 * blocks * hidden * sizeof(float), ws_bytes);
     bool launched = true;
-    if (wide) {
+    if (stats) {
+        const int ch = (int)((vecs + wide_tpr - 1) / wide_tpr);
+        const size_t lds = 3 * hidden * sizeof(float);
+#define LN_STATS(TPRV, CHV) layernorm_bwd_stats_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kRmsWideBlock), lds, st>>>( \
+            (const T*)x, (const T*)w, (const T*)dy, mean, rstd, (T*)dx, (float*)ws, n_rows, (int)hidden)
+        if (wide_tpr == 256) { if (ch <= 1) LN_STATS(256, 1); else LN_STATS(256, 2); }
+        else LN_STATS(512, 2);
+#undef LN_STATS
+    } else if (wide) {
         const int ch = (int)((vecs + wide_tpr - 1) / wide_tpr);
         const size_t lds = 3 * hidden * sizeof(float);
 #define LN_WIDE(TPRV, CHV) layernorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kWideBlock), lds, st>>>( \
@@ -885,14 +1033,15 @@ int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, 
     return MI_OK;
 }
 
-int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* y, int64_t n_rows, int64_t hidden,
-                     float eps, int dtype, void* stream) {
+int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* y, float* mean, float* rstd,
+                     int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream) {
     if (!x || !weight || !y) return mi_fail(MI_E_NULL, "layernorm_fwd: null pointer");
+    if ((mean == nullptr) != (rstd == nullptr)) return mi_fail(MI_E_NULL, "layernorm_fwd: mean and rstd go together");
     if (n_rows < 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "layernorm_fwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
     if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(y) || (bias && !mi_aligned16(bias)))
         return mi_fail(MI_E_ALIGN, "layernorm_fwd: pointers must be 16-byte aligned");
     if (n_rows == 0) return MI_OK;
-    MI_DISPATCH_DTYPE(dtype, return launch_ln_fwd<T>(x, weight, bias, y, n_rows, hidden, eps, (hipStream_t)stream));
+    MI_DISPATCH_DTYPE(dtype, return launch_ln_fwd<T>(x, weight, bias, y, mean, rstd, n_rows, hidden, eps, (hipStream_t)stream));
     return MI_OK;
 }
 
@@ -901,16 +1050,17 @@ size_t mi_layernorm_bwd_workspace_bytes(int64_t n_rows, int64_t hidden) {
     return (size_t)2 * kLnMaxBlocks * (size_t)(hidden > 0 ? hidden : 0) * sizeof(float);
 }
 
-int mi_layernorm_bwd(const void* x, const void* weight, const void* dy, void* dx, void* dweight, void* dbias,
-                     void* workspace, size_t workspace_bytes, int64_t n_rows, int64_t hidden, float eps, int dtype,
-                     void* stream) {
+int mi_layernorm_bwd(const void* x, const void* weight, const void* dy, const float* mean, const float* rstd, void* dx,
+                     void* dweight, void* dbias, void* workspace, size_t workspace_bytes, int64_t n_rows, int64_t hidden,
+                     float eps, int dtype, void* stream) {
     if (!x || !weight || !dy || !dx || !dweight) return mi_fail(MI_E_NULL, "layernorm_bwd: null pointer");
+    if ((mean == nullptr) != (rstd == nullptr)) return mi_fail(MI_E_NULL, "layernorm_bwd: mean and rstd go together");
     if (n_rows <= 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "layernorm_bwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
     if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(dy) || !mi_aligned16(dx) || !mi_aligned16(workspace))
         return mi_fail(MI_E_ALIGN, "layernorm_bwd: pointers must be 16-byte aligned");
     if (2 * hidden * sizeof(float) > 160 * 1024 - 256) return mi_fail(MI_E_SHAPE, "layernorm_bwd: hidden too large for LDS");
-    MI_DISPATCH_DTYPE(dtype, return launch_ln_bwd<T>(x, weight, dy, dx, dweight, dbias, workspace, workspace_bytes, n_rows,
-                                                     hidden, eps, (hipStream_t)stream));
+    MI_DISPATCH_DTYPE(dtype, return launch_ln_bwd<T>(x, weight, dy, mean, rstd, dx, dweight, dbias, workspace, workspace_bytes,
+                                                     n_rows, hidden, eps, (hipStream_t)stream));
     return MI_OK;
 }
 

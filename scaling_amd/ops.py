@@ -92,21 +92,31 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.
 # ------------------------------------------------------------------------------------------------
 # LayerNorm, GELU (the reference's default norm / activation)
 # ------------------------------------------------------------------------------------------------
-def layer_norm_forward(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+def layer_norm_forward(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                       save_stats: bool = False):
+    """y, or (y, stats) with stats an fp32 [2, n_rows] tensor (row means, then reciprocal standard deviations)
+    for layer_norm_backward when save_stats is set."""
     _need_cuda(x, weight, bias)
     assert x.shape[-1] == weight.shape[0] and weight.dtype == x.dtype
     x2 = x.contiguous().view(-1, x.shape[-1])
     w = weight.contiguous()
     b = bias.contiguous() if bias is not None else None
     y = torch.empty_like(x2)
-    check(_lib.load().mi_layernorm_fwd(ptr(x2), ptr(w), ptr(b), ptr(y), x2.shape[0], x2.shape[1], float(eps),
+    stats = torch.empty(2, x2.shape[0], dtype=torch.float32, device=x.device) if save_stats else None
+    check(_lib.load().mi_layernorm_fwd(ptr(x2), ptr(w), ptr(b), ptr(y), ptr(stats[0]) if save_stats else None,
+                                       ptr(stats[1]) if save_stats else None, x2.shape[0], x2.shape[1], float(eps),
                                        dtype_code(x.dtype), stream_ptr()), "mi_layernorm_fwd")
-    return y.view(x.shape)
+    return (y.view(x.shape), stats) if save_stats else y.view(x.shape)
 
 
-def layer_norm_backward(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor, eps: float, need_bias_grad: bool = True):
+def layer_norm_backward(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor, eps: float, need_bias_grad: bool = True,
+                        stats: Optional[torch.Tensor] = None):
+    """(dx, dweight, dbias).  `stats` is what layer_norm_forward(save_stats=True) returned for the same x, or
+    None to have the statistics recomputed."""
     _need_cuda(x, weight, dy)
     lib = _lib.load()
+    if stats is not None:
+        assert stats.dtype == torch.float32 and stats.is_contiguous() and stats.shape == (2, x.numel() // x.shape[-1])
     x2 = x.contiguous().view(-1, x.shape[-1])
     dy2 = dy.contiguous().view(-1, x.shape[-1])
     w = weight.contiguous()
@@ -115,23 +125,25 @@ def layer_norm_backward(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor,
     db = torch.empty_like(w) if need_bias_grad else None
     nbytes = lib.mi_layernorm_bwd_workspace_bytes(x2.shape[0], x2.shape[1])
     ws = torch.empty(nbytes // 4, dtype=torch.float32, device=x.device)
-    check(lib.mi_layernorm_bwd(ptr(x2), ptr(w), ptr(dy2), ptr(dx), ptr(dw), ptr(db), ptr(ws), nbytes, x2.shape[0],
-                               x2.shape[1], float(eps), dtype_code(x.dtype), stream_ptr()), "mi_layernorm_bwd")
+    check(lib.mi_layernorm_bwd(ptr(x2), ptr(w), ptr(dy2), ptr(stats[0]) if stats is not None else None,
+                               ptr(stats[1]) if stats is not None else None, ptr(dx), ptr(dw), ptr(db), ptr(ws), nbytes,
+                               x2.shape[0], x2.shape[1], float(eps), dtype_code(x.dtype), stream_ptr()), "mi_layernorm_bwd")
     return dx.view(x.shape), dw, db
 
 
 class _LayerNorm(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, eps):
-        ctx.save_for_backward(x, weight)
+        y, stats = layer_norm_forward(x, weight, bias, eps, save_stats=True)
+        ctx.save_for_backward(x, weight, stats)
         ctx.eps = eps
         ctx.has_bias = bias is not None
-        return layer_norm_forward(x, weight, bias, eps)
+        return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, weight = ctx.saved_tensors
-        dx, dw, db = layer_norm_backward(x, weight, dy, ctx.eps, ctx.has_bias)
+        x, weight, stats = ctx.saved_tensors
+        dx, dw, db = layer_norm_backward(x, weight, dy, ctx.eps, ctx.has_bias, stats)
         return dx, dw, db, None
 
 

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import oracle
-from scaling_amd import ops
+from scaling_amd import _lib, ops
 from tests.parity import check
 
 pytestmark = pytest.mark.gpu
@@ -201,6 +201,45 @@ def test_layernorm_parity(rows, hidden, dtype, with_bias):
     check("layernorm.dw", wg.grad, ref[2], ref_o[2], **tol)
     if with_bias:
         check("layernorm.db", bg.grad, ref[3], ref_o[3], **tol)
+
+
+@pytest.mark.parametrize("rows,hidden", [(1024, 4096), (19, 8192), (5, 8000), (3000, 2048), (37, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_layernorm_saved_statistics_and_recomputed_backward_agree(rows, hidden, dtype):
+    """The backward runs with the statistics the forward saved (what the autograd function does) or
+    recomputes them when none are passed: both must match the oracle, and the saved statistics are the row
+    mean and 1 / sqrt(biased variance + eps) (torch.native_layer_norm's second and third results)."""
+    print(f"case layernorm stats rows={rows} hidden={hidden} dtype={dtype}", flush=True)
+    g = torch.Generator().manual_seed(rows + 3 * hidden)
+    x = (_rand(g, rows, hidden, dtype=torch.float32) * 1.5 - 2.0).to(dtype)
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(hidden, generator=g)).to(dtype)
+    dy = _rand(g, rows, hidden, dtype=dtype)
+    xr, wr, br = x.float().requires_grad_(), w.float().requires_grad_(), b.float().requires_grad_()
+    oracle.layer_norm(xr, wr, br, 1e-5).backward(dy.float())
+    _, mean_ref, rstd_ref = torch.native_layer_norm(x.float(), [hidden], w.float(), b.float(), 1e-5)
+
+    xg, wg, bg, dyg = x.to(DEV), w.to(DEV), b.to(DEV), dy.to(DEV)
+    y, stats = ops.layer_norm_forward(xg, wg, bg, 1e-5, save_stats=True)
+    assert torch.equal(y, ops.layer_norm_forward(xg, wg, bg, 1e-5))
+    assert stats.shape == (2, rows) and stats.dtype == torch.float32
+    assert torch.allclose(stats[0].cpu(), mean_ref.view(-1), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(stats[1].cpu(), rstd_ref.view(-1), rtol=1e-5, atol=0)
+    tol = dict(max_abs_tol=2e-2, mean_rel_tol=1e-3) if dtype == torch.bfloat16 else dict(max_abs_tol=1e-4, mean_rel_tol=1e-5)
+    for name, st in (("saved", stats), ("recomputed", None)):
+        dx, dw, db = ops.layer_norm_backward(xg, wg, dyg, 1e-5, True, st)
+        torch.cuda.synchronize()
+        check(f"layernorm[{name}].dx", dx, xr.grad, **tol)
+        check(f"layernorm[{name}].dw", dw, wr.grad, **tol)
+        check(f"layernorm[{name}].db", db, br.grad, **tol)
+    # half of a pair is refused
+    lib = _lib.load()
+    ws = torch.empty(lib.mi_layernorm_bwd_workspace_bytes(rows, hidden) // 4, dtype=torch.float32, device=DEV)
+    dx = torch.empty_like(xg)
+    rc = lib.mi_layernorm_bwd(xg.data_ptr(), wg.data_ptr(), dyg.data_ptr(), stats[0].data_ptr(), None, dx.data_ptr(),
+                              dx.data_ptr(), None, ws.data_ptr(), ws.numel() * 4, rows, hidden, 1e-5,
+                              _lib.dtype_code(dtype), torch.cuda.current_stream().cuda_stream)
+    assert rc == -1 and "mean and rstd" in lib.mi_last_error().decode()   # MI_E_NULL
 
 
 @pytest.mark.parametrize("shape", [(2, 128, 1024), (3, 7, 5), (4, 1000, 4096), (1, 1, 8)])
