@@ -172,7 +172,10 @@ int mi_rotary_complex(const void* x, void* out, const float* cos, const float* s
  *
  * Fused rotary (optional): if rotary_cos != NULL, q and k are rotated on load (rotate-half, the
  * whole head_dim; tables [rotary_table_rows, head_dim] in the I/O dtype; position ids int64 per
- * token, required).  Supported: dtype MI_BF16, head_dim in {64, 128}.
+ * token, required).  With rotary_interleaved != 0 the rotation is the interleaved-pair ("complex")
+ * one of core/nn/rotary.py:59-90 instead: pairs (2i, 2i+1), fp32 tables [rotary_table_rows,
+ * head_dim / 2] (real and imaginary part of freqs_cis), fp32 arithmetic, one rounding -- the same
+ * bits as mi_rotary_complex followed by the plain call.  Supported: dtype MI_BF16, head_dim in {64, 128}.
  * Algorithmic work: 4 * head_dim * n_q_heads * P flop forward, 10 * head_dim * n_q_heads * P backward,
  * P = number of allowed (query, key) pairs per head.
  * ------------------------------------------------------------------------------------------ */
@@ -221,6 +224,7 @@ typedef struct mi_attn_args {
      * Not available together with the fused rotary of the forward. */
     float dropout_p;
     uint64_t dropout_seed;
+    int32_t rotary_interleaved;    /* fused rotary: 0 = rotate-half, 1 = interleaved pairs with fp32 tables */
 } mi_attn_args;
 
 int mi_attn_fwd(const mi_attn_args* args);
@@ -254,7 +258,8 @@ int mi_attn_bwd(const mi_attn_bwd_args* args);
  *
  * If k_new/v_new != NULL the kernel first appends them at position ctx_len[b]-1 (in-place append
  * instead of torch.cat); with rotary_cos != NULL it rotates q and k_new by position_ids[b] before
- * use/append (fused rotary).  o: [batch, n_q_heads, head_dim] contiguous; q likewise unless q_stride_batch is set.
+ * use/append (fused rotary; rotary_interleaved selects the pairing and table format as in mi_attn_args).
+ * o: [batch, n_q_heads, head_dim] contiguous; q likewise unless q_stride_batch is set.
  * The key axis is split into n_splits chunks processed by different workgroups and merged by a
  * second kernel; workspace = mi_attn_decode_workspace_bytes() bytes of fp32 scratch.
  * Algorithmic HBM bytes: 2 * sum_b ctx_len[b] * n_kv_heads * head_dim * e  (K and V read once).
@@ -267,7 +272,7 @@ typedef struct mi_decode_args {
     const int32_t* ctx_len;        /* device, [batch] */
     const void* k_new;             /* [batch, n_kv_heads, head_dim] or NULL */
     const void* v_new;
-    const void* rotary_cos;        /* [rotary_table_rows, head_dim] or NULL */
+    const void* rotary_cos;        /* [rotary_table_rows, head_dim] ([.., head_dim / 2] fp32 when interleaved) or NULL */
     const void* rotary_sin;
     const int64_t* position_ids;   /* device, [batch]; required with rotary */
     int64_t rotary_table_rows;
@@ -286,6 +291,7 @@ typedef struct mi_decode_args {
     /* element strides between the sequences of q / k_new / v_new (their [heads, head_dim] part stays contiguous);
      * 0 = packed ([batch, heads, head_dim] contiguous).  Lets q, k and v be column slices of one fused projection. */
     int64_t q_stride_batch, k_new_stride_batch, v_new_stride_batch;
+    int32_t rotary_interleaved;    /* fused rotary: 0 = rotate-half, 1 = interleaved pairs with fp32 tables */
 } mi_decode_args;
 
 size_t mi_attn_decode_workspace_bytes(int32_t batch, int32_t n_q_heads, int32_t head_dim, int32_t max_ctx);

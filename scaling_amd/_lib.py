@@ -42,7 +42,7 @@ class MiAttnArgs(Structure):
         ("position_ids_q", c_void_p), ("position_ids_k", c_void_p),
         ("rotary_table_rows", c_int64),
         ("stream", c_void_p),
-        ("dropout_p", c_float), ("dropout_seed", c_uint64),
+        ("dropout_p", c_float), ("dropout_seed", c_uint64), ("rotary_interleaved", c_int32),
     ]
 
 
@@ -69,6 +69,7 @@ class MiDecodeArgs(Structure):
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("stream", c_void_p),
         ("q_stride_batch", c_int64), ("k_new_stride_batch", c_int64), ("v_new_stride_batch", c_int64),
+        ("rotary_interleaved", c_int32),
     ]
 
 

@@ -22,6 +22,7 @@ struct AttnParams {
     int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;
     float scale_log2;   // softmax_scale * log2(e)
     const __bf16* cos; const __bf16* sin; const int64_t* pos_q; const int64_t* pos_k; int table_rows;
+    const float* cos32; const float* sin32;   // interleaved-pair rotary: fp32 tables [table_rows, head_dim / 2]
     // backward only
     const __bf16* d_o; __bf16* dq; __bf16* dk; __bf16* dv; float* delta;
     int64_t dk_st, dk_sh, dv_st, dv_sh;
@@ -296,6 +297,19 @@ __device__ __forceinline__ void rotate_pair(uint4& lo, uint4& hi, const uint4& c
         const float sa = sign * bf16_lo(sw[i]), sb = sign * bf16_hi(sw[i]);
         l[i] = pack_bf16x2(x0a * ca - x1a * sa, x0b * cb - x1b * sb);
         h[i] = pack_bf16x2(x1a * ca + x0a * sa, x1b * cb + x0b * sb);
+    }
+}
+
+// interleaved-pair rotary of one 8-element vector = 4 pairs (2i, 2i+1); c / s hold the 4 fp32 table values
+__device__ __forceinline__ void rotate_interleaved(uint4& v, const uint4& c, const uint4& s, float sign) {
+    uint32_t* w = reinterpret_cast<uint32_t*>(&v);
+    const uint32_t* cw = reinterpret_cast<const uint32_t*>(&c);
+    const uint32_t* sw = reinterpret_cast<const uint32_t*>(&s);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float x0 = bf16_lo(w[i]), x1 = bf16_hi(w[i]);
+        rotate_complex_pair(x0, x1, __uint_as_float(cw[i]), sign * __uint_as_float(sw[i]));
+        w[i] = pack_bf16x2(x0, x1);
     }
 }
 

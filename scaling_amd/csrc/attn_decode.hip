@@ -24,6 +24,7 @@ struct DecodeParams {
     const int32_t* ctx_len;
     const __bf16* k_new; const __bf16* v_new;
     const __bf16* cos; const __bf16* sin; const int64_t* pos; int table_rows;
+    const float* cos32; const float* sin32;   // interleaved-pair rotary: fp32 tables [table_rows, D / 2]
     int batch, max_ctx, nq, nkv, n_rep, n_splits;
     int64_t c_sb, c_st, c_sh;
     int64_t q_sb, kn_sb, vn_sb;   // element strides between sequences of q / k_new / v_new
@@ -57,6 +58,13 @@ __global__ void decode_append_kernel(const DecodeParams p) {
         const uint4 cv = *reinterpret_cast<const uint4*>(p.cos + pos * D + 8 * c);
         const uint4 sv = *reinterpret_cast<const uint4*>(p.sin + pos * D + 8 * c);
         rotate_pair(lo, hi, cv, sv, 1.0f);
+    } else if (p.cos32 != nullptr) {
+        int64_t pos = p.pos[b];
+        pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+        const float* cr = p.cos32 + pos * (D / 2) + 4 * c;   // features 8 c .. + 8 = pairs 4 c .. + 4
+        const float* sr = p.sin32 + pos * (D / 2) + 4 * c;
+        rotate_interleaved(lo, ld128(cr), ld128(sr), 1.0f);
+        rotate_interleaved(hi, ld128(cr + D / 4), ld128(sr + D / 4), 1.0f);
     }
     *reinterpret_cast<uint4*>(p.kc + dst) = lo;
     *reinterpret_cast<uint4*>(p.kc + dst + D / 2) = hi;
@@ -67,7 +75,8 @@ __global__ void decode_append_kernel(const DecodeParams p) {
 // ---- split kernel ----------------------------------------------------------------------------------
 // NWV wavefronts (4 or 8) share the keys of one (batch, KV head, split); with a single split the merged result
 // is the attention output and goes straight to `o`, otherwise the partial goes to the workspace.
-template <int D, bool ROT, int NWV>
+// ROT: 0 = q as it is, 1 = rotate-half rotary on the q load, 2 = interleaved-pair rotary on the q load.
+template <int D, int ROT, int NWV>
 __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeParams p) {
     constexpr int kThreads = 64 * NWV;
     constexpr int KS = D / 32;          // contraction steps of Q K^T (32 features each)
@@ -105,7 +114,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qr + 32 * ks);
-        if constexpr (ROT) {
+        if constexpr (ROT == 1) {
             int64_t pos = p.pos[b];
             pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
 #pragma unroll
@@ -113,6 +122,15 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
                 const uint4 cv = *reinterpret_cast<const uint4*>(p.cos + pos * D + 32 * ks + 8 * G);
                 const uint4 sv = *reinterpret_cast<const uint4*>(p.sin + pos * D + 32 * ks + 8 * G);
                 rotate_pair(raw[ks], raw[ks + KS / 2], cv, sv, 1.0f);
+            }
+        } else if constexpr (ROT == 2) {
+            int64_t pos = p.pos[b];
+            pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {   // features 32 ks + 8 G .. + 8 = pairs 16 ks + 4 G .. + 4
+                const float* cr = p.cos32 + pos * (D / 2) + 16 * ks + 4 * G;
+                const float* sr = p.sin32 + pos * (D / 2) + 16 * ks + 4 * G;
+                rotate_interleaved(raw[ks], ld128(cr), ld128(sr), 1.0f);
             }
         }
 #pragma unroll
@@ -306,18 +324,16 @@ int choose_splits(int batch, int nkv, int max_ctx) {
     return (int)s;
 }
 
-template <int D, int NWV> int launch_split(const DecodeParams& p, bool rot, hipStream_t st) {
+// rot: 0 = none, 1 = rotate-half, 2 = interleaved pairs
+template <int D, int NWV> int launch_split(const DecodeParams& p, int rot, hipStream_t st) {
     const unsigned grid = (unsigned)p.batch * p.nkv * p.n_splits;
-    if (rot) {
-        if constexpr (D == 64 || D == 128) decode_split_kernel<D, true, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
-        else return mi_fail(MI_E_SHAPE, "attn_decode: fused rotary needs head_dim 64 or 128");
-    } else {
-        decode_split_kernel<D, false, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
-    }
+    if (rot == 2) decode_split_kernel<D, 2, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
+    else if (rot == 1) decode_split_kernel<D, 1, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
+    else decode_split_kernel<D, 0, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
     return mi_check_launch("decode_split");
 }
 
-template <int D> int launch_decode(const DecodeParams& p, bool append, bool rot, hipStream_t st) {
+template <int D> int launch_decode(const DecodeParams& p, bool append, int rot, hipStream_t st) {
     if (append) {
         const int n = p.batch * p.nkv * (D / 16);
         decode_append_kernel<D><<<dim3((n + 127) / 128), dim3(128), 0, st>>>(p);
@@ -371,7 +387,12 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     DecodeParams p{};
     p.q = (const __bf16*)a->q; p.kc = (__bf16*)a->k_cache; p.vc = (__bf16*)a->v_cache; p.o = (__bf16*)a->o;
     p.ctx_len = a->ctx_len; p.k_new = (const __bf16*)a->k_new; p.v_new = (const __bf16*)a->v_new;
-    p.cos = (const __bf16*)a->rotary_cos; p.sin = (const __bf16*)a->rotary_sin; p.pos = a->position_ids;
+    if (a->rotary_interleaved) {
+        p.cos32 = (const float*)a->rotary_cos; p.sin32 = (const float*)a->rotary_sin;
+    } else {
+        p.cos = (const __bf16*)a->rotary_cos; p.sin = (const __bf16*)a->rotary_sin;
+    }
+    p.pos = a->position_ids;
     p.table_rows = (int)a->rotary_table_rows;
     p.batch = a->batch; p.max_ctx = a->max_ctx; p.nq = a->n_q_heads; p.nkv = a->n_kv_heads;
     p.n_rep = a->n_q_heads / a->n_kv_heads; p.n_splits = splits;
@@ -383,6 +404,7 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     p.ws_o = (float*)a->workspace;
     p.ws_ml = p.ws_o + (size_t)a->batch * a->n_q_heads * splits * a->head_dim;
     hipStream_t st = (hipStream_t)a->stream;
-    if (a->head_dim == 64) return launch_decode<64>(p, a->k_new != nullptr, rot, st);
-    return launch_decode<128>(p, a->k_new != nullptr, rot, st);
+    const int rot_mode = rot ? (a->rotary_interleaved ? 2 : 1) : 0;
+    if (a->head_dim == 64) return launch_decode<64>(p, a->k_new != nullptr, rot_mode, st);
+    return launch_decode<128>(p, a->k_new != nullptr, rot_mode, st);
 }

@@ -24,7 +24,9 @@ namespace {
 constexpr int BN = 64;               // keys per tile
 constexpr float kRescaleGap = 8.0f;  // log2 units by which a row max may lag before O is rescaled
 
-template <int D, int NW, bool ROT, bool DROP>
+// ROT: 0 = q / k are used as they are, 1 = rotate-half rotary applied on load (tables in the I/O dtype),
+// 2 = interleaved-pair rotary applied on load (fp32 tables)
+template <int D, int NW, int ROT, bool DROP>
 __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p) {
     constexpr int BM = 32 * NW;
     constexpr int KS = D / 16;            // contraction steps of Q K^T
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qrow + 16 * ks);
-        if constexpr (ROT) {
+        if constexpr (ROT == 1) {
             int64_t pos = p.pos_q[tl];
             pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
             const __bf16* cr = p.cos + pos * D + 8 * g;
@@ -77,6 +79,14 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 const uint4 s = *reinterpret_cast<const uint4*>(sr + 16 * ks);
                 rotate_pair(raw[ks], raw[ks + KS / 2], c, s, 1.0f);
             }
+        } else if constexpr (ROT == 2) {
+            int64_t pos = p.pos_q[tl];
+            pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+            const float* cr = p.cos32 + pos * (D / 2) + 4 * g;   // features 16 ks + 8 g .. + 8 = pairs 8 ks + 4 g .. + 4
+            const float* sr = p.sin32 + pos * (D / 2) + 4 * g;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                rotate_interleaved(raw[ks], ld128(cr + 8 * ks), ld128(sr + 8 * ks), 1.0f);
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
@@ -116,7 +126,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     const int lw = wave & 3;                                         // loader index within the role
     const int ltid = (NW == 4) ? tid : (tid & 255);
     uint4 kraw[ROT ? KV_VECS : 1];
-    uint4 craw[ROT ? KV_VECS / 2 : 1], sraw[ROT ? KV_VECS / 2 : 1];  // rotary table rows of the K tile
+    constexpr int TAB_VECS = ROT == 2 ? KV_VECS : (ROT == 1 ? KV_VECS / 2 : 1);
+    uint4 craw[TAB_VECS], sraw[TAB_VECS];                            // rotary table rows of the K tile
     int64_t kpos[ROT ? KV_VECS / 2 : 1];                             // their positions, fetched a tile ahead
     const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
     const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
@@ -143,8 +154,15 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 kraw[2 * j + 1] = ld128(kr + D / 2);
                 int64_t pos = kpos[j];
                 pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
-                craw[j] = ld128(p.cos + pos * D + 8 * c);
-                sraw[j] = ld128(p.sin + pos * D + 8 * c);
+                if constexpr (ROT == 1) {
+                    craw[j] = ld128(p.cos + pos * D + 8 * c);
+                    sraw[j] = ld128(p.sin + pos * D + 8 * c);
+                } else {                          // pairs 4 c .. + 4 of the first vector, D / 4 further on for the second
+                    craw[2 * j] = ld128(p.cos32 + pos * (D / 2) + 4 * c);
+                    sraw[2 * j] = ld128(p.sin32 + pos * (D / 2) + 4 * c);
+                    craw[2 * j + 1] = ld128(p.cos32 + pos * (D / 2) + 4 * c + D / 4);
+                    sraw[2 * j + 1] = ld128(p.sin32 + pos * (D / 2) + 4 * c + D / 4);
+                }
             }
         }
     };
@@ -155,7 +173,12 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
             for (int j = 0; j < KV_VECS / 2; ++j) {
                 const int idx = ltid + 256 * j;
                 const int row = idx / (D / 16), c = idx % (D / 16);
-                rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);
+                if constexpr (ROT == 1) {
+                    rotate_pair(kraw[2 * j], kraw[2 * j + 1], craw[j], sraw[j], 1.0f);
+                } else {
+                    rotate_interleaved(kraw[2 * j], craw[2 * j], sraw[2 * j], 1.0f);
+                    rotate_interleaved(kraw[2 * j + 1], craw[2 * j + 1], sraw[2 * j + 1], 1.0f);
+                }
                 st128(ks + Tile::unit_offset(row, c), kraw[2 * j]);
                 st128(ks + Tile::unit_offset(row, c + D / 16), kraw[2 * j + 1]);
             }
@@ -388,7 +411,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     }
 }
 
-template <int D, int NW, bool ROT, bool DROP> int launch(const AttnParams& p, hipStream_t st) {
+template <int D, int NW, int ROT, bool DROP> int launch(const AttnParams& p, hipStream_t st) {
     constexpr int BM = 32 * NW;
     const int64_t nqb = ((int64_t)p.total_q + BM - 1) / BM;
     const int64_t grid = nqb * p.nq;
@@ -397,19 +420,21 @@ template <int D, int NW, bool ROT, bool DROP> int launch(const AttnParams& p, hi
     return mi_check_launch("attn_fwd");
 }
 
-template <int D> int launch_d(const AttnParams& p, bool rot, int nw, hipStream_t st) {
+// rot: 0 = none, 1 = rotate-half, 2 = interleaved pairs
+template <int D> int launch_d(const AttnParams& p, int rot, int nw, hipStream_t st) {
     if (p.drop_thr != 0) {               // dropout: one tiling per head_dim (256-query workgroups), no fused rotary
         if (rot) return mi_fail(MI_E_SHAPE, "attn_fwd: dropout and fused rotary cannot be combined");
-        return launch<D, 8, false, true>(p, st);
+        return launch<D, 8, 0, true>(p, st);
     }
     if (rot) {
         if constexpr (D == 64 || D == 128) {
-            return nw == 8 ? launch<D, 8, true, false>(p, st) : launch<D, 4, true, false>(p, st);
+            if (rot == 2) return nw == 8 ? launch<D, 8, 2, false>(p, st) : launch<D, 4, 2, false>(p, st);
+            return nw == 8 ? launch<D, 8, 1, false>(p, st) : launch<D, 4, 1, false>(p, st);
         } else {
             return mi_fail(MI_E_SHAPE, "attn_fwd: fused rotary needs head_dim 64 or 128");
         }
     }
-    return nw == 8 ? launch<D, 8, false, false>(p, st) : launch<D, 4, false, false>(p, st);
+    return nw == 8 ? launch<D, 8, 0, false>(p, st) : launch<D, 4, 0, false>(p, st);
 }
 
 }  // namespace
@@ -426,7 +451,7 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     if (a->total_q == 0) return MI_OK;
     AttnParams p;
     mi_attn_fill_params(a, &p);
-    const bool rot = a->rotary_cos != nullptr;
+    const int rot = a->rotary_cos == nullptr ? 0 : (a->rotary_interleaved ? 2 : 1);
     // 256-query workgroups halve the K/V staging work per query; worth it once the grid still fills
     // the 256 compute units a few times over
     const int64_t blocks_256 = (((int64_t)p.total_q + 255) / 256) * p.nq;

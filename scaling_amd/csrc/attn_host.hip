@@ -45,7 +45,11 @@ void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p) {
     p->o_st = a->o_stride_token; p->o_sh = a->o_stride_head;
     p->scale = a->softmax_scale;
     p->scale_log2 = a->softmax_scale * 1.4426950408889634f;
-    p->cos = (const __bf16*)a->rotary_cos; p->sin = (const __bf16*)a->rotary_sin;
+    if (a->rotary_interleaved) {
+        p->cos32 = (const float*)a->rotary_cos; p->sin32 = (const float*)a->rotary_sin;
+    } else {
+        p->cos = (const __bf16*)a->rotary_cos; p->sin = (const __bf16*)a->rotary_sin;
+    }
     p->pos_q = a->position_ids_q; p->pos_k = a->position_ids_k; p->table_rows = (int)a->rotary_table_rows;
     if (a->dropout_p > 0.f) {
         int t = (int)(a->dropout_p * 256.0f + 0.5f);

@@ -80,6 +80,15 @@ template <> struct Elem<float> {
     static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
 };
 
+// One pair of the interleaved ("complex") rotary: (x0 + i x1) * (c + i s).  The roundings are spelled out so
+// that every kernel that applies the rotation (stand-alone or fused into an attention load) gives the same bits.
+__device__ __forceinline__ void rotate_complex_pair(float& x0, float& x1, float c, float s) {
+    const float re = __builtin_fmaf(x0, c, -(x1 * s));
+    const float im = __builtin_fmaf(x0, s, x1 * c);
+    x0 = re;
+    x1 = im;
+}
+
 // ---- wavefront reductions (64 lanes) -------------------------------------------------------
 template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
 #pragma unroll

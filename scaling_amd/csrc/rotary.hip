@@ -126,9 +126,9 @@ __global__ __launch_bounds__(kBlock) void rotary_complex_kernel(RotaryParams p) 
     Elem<T>::unpack(*reinterpret_cast<const uint4*>(xrow), x);
 #pragma unroll
     for (int i = 0; i < V / 2; ++i) {
-        const float c = cr[i], sn = p.sign * sr[i];
-        o[2 * i] = x[2 * i] * c - x[2 * i + 1] * sn;
-        o[2 * i + 1] = x[2 * i] * sn + x[2 * i + 1] * c;
+        o[2 * i] = x[2 * i];
+        o[2 * i + 1] = x[2 * i + 1];
+        rotate_complex_pair(o[2 * i], o[2 * i + 1], cr[i], p.sign * sr[i]);
     }
     *reinterpret_cast<uint4*>(orow) = Elem<T>::pack(o);
 }

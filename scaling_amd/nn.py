@@ -146,12 +146,13 @@ class RotaryEmbeddingComplex(torch.nn.Module):
         self.max_seq_length = n
 
     def tables(self) -> Tuple[torch.Tensor, torch.Tensor]:
-        return self.freqs_cis_real, self.freqs_cis_imag
+        """fp32 [max_seq, dim / 2] real and imaginary parts (no copy unless the buffers were cast)."""
+        return self.freqs_cis_real.float().contiguous(), self.freqs_cis_imag.float().contiguous()
 
     def rotate_tokens(self, x: torch.Tensor, position_ids: Optional[torch.Tensor], seq_len: int) -> torch.Tensor:
         assert x.shape[-1] == self.dimensions, "the interleaved variant rotates the whole head (rotary.py:69-70)"
-        return ops.rotary_embedding_complex(x, self.freqs_cis_real.float().contiguous(),
-                                            self.freqs_cis_imag.float().contiguous(), position_ids, seq_len)
+        real, imag = self.tables()
+        return ops.rotary_embedding_complex(x, real, imag, position_ids, seq_len)
 
     def forward(self, query: torch.Tensor, key: torch.Tensor, query_position_ids: Optional[torch.Tensor] = None,
                 key_position_ids: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -306,9 +307,9 @@ class ParallelSelfAttention(torch.nn.Module):
         elif relative_position_embedding_type == RelativePositionEmbeddingType.ROTARY_COMPLEX:
             assert rotary_config is not None
             self.rotary_embedding = RotaryEmbeddingComplex(config=rotary_config, device=self._device)
-        # rotary can be applied inside the attention kernels (on the Q/K load) for the rotate-half variant
+        # rotary can be applied inside the attention kernels (on the Q/K load), either pairing
         # when it covers the whole head
-        self._fusable_rotary = isinstance(self.rotary_embedding, RotaryEmbedding) and \
+        self._fusable_rotary = self.rotary_embedding is not None and \
             rotary_config.dimensions == self.hidden_size_per_attention_head and self.hidden_size_per_attention_head in (64, 128)
 
         self.key_query_norm = key_query_norm
@@ -483,7 +484,7 @@ class ParallelSelfAttention(torch.nn.Module):
             if self._fusable_rotary:
                 cos, sin = self.rotary_embedding.tables()
                 rotary = (cos, sin, pos)
-            else:  # partial or interleaved rotary: stand-alone kernel, then a plain append
+            else:  # partial rotary: stand-alone kernel, then a plain append
                 q = self.rotary_embedding.rotate_tokens(q, pos, 1)
                 k = self.rotary_embedding.rotate_tokens(k, pos, 1)
         if cache.workspace is None:

@@ -407,6 +407,18 @@ def linear_cross_entropy(h: torch.Tensor, weight: torch.Tensor, targets: torch.T
 # ------------------------------------------------------------------------------------------------
 # attention core
 # ------------------------------------------------------------------------------------------------
+def _fused_rotary_kind(cos: torch.Tensor, sin: torch.Tensor, head_dim: int, dtype: torch.dtype) -> bool:
+    """Checks the tables of a fused rotary; True for the interleaved-pair variant (fp32 tables [rows, head_dim / 2],
+    RotaryEmbeddingComplex), False for rotate-half (tables [rows, head_dim] in the tensors' dtype)."""
+    assert cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape and cos.dim() == 2
+    if cos.dtype == torch.float32 and cos.shape[1] * 2 == head_dim and dtype != torch.float32:
+        assert sin.dtype == torch.float32
+        return True
+    assert cos.dtype == dtype and sin.dtype == dtype and cos.shape[1] == head_dim, \
+        "fused rotary takes [rows, head_dim] tables in the data dtype or fp32 [rows, head_dim / 2] tables (interleaved pairs)"
+    return False
+
+
 def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, flags=0, dropout=None) -> MiAttnArgs:
     a = MiAttnArgs()
     a.flags = int(flags)
@@ -427,6 +439,7 @@ def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, fla
         a.rotary_cos, a.rotary_sin = ptr(cos), ptr(sin)
         a.position_ids_q, a.position_ids_k = ptr(pos_q), ptr(pos_k)
         a.rotary_table_rows = cos.shape[0]
+        a.rotary_interleaved = int(_fused_rotary_kind(cos, sin, q.shape[2], q.dtype))
     if dropout is not None and dropout[0] > 0.0:
         a.dropout_p, a.dropout_seed = float(dropout[0]), int(dropout[1]) & 0xFFFFFFFFFFFFFFFF
     a.stream = stream_ptr()
@@ -447,6 +460,9 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
                       dropout=None):
     """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens]).
 
+    rotary: optional (cos, sin, position_ids_q, position_ids_k), q and k are rotated while they are loaded:
+    rotate-half with [rows, head_dim] tables in q's dtype, interleaved pairs with fp32 [rows, head_dim / 2] tables.
+
     dropout: optional (p, seed) for dropout on the attention probabilities; the backward needs the same pair.
 
     flags: 0 lets the library pick the tiling; 1 / 2 pin one / two query groups per wavefront."""
@@ -455,7 +471,7 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
     if rotary is not None:
         cos, sin, pos_q, pos_k = rotary
-        assert cos.dtype == q.dtype and cos.is_contiguous() and sin.is_contiguous() and cos.shape[1] == q.shape[2]
+        _fused_rotary_kind(cos, sin, q.shape[2], q.dtype)
         assert pos_q.dtype == torch.int64 and pos_q.is_contiguous() and pos_q.numel() == q.shape[0]
         assert pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0]
     o = torch.empty((q.shape[0], q.shape[1], q.shape[2]), dtype=q.dtype, device=q.device)
@@ -559,7 +575,8 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      n_splits: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One decode step.  q [B, n_q, d]; caches [B, max_ctx, n_kv, d]; ctx_len int32 [B] counts the valid
     keys INCLUDING the token appended by this call (k_new/v_new [B, n_kv, d], written at ctx_len-1).
-    rotary = (cos, sin, position_ids[B]) rotates q and k_new inside the kernels.  q, k_new and v_new may be
+    rotary = (cos, sin, position_ids[B]) rotates q and k_new inside the kernels (table formats as for
+    attention_forward: rotate-half or interleaved pairs).  q, k_new and v_new may be
     column slices of one projection output: only their [heads, d] part has to be contiguous."""
     _need_cuda(q, k_cache, v_cache, ctx_len)
     B, nq, d = q.shape
@@ -586,7 +603,7 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         a.k_new_stride_batch, a.v_new_stride_batch = _rows(k_new), _rows(v_new)
     if rotary is not None:
         cos, sin, pos = rotary
-        assert cos.dtype == q.dtype and cos.is_contiguous() and sin.is_contiguous() and cos.shape[1] == d
+        a.rotary_interleaved = int(_fused_rotary_kind(cos, sin, d, q.dtype))
         assert pos.dtype == torch.int64 and pos.numel() == B and pos.is_contiguous()
         a.rotary_cos, a.rotary_sin, a.position_ids = ptr(cos), ptr(sin), ptr(pos)
         a.rotary_table_rows = cos.shape[0]

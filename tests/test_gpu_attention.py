@@ -111,6 +111,46 @@ def test_attention_fused_rotary_matches_separate_rotary():
     assert float(diff.max()) <= 2e-2 and float((diff > 0).float().mean()) < 0.02
 
 
+def _complex_tables(d, rows, base):
+    """fp32 [rows, d / 2] real / imaginary parts of freqs_cis (core/nn/rotary.py:45-56)."""
+    inv_freq = 1.0 / (float(base) ** (torch.arange(0, d, 2)[: d // 2].float() / d))
+    ang = torch.outer(torch.arange(rows).float(), inv_freq).float()
+    return ang.cos().contiguous(), ang.sin().contiguous()
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("flags", [1, 2])
+def test_attention_fused_interleaved_rotary_matches_separate_rotary(d, flags):
+    """Interleaved-pair ("complex") rotary applied while q / k are loaded: same bits as the stand-alone kernel
+    followed by the plain call, and the oracle's complex rotary followed by its attention within the gates."""
+    print(f"case fused interleaved rotary d={d} flags={flags}", flush=True)
+    b, s, nq, nkv = 2, 320, 4, 2
+    q, k, v, _ = U.make_qkv(b, s, nq, nkv, d, seed=9)
+    cu = U.make_cu(b, s, (70, 400))
+    pos = U.position_ids_from_cu(cu, b * s)
+    ids = pos.view(b, s).transpose(0, 1)
+    scale = 1 / math.sqrt(d)
+    n_rep = nq // nkv
+    qr, kr = oracle.apply_rotary_complex(U.to_sbnd(q.float(), b, s), U.to_sbnd(k.float(), b, s), d, s, 10000.0, ids, ids)
+    ref = U.from_bn_s_d(oracle.multi_head_attention(qr, oracle.repeat_kv(kr, n_rep), oracle.repeat_kv(U.to_sbnd(v.float(), b, s), n_rep),
+                                                    cu, True, scale, softmax_in_fp32=True), b, nq)
+    qo, ko = oracle.apply_rotary_complex(U.to_sbnd(q, b, s), U.to_sbnd(k, b, s), d, s, 10000.0, ids, ids)
+    ref_o = U.from_bn_s_d(oracle.multi_head_attention(qo, oracle.repeat_kv(ko, n_rep), oracle.repeat_kv(U.to_sbnd(v, b, s), n_rep),
+                                                      cu, True, scale, softmax_in_fp32=True), b, nq)
+    real, imag = (t.to(DEV) for t in _complex_tables(d, s, 10000.0))
+    qd, kd, vd, cud, posd = q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), pos.to(DEV)
+    fused, lse_f = ops.attention_forward(qd, kd, vd, cud, None, True, None, rotary=(real, imag, posd, posd), flags=flags)
+    q2 = ops.rotary_embedding_complex(qd, real, imag, posd)
+    k2 = ops.rotary_embedding_complex(kd, real, imag, posd)
+    sep, lse_s = ops.attention_forward(q2, k2, vd, cud, None, True, None, flags=flags)
+    torch.cuda.synchronize()
+    check("attn.fused_interleaved_rotary", fused, ref, ref_o)
+    assert torch.equal(fused, sep) and torch.equal(lse_f, lse_s)
+    # tables of the wrong shape or type are refused before the launch
+    with pytest.raises(AssertionError):
+        ops.attention_forward(qd, kd, vd, cud, None, True, None, rotary=(real[:, : d // 4].contiguous(), imag[:, : d // 4].contiguous(), posd, posd))
+
+
 def test_attention_is_bit_reproducible_and_gqa_equals_repeated_heads():
     b, s, nq, nkv, d = 1, 320, 8, 2, 128
     q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=9)

@@ -94,6 +94,49 @@ def test_decode_append_and_fused_rotary():
     assert torch.equal(kcd.cpu()[mask], kc[mask]) and torch.equal(vcd.cpu()[mask], vc[mask])
 
 
+@pytest.mark.parametrize("B,nq,nkv,d", [(3, 8, 2, 128), (2, 4, 4, 64), (32, 32, 8, 128)])
+def test_decode_append_and_fused_interleaved_rotary(B, nq, nkv, d):
+    """Interleaved-pair rotary of q and of the appended key inside the decode kernels: same bits as the stand-alone
+    kernel followed by a plain append, and within the gates of the oracle."""
+    print(f"case decode fused interleaved rotary B={B} nq={nq} nkv={nkv} d={d}", flush=True)
+    max_ctx = 96
+    g = torch.Generator().manual_seed(B + d)
+    lens = [(7 * i) % max_ctx + 1 for i in range(B)]
+    lens[0] = max_ctx
+    q = torch.randn(B, nq, d, generator=g).bfloat16()
+    k_new = torch.randn(B, nkv, d, generator=g).bfloat16()
+    v_new = torch.randn(B, nkv, d, generator=g).bfloat16()
+    kc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16()
+    vc = torch.randn(B, max_ctx, nkv, d, generator=g).bfloat16()
+    ctx = torch.tensor(lens, dtype=torch.int32)
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int64)
+    scale = 1 / math.sqrt(d)
+    qr, kr = oracle.apply_rotary_complex(q.unsqueeze(0), k_new.unsqueeze(0), d, max_ctx, 10000.0, pos.view(1, B), pos.view(1, B))
+    qr, kr = qr[0], kr[0]                           # fp32 math, one rounding to bf16 (the reference's order)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    for b in range(B):
+        kc_ref[b, lens[b] - 1] = kr[b]
+        vc_ref[b, lens[b] - 1] = v_new[b]
+    ref = _oracle_decode(qr, kc_ref, vc_ref, ctx, scale, torch.float32)
+    ref_o = _oracle_decode(qr, kc_ref, vc_ref, ctx, scale, torch.bfloat16)
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, d, 2)[: d // 2].float() / d))
+    ang = torch.outer(torch.arange(max_ctx).float(), inv_freq).float()
+    real, imag = ang.cos().contiguous().to(DEV), ang.sin().contiguous().to(DEV)
+    qd, knd, vnd, ctxd, posd = q.to(DEV), k_new.to(DEV), v_new.to(DEV), ctx.to(DEV), pos.to(DEV)
+    kc1, vc1 = kc.to(DEV), vc.to(DEV)
+    fused = ops.decode_attention(qd, kc1, vc1, ctxd, knd, vnd, rotary=(real, imag, posd), softmax_scale=scale)
+    kc2, vc2 = kc.to(DEV), vc.to(DEV)
+    q2 = ops.rotary_embedding_complex(qd, real, imag, posd)
+    k2 = ops.rotary_embedding_complex(knd, real, imag, posd)
+    sep = ops.decode_attention(q2, kc2, vc2, ctxd, k2, vnd, softmax_scale=scale)
+    torch.cuda.synchronize()
+    check("decode.o(append+interleaved rotary)", fused, ref, ref_o)
+    assert torch.equal(fused, sep) and torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    for b in range(B):
+        kd = (kc1[b, lens[b] - 1].float().cpu() - kr[b].float()).abs()
+        assert float(kd.max()) <= 2e-2 and float((kd > 0).float().mean()) < 0.02
+
+
 def test_decode_equals_last_row_of_prefill_kernel():
     """Cached == uncached: the decode kernel agrees with the last query row of the forward kernel."""
     nq, nkv, d, n = 8, 2, 128, 333

@@ -106,8 +106,10 @@ def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
         assert m["finite"] and m["mean_rel"] <= max(1e-3, 1.25 * f["mean_rel"]), (k, m, f)
 
 
-def test_cached_generation_matches_uncached_and_oracle():
-    cfg = _arch(attention_num_kv_heads=2)
+@pytest.mark.parametrize("rotary", ["rotary", "rotary_complex"])
+def test_cached_generation_matches_uncached_and_oracle(rotary):
+    # both pairings are applied inside the attention kernels here (head_dim 64, whole head rotated)
+    cfg = _arch(attention_num_kv_heads=2, relative_position_embedding_type=rotary)
     model = TransformerInferenceModule(cfg, device=DEV, init_std=0.2, seed=3)
     prompt = [5, 17, 3, 90, 41, 8, 63]
     tok_c, log_c = model.generate(6, prompt, use_cache=True)
@@ -122,6 +124,7 @@ def test_cached_generation_matches_uncached_and_oracle():
         om = {"embedding.weight": sd["_layers.0.embedding.weight"], "layers": layers,
               "final": {"norm.weight": sd["_layers.3.norm.weight"]}, "lm_head.weight": sd["_layers.4.linear.weight"]}
         spec = _spec(cfg, dtype)
+        spec.rotary = rotary
         full = torch.tensor([prompt + tok_c[0][:-1]])
         cu = oracle.get_cumulative_seq_lengths(full)
         with torch.no_grad():

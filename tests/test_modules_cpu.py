@@ -135,7 +135,11 @@ def test_unsupported_options_raise():
         ParallelSelfAttention(256, 4, hip, dtype=torch.float32, device=CPU)
     cplx = ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, rotary_config=C.RotaryConfig(dimensions=64, max_seq_length=16),
                                  relative_position_embedding_type=C.RelativePositionEmbeddingType.ROTARY_COMPLEX)
-    assert cplx.rotary_embedding.freqs_cis_real.shape == (16, 32) and not cplx._fusable_rotary
+    assert cplx.rotary_embedding.freqs_cis_real.shape == (16, 32) and cplx._fusable_rotary
+    real, imag = cplx.rotary_embedding.tables()      # the fused kernels take fp32 [rows, d / 2] tables
+    assert real.dtype == torch.float32 and real.shape == (16, 32) and imag.shape == (16, 32)
+    partial = ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, rotary_config=C.RotaryConfig(dimensions=32, max_seq_length=16))
+    assert not partial._fusable_rotary               # rotary over part of the head: stand-alone kernel
     assert all("freqs_cis" not in k for k in cplx.state_dict())
     with pytest.raises(AssertionError, match="kv heads"):
         ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, num_kv_heads=2, qkv_in_one=True,
