@@ -259,8 +259,6 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // 128-bit load / store through a native vector type.  Copying a uint4 (a struct) between address spaces
 // becomes a memcpy that keeps staging arrays in scratch memory; building the value element-wise lets
 // them live in registers.
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-
 __device__ __forceinline__ uint4 ld128(const void* p) {
     const u32x4_t v = *reinterpret_cast<const u32x4_t*>(p);
     return make_uint4(v[0], v[1], v[2], v[3]);

@@ -166,7 +166,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
             const int tok = min(key0 + 16 * t + l16, last);
             const __bf16* kr = kbase + (int64_t)tok * p.c_st + 8 * G;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) c.kf[t][ks] = *reinterpret_cast<const bf16x8_t*>(kr + 32 * ks);
+            for (int ks = 0; ks < KS; ++ks) c.kf[t][ks] = __builtin_bit_cast(bf16x8_t, ldg_nt(reinterpret_cast<const uint4*>(kr + 32 * ks)));
         }
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int tok = min(key0 + 4 * quad + r, last);
-                c.vraw[j][r] = *reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.c_st + 8 * dg);
+                c.vraw[j][r] = ldg_nt(reinterpret_cast<const uint4*>(vbase + (int64_t)tok * p.c_st + 8 * dg));
             }
         }
     };

@@ -113,7 +113,7 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
     auto row_ptr = [&](int64_t r) { return reinterpret_cast<const T*>(a.logits) + r * a.logits_stride; };
     auto load_vec = [&](int64_t r, int j) {
         const int v = j * kCeBlock + threadIdx.x;
-        if (v < vecs) raw[j] = reinterpret_cast<const uint4*>(row_ptr(r))[v];
+        if (v < vecs) raw[j] = ldg_nt(reinterpret_cast<const uint4*>(row_ptr(r)) + v);
     };
     auto load_target = [&](int64_t r, int64_t& target, bool& ignored, float& x_target) {
         target = a.targets[r];
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
                 Elem<T>::unpack(raw[j], f);
 #pragma unroll
                 for (int i = 0; i < V; ++i) f[i] = __builtin_amdgcn_exp2f(f[i] * kLog2e - l2) * scale;
-                reinterpret_cast<uint4*>(dx)[v] = Elem<T>::pack(f);
+                stg_nt(reinterpret_cast<uint4*>(dx) + v, Elem<T>::pack(f));
                 if (v == v_target)
                     Elem<T>::store1(dx + target, (__builtin_amdgcn_exp2f(x_target * kLog2e - l2) - 1.0f) * scale);
             }
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(kFwdBlock) void ce_fwd_kernel(const CeArgs a) {
 #pragma unroll
     for (int d = 0; d < kFwdDepth; ++d) {
         const int v = threadIdx.x + d * kFwdBlock;
-        buf[d] = v < vecs ? xr[v] : neg_inf_vec<T>();
+        buf[d] = v < vecs ? ldg_nt(xr + v) : neg_inf_vec<T>();
     }
     for (int v0 = threadIdx.x; v0 < vecs; v0 += kFwdDepth * kFwdBlock) {
 #pragma unroll
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(kFwdBlock) void ce_fwd_kernel(const CeArgs a) {
             float f[V];
             Elem<T>::unpack(buf[d], f);
             const int vn = v0 + (d + kFwdDepth) * kFwdBlock;
-            buf[d] = vn < vecs ? xr[vn] : neg_inf_vec<T>();
+            buf[d] = vn < vecs ? ldg_nt(xr + vn) : neg_inf_vec<T>();
             float vm = f[0];
 #pragma unroll
             for (int i = 1; i < V; ++i) vm = fmaxf(vm, f[i]);

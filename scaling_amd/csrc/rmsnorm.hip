@@ -80,7 +80,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
             Elem<T>::unpack(wr[v], g);
 #pragma unroll
             for (int i = 0; i < V; ++i) f[i] = (f[i] * rstd) * g[i];
-            yr[v] = Elem<T>::pack(f);
+            if constexpr (ADD) yr[v] = Elem<T>::pack(f);
+            else stg_nt(yr + v, Elem<T>::pack(f));
         }
     }
 }
@@ -518,7 +519,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(const T* __restri
             if (b != nullptr) Elem<T>::unpack(br[v], bb);
 #pragma unroll
             for (int i = 0; i < V; ++i) o[i] = (f[c][i] - mean) * rstd * g[i] + (b != nullptr ? bb[i] : 0.f);
-            yr[v] = Elem<T>::pack(o);
+            stg_nt(yr + v, Elem<T>::pack(o));
         }
     }
 }

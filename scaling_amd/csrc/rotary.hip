@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kBlock) void rotary_vec_kernel(RotaryParams p) {
     if (v >= half_vecs) {  // unrotated tail
         const int c = p.rot_dim + (v - half_vecs) * V;
         if ((const void*)xrow != (const void*)orow)
-            *reinterpret_cast<uint4*>(orow + c) = *reinterpret_cast<const uint4*>(xrow + c);
+            stg_nt(reinterpret_cast<uint4*>(orow + c), *reinterpret_cast<const uint4*>(xrow + c));
         return;
     }
     const int c0 = v * V, c1 = c0 + p.rot_dim / 2;
@@ -73,8 +73,8 @@ __global__ __launch_bounds__(kBlock) void rotary_vec_kernel(RotaryParams p) {
         o0[i] = x0[i] * cA[i] - x1[i] * (p.sign * sA[i]);
         o1[i] = x1[i] * cB[i] + x0[i] * (p.sign * sB[i]);
     }
-    *reinterpret_cast<uint4*>(orow + c0) = Elem<T>::pack(o0);
-    *reinterpret_cast<uint4*>(orow + c1) = Elem<T>::pack(o1);
+    stg_nt(reinterpret_cast<uint4*>(orow + c0), Elem<T>::pack(o0));
+    stg_nt(reinterpret_cast<uint4*>(orow + c1), Elem<T>::pack(o1));
 }
 
 template <typename T, typename TT>
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kBlock) void rotary_complex_kernel(RotaryParams p) 
         o[2 * i + 1] = x[2 * i + 1];
         rotate_complex_pair(o[2 * i], o[2 * i + 1], cr[i], p.sign * sr[i]);
     }
-    *reinterpret_cast<uint4*>(orow) = Elem<T>::pack(o);
+    stg_nt(reinterpret_cast<uint4*>(orow), Elem<T>::pack(o));
 }
 
 template <typename T, typename TT> int launch(const RotaryParams& p, hipStream_t st) {

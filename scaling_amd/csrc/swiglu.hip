@@ -18,8 +18,8 @@ __global__ __launch_bounds__(kBlock) void swiglu_fwd_kernel(const T* __restrict_
     for (int u = 0; u < kUnroll; ++u) {
         const int64_t v = base + (int64_t)u * kBlock;
         if (v < n_vec) {
-            ra[u] = reinterpret_cast<const uint4*>(a)[v];
-            rg[u] = reinterpret_cast<const uint4*>(g)[v];
+            ra[u] = ldg_nt(reinterpret_cast<const uint4*>(a) + v);
+            rg[u] = ldg_nt(reinterpret_cast<const uint4*>(g) + v);
         }
     }
 #pragma unroll
@@ -54,9 +54,9 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const T* __restrict_
     for (int u = 0; u < kUnroll; ++u) {
         const int64_t v = base + (int64_t)u * kBlock;
         if (v < n_vec) {
-            ra[u] = reinterpret_cast<const uint4*>(a)[v];
-            rg[u] = reinterpret_cast<const uint4*>(g)[v];
-            rd[u] = reinterpret_cast<const uint4*>(dout)[v];
+            ra[u] = ldg_nt(reinterpret_cast<const uint4*>(a) + v);
+            rg[u] = ldg_nt(reinterpret_cast<const uint4*>(g) + v);
+            rd[u] = ldg_nt(reinterpret_cast<const uint4*>(dout) + v);
         }
     }
 #pragma unroll
@@ -73,8 +73,8 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const T* __restrict_
                 oa[i] = fd[i] * fg[i] * s * (1.0f + fa[i] * (1.0f - s));
                 og[i] = fd[i] * (fa[i] * s);
             }
-            reinterpret_cast<uint4*>(da)[v] = Elem<T>::pack(oa);
-            reinterpret_cast<uint4*>(dg)[v] = Elem<T>::pack(og);
+            stg_nt(reinterpret_cast<uint4*>(da) + v, Elem<T>::pack(oa));   // three streams in, two out: both sides hinted
+            stg_nt(reinterpret_cast<uint4*>(dg) + v, Elem<T>::pack(og));
         }
     }
     if (blockIdx.x == gridDim.x - 1) {
@@ -136,8 +136,9 @@ __global__ __launch_bounds__(kBlock) void gelu_kernel(const T* __restrict__ x, c
     for (int u = 0; u < kUnroll; ++u) {
         const int64_t v = base + (int64_t)u * kBlock;
         if (v < n_vec) {
-            rx[u] = reinterpret_cast<const uint4*>(x)[v];
-            if (BWD) rd[u] = reinterpret_cast<const uint4*>(dy)[v];
+            // the side with more streams carries the hint: the loads of the backward, the store of the forward
+            rx[u] = BWD ? ldg_nt(reinterpret_cast<const uint4*>(x) + v) : reinterpret_cast<const uint4*>(x)[v];
+            if (BWD) rd[u] = ldg_nt(reinterpret_cast<const uint4*>(dy) + v);
         }
     }
 #pragma unroll
@@ -149,7 +150,8 @@ __global__ __launch_bounds__(kBlock) void gelu_kernel(const T* __restrict__ x, c
             if (BWD) Elem<T>::unpack(rd[u], fd);
 #pragma unroll
             for (int i = 0; i < V; ++i) fx[i] = BWD ? fd[i] * G::grad(fx[i]) : G::value(fx[i]);
-            reinterpret_cast<uint4*>(y)[v] = Elem<T>::pack(fx);
+            if (BWD) reinterpret_cast<uint4*>(y)[v] = Elem<T>::pack(fx);
+            else stg_nt(reinterpret_cast<uint4*>(y) + v, Elem<T>::pack(fx));
         }
     }
     if (blockIdx.x == gridDim.x - 1) {
