@@ -333,16 +333,26 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* 
     const int col = blockIdx.x * 16 + cl;
     float s = 0.f;
     if (col < hidden) {
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        // the launch is latency bound (a few MB, one short dependent chain per thread): 16 loads are requested
+        // before the first is used, so 256 partial rows cost one memory round trip instead of four
+        constexpr int K = 16;
+        float acc[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) acc[k] = 0.f;
         int p = pg;
-        for (; p + 48 < n_partial; p += 64) {   // four independent loads in flight per thread
-            s0 += partial[(int64_t)p * hidden + col];
-            s1 += partial[(int64_t)(p + 16) * hidden + col];
-            s2 += partial[(int64_t)(p + 32) * hidden + col];
-            s3 += partial[(int64_t)(p + 48) * hidden + col];
+        for (; p + 16 * (K - 1) < n_partial; p += 16 * K) {
+            float v[K];
+#pragma unroll
+            for (int k = 0; k < K; ++k) v[k] = partial[(int64_t)(p + 16 * k) * hidden + col];
+#pragma unroll
+            for (int k = 0; k < K; ++k) acc[k] += v[k];
         }
-        for (; p < n_partial; p += 16) s0 += partial[(int64_t)p * hidden + col];
-        s = (s0 + s1) + (s2 + s3);
+        for (; p < n_partial; p += 16) acc[0] += partial[(int64_t)p * hidden + col];
+#pragma unroll
+        for (int w = K / 2; w > 0; w >>= 1)          // fixed pairwise order
+#pragma unroll
+            for (int k = 0; k < w; ++k) acc[k] += acc[k + w];
+        s = acc[0];
     }
     lds[pg][cl] = s;
     __syncthreads();
