@@ -111,6 +111,67 @@ def test_attention_fused_rotary_matches_separate_rotary():
     assert float(diff.max()) <= 2e-2 and float((diff > 0).float().mean()) < 0.02
 
 
+def _cross_length_reference(q, k, v, do, cu_q, cu_k, causal, scale, dtype=torch.float32):
+    """Brute force from the mask predicate of the C header, one document at a time: query t of document j may
+    attend key u of the same document iff (not causal) or u_local <= t_local + (len_k - len_q); rows without any
+    allowed key give zeros.  dtype float32 is the target; bfloat16 follows the reference's rounding points (scores
+    and probabilities in bf16 around an fp32 softmax, attention.py:160-211) and gives the error floor.
+    Returns o, dq, dk, dv."""
+    q, k, v = (t.to(dtype).clone().requires_grad_() for t in (q, k, v))
+    n_rep = q.shape[1] // k.shape[1]
+    outs = []
+    for j in range(cu_q.numel() - 1):
+        q0, q1, k0, k1 = int(cu_q[j]), int(cu_q[j + 1]), int(cu_k[j]), int(cu_k[j + 1])
+        lq, lk = q1 - q0, k1 - k0
+        if lq == 0:
+            continue
+        kj = k[k0:k1].repeat_interleave(n_rep, dim=1)
+        vj = v[k0:k1].repeat_interleave(n_rep, dim=1)
+        sc = (torch.einsum("tnd,und->ntu", q[q0:q1], kj) * scale).float()
+        allowed = torch.ones(lq, lk, dtype=torch.bool)
+        if causal:
+            allowed = torch.arange(lk)[None, :] <= torch.arange(lq)[:, None] + (lk - lq)
+        sc = sc.masked_fill(~allowed[None], float("-inf"))
+        p = torch.softmax(sc, dim=-1)
+        p = torch.where(allowed.any(dim=1)[None, :, None], p, torch.zeros_like(p))   # rows with no key: zeros, not NaN
+        outs.append(torch.einsum("ntu,und->tnd", p.to(dtype), vj))
+    o = torch.cat(outs, dim=0)
+    o.backward(do.to(dtype))
+    return o.detach(), q.grad, k.grad, v.grad
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("nq,nkv,d", [(4, 2, 128), (2, 2, 64)])
+def test_attention_with_separate_key_lengths(causal, nq, nkv, d):
+    """Documents whose query and key lengths differ (cu_seqlens_k given): chunked prefill against a longer key
+    prefix, single-query documents, more queries than keys (causal: the first rows see nothing and must be zero),
+    and an empty document."""
+    print(f"case cross-length causal={causal} nq={nq} nkv={nkv} d={d}", flush=True)
+    len_q = [5, 64, 1, 130, 0, 10, 257]
+    len_k = [70, 64, 33, 200, 0, 4, 300]
+    cu_q = torch.tensor([0] + torch.tensor(len_q).cumsum(0).tolist(), dtype=torch.int32)
+    cu_k = torch.tensor([0] + torch.tensor(len_k).cumsum(0).tolist(), dtype=torch.int32)
+    g = torch.Generator().manual_seed(17 + d)
+    q = torch.randn(int(cu_q[-1]), nq, d, generator=g).bfloat16()
+    k = torch.randn(int(cu_k[-1]), nkv, d, generator=g).bfloat16()
+    v = torch.randn(int(cu_k[-1]), nkv, d, generator=g).bfloat16()
+    do = torch.randn(int(cu_q[-1]), nq, d, generator=g).bfloat16()
+    scale = 1 / math.sqrt(d)
+    ref = _cross_length_reference(q, k, v, do, cu_q, cu_k, causal, scale)
+    ref_o = _cross_length_reference(q, k, v, do, cu_q, cu_k, causal, scale, torch.bfloat16)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o = ops.attention(qg, kg, vg, cu_q.to(DEV), cu_k.to(DEV), causal, scale)
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    check("cross.o", o, ref[0], ref_o[0])
+    check("cross.dq", qg.grad, ref[1], ref_o[1])
+    check("cross.dk", kg.grad, ref[2], ref_o[2])
+    check("cross.dv", vg.grad, ref[3], ref_o[3])
+    if causal:   # document 5: 10 queries, 4 keys -> queries 0..5 have no key
+        a = int(cu_q[5])
+        assert torch.count_nonzero(o[a:a + 6]) == 0 and torch.count_nonzero(qg.grad[a:a + 6]) == 0
+
+
 def _complex_tables(d, rows, base):
     """fp32 [rows, d / 2] real / imaginary parts of freqs_cis (core/nn/rotary.py:45-56)."""
     inv_freq = 1.0 / (float(base) ** (torch.arange(0, d, 2)[: d // 2].float() / d))
