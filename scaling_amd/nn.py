@@ -423,6 +423,11 @@ class ParallelSelfAttention(torch.nn.Module):
         return self.dense(ctx.view(b, s, nq * d))
 
     # ---- KV cache ----------------------------------------------------------------------------------
+    def merge_lora_weights(self) -> None:
+        """attention.py:1033-1034: the trainer calls this on every attention module when it is told to merge LoRA
+        weights after loading a checkpoint; this module never holds any (its constructor refuses `lora_config`)."""
+        raise AssertionError("Merge of LoRa weights called without proper configuration.")
+
     def _cache_capacity(self) -> int:
         if self.max_cache_length is not None:
             return self.max_cache_length

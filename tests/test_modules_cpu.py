@@ -140,6 +140,8 @@ def test_unsupported_options_raise():
     assert real.dtype == torch.float32 and real.shape == (16, 32) and imag.shape == (16, 32)
     partial = ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, rotary_config=C.RotaryConfig(dimensions=32, max_seq_length=16))
     assert not partial._fusable_rotary               # rotary over part of the head: stand-alone kernel
+    with pytest.raises(AssertionError, match="LoRa"):   # same failure as the reference without a LoRA configuration
+        partial.merge_lora_weights()
     assert all("freqs_cis" not in k for k in cplx.state_dict())
     with pytest.raises(AssertionError, match="kv heads"):
         ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, num_kv_heads=2, qkv_in_one=True,
