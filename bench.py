@@ -245,6 +245,62 @@ def bandwidth_cases(steps, warmup):
     return out
 
 
+def layer_case(steps, warmup):
+    """Config 4: one transformer layer (pre-RMSNorm, GQA 32/8 x 128, rotary, SwiGLU 14336) forward + backward on
+    [2, 4096, 4096] bf16.  The projections run on PyTorch matmul; the time of this library's kernels inside the step
+    is the step time minus the time of the same projections alone (forward, input gradient, weight gradient)."""
+    import torch
+    from scaling_amd import config as C
+    from scaling_amd.layer import TransformerLayer, TransformerLayerIO
+    dev = "cuda"
+    bsz, seq, hidden = 2, 4096, 4096
+    cfg = C.TransformerArchitectureConfig.from_dict(dict(
+        vocab_size=128256, hidden_size=hidden, num_layers=1, num_attention_heads=32, attention_num_kv_heads=8,
+        attention_qkv_in_one=False, norm_type="rms", mlp_type="swiglu", mlp_factor=3.5, attention_bias=False, mlp_bias=False,
+        precision="bfloat16", sequence_length=seq, rotary_embedding_base=500000,
+        masked_softmax={"kernel": "hip", "softmax_in_fp32": True}, weight_tying=False))
+    g = torch.Generator().manual_seed(4)
+
+    def init(w):
+        w.data.copy_((torch.randn(w.shape, generator=g) * 0.02).to(w.dtype))
+        return w
+
+    layer = TransformerLayer(cfg, layer_index=0, init_method=init, device=dev)
+    x = torch.randn(bsz, seq, hidden, generator=g).bfloat16().to(dev).requires_grad_()
+    dy = torch.randn(bsz, seq, hidden, generator=g).bfloat16().to(dev)
+    pos = torch.arange(seq, device=dev).repeat(bsz, 1)
+    cu = torch.arange(0, bsz * seq + 1, seq, dtype=torch.int32, device=dev)
+
+    def step():
+        for p_ in layer.parameters():
+            p_.grad = None
+        x.grad = None
+        out = layer(TransformerLayerIO(activations=x, position_ids=pos, cumulative_seq_lengths=cu))
+        out.activations.backward(dy)
+
+    ms = time_gpu(step, steps, warmup)
+    # the projections alone: y = x W^T, dx = dy W, dW = dy^T x for each of the seven weights
+    n_tok = bsz * seq
+    shapes = [(hidden, hidden), (1024, hidden), (1024, hidden), (hidden, hidden), (14336, hidden), (14336, hidden), (hidden, 14336)]
+    mats = [(torch.randn(n_tok, i, device=dev, dtype=torch.bfloat16), torch.randn(o, i, device=dev, dtype=torch.bfloat16),
+             torch.randn(n_tok, o, device=dev, dtype=torch.bfloat16)) for o, i in shapes]
+
+    def gemms():
+        for xin, w, dout in mats:
+            torch.nn.functional.linear(xin, w)
+            torch.matmul(dout, w)
+            torch.matmul(dout.t(), xin)
+
+    ms_gemm = time_gpu(gemms, steps, warmup)
+    gemm_flop = 3 * 2 * n_tok * sum(o * i for o, i in shapes)
+    pairs = bsz * seq * (seq + 1) // 2
+    attn_flop = 14 * 128 * 32 * pairs
+    return {"ms_step": ms, "tokens_per_s": n_tok / (ms * 1e-3), "ms_projection_gemms_alone": ms_gemm,
+            "ms_everything_else": ms - ms_gemm, "share_outside_gemms": (ms - ms_gemm) / ms,
+            "tflops_model": (gemm_flop + attn_flop) / (ms * 1e-3) / 1e12,
+            "note": "everything else = attention core, rotary, RMSNorm, SwiGLU, residual adds and autograd glue"}
+
+
 def decode_case(steps, layers=32, batch=32, prompt=4096):
     """Config 5: random-init 8B-class decoder, batch of prompts prefilled, then greedy cached decoding.
     Reports decode tokens/s (batch * steps / decode wall time) and the prefill time."""
@@ -378,6 +434,7 @@ def main():
         extra["config3_gqa_packed_rotary_s8192"] = attention_case(1, 8192, 32, 8, 128, cu3, args.steps, args.warmup, seed=3, rotary=True)
         extra["config3_gqa_packed_rotary_s8192"]["n_docs"] = len(cu3) - 1
         extra.update(bandwidth_cases(args.steps, args.warmup))
+        extra["config4_layer_fwd_bwd_b2_s4096_h4096"] = layer_case(max(5, args.steps // 2), 3)
         extra["config5_decode_8b_b32_ctx4096"] = decode_case(args.decode_steps, layers=args.decode_layers)
 
     line = {
