@@ -316,7 +316,9 @@ bool wide_blocks(int batch, int nkv) { return (int64_t)batch * nkv >= 192; }
 int choose_splits(int batch, int nkv, int max_ctx) {
     const int64_t pairs = (int64_t)batch * nkv;
     if (wide_blocks(batch, nkv)) return 1;
-    int64_t s = (512 + pairs - 1) / pairs;
+    // one workgroup per compute unit: measured best or within a few percent of it for batch 1 - 16 at contexts
+    // of 1k - 16k (two per compute unit, the earlier choice, cost 5 - 10 % in merge work at batch 4 - 16)
+    int64_t s = (256 + pairs - 1) / pairs;
     const int64_t by_len = ((int64_t)max_ctx + 4 * kChunk - 1) / (4 * kChunk);
     if (s > by_len) s = by_len;
     if (s > kMaxSplits) s = kMaxSplits;
