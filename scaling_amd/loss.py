@@ -67,7 +67,7 @@ class TransformerLMHead(torch.nn.Module):
                                   loss_weights=x.loss_weights, inference_settings=x.inference_settings,
                                   embeddings=x.embeddings)
 
-    def loss(self, x: TransformerLayerIO, batch, chunk_rows: int = 2048) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
+    def loss(self, x: TransformerLayerIO, batch, chunk_rows: int = 8192) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
         h = x.activations.reshape(-1, x.activations.shape[-1])
         targets = batch.target_token_ids.flatten()
         weights = batch.loss_weights.float().flatten()

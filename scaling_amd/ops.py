@@ -366,7 +366,7 @@ class _LinearCrossEntropy(torch.autograd.Function):
         row_scale = (w32 / total).contiguous()
         need_dh, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         dh = torch.empty_like(h) if need_dh else None
-        dw = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device) if need_dw else None
+        dw = None      # one chunk: the product itself; several chunks: their sum, accumulated in fp32
         losses = torch.empty(n, dtype=torch.float32, device=h.device)
         argmax = torch.empty(n, dtype=torch.int32, device=h.device)
         for r0 in range(0, n, chunk_rows):
@@ -379,7 +379,13 @@ class _LinearCrossEntropy(torch.autograd.Function):
             if need_dh:
                 torch.matmul(logits, weight, out=dh[r0:r1])
             if need_dw:
-                dw.add_(torch.matmul(logits.t(), h[r0:r1]))                   # chunk product, accumulated in fp32
+                prod = torch.matmul(logits.t(), h[r0:r1])
+                if n <= chunk_rows:
+                    dw = prod
+                elif dw is None:
+                    dw = prod.float()
+                else:
+                    dw.add_(prod)
         loss = (losses * w32).sum() / total
         ctx.save_for_backward(dh if need_dh else torch.empty(0), dw if need_dw else torch.empty(0))
         ctx.flags = (need_dh, need_dw, weight.dtype)
@@ -394,8 +400,11 @@ class _LinearCrossEntropy(torch.autograd.Function):
 
 
 def linear_cross_entropy(h: torch.Tensor, weight: torch.Tensor, targets: torch.Tensor, loss_weights: torch.Tensor,
-                         chunk_rows: int = 2048) -> Tuple[torch.Tensor, torch.Tensor]:
+                         chunk_rows: int = 8192) -> Tuple[torch.Tensor, torch.Tensor]:
     """LM head + weighted cross entropy, chunked over rows.  h [rows, hidden], weight [vocab, hidden].
+    The transient logits take chunk_rows * vocab * 2 bytes (2.1 GB at the default and a 128k vocabulary); larger
+    chunks keep the three GEMMs efficient and the fp32 accumulation of dweight rare (measured at 8192 rows x 128256:
+    23.4 ms with one chunk, 28.4 ms with four, 39.9 ms with eight).
 
     Returns (loss, argmax int32 [rows]); the gradients of h and weight are computed in the forward pass."""
     _need_cuda(h, weight, targets, loss_weights)
