@@ -82,7 +82,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 
     const int nkb = (p.total_k + BNK - 1) / BNK;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
-    const int kb = work % nkb;            // early key blocks (most queries under a causal mask) first
+    const int kb = block_for_rank(work % nkb, nkb, p.total_k, p.n_docs, BNK, false, gridDim.x <= 1024);   // most queries first
     const int kvh = work / nkb;
     const int key = kb * BNK + kgp * 32 + l32;
 
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     const int nqb = (p.total_q + BM - 1) / BM;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
     const int rep = work % p.n_rep;
-    const int qb = nqb - 1 - (work / p.n_rep) % nqb;
+    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.total_q, p.n_docs, BM, true, p.n_rep == 1);
     const int kvh = work / (p.n_rep * nqb);
     const int head = kvh * p.n_rep + rep;
     const int tq = qb * BM + wave * 32 + l32;

@@ -311,6 +311,24 @@ __device__ __forceinline__ void rotate_interleaved(uint4& v, const uint4& c, con
     }
 }
 
+// Block of the token axis that is handed out rank-th: longest first under a causal mask, where a query block has
+// the more work the later it sits in its document (late_first) and a key block the earlier.  By position on the
+// whole axis (exact for one document) or, with `across_docs`, the r-th longest blocks of all documents before the
+// (r + 1)-th longest, assuming n_docs documents of one length that is a multiple of the block size (all that can
+// be told without reading the cumulative lengths; a wrong guess only costs balance).  Handing out across documents
+// balances the tail of the launch but separates blocks of one document that would share operands in L2, so the
+// callers ask for it only where that sharing does not exist or the launch has few workgroups per compute unit
+// (measured on batches of 3 - 16 sequences of 512 - 2048 tokens: 10 - 25 % either way).  Always a permutation.
+__device__ __forceinline__ int block_for_rank(int rank, int n_blocks, int total_tokens, int n_docs, int block, bool late_first,
+                                              bool across_docs) {
+    if (across_docs && n_docs > 1 && total_tokens % n_docs == 0 && (total_tokens / n_docs) % block == 0) {
+        const int per_doc = total_tokens / n_docs / block;
+        const int pos = rank / n_docs, doc = rank - pos * n_docs;
+        return doc * per_doc + (late_first ? per_doc - 1 - pos : pos);
+    }
+    return late_first ? n_blocks - 1 - rank : rank;
+}
+
 // maps the linear workgroup id to a work item so that the workgroups an XCD receives (ids congruent
 // modulo 8) form one contiguous range of work items (neighbouring items share K/V in that XCD's L2)
 __device__ __forceinline__ int xcd_remap(int linear, int total) {

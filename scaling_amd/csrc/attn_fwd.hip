@@ -52,7 +52,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     const int nqb = (p.total_q + BM - 1) / BM;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
     const int rep = work % p.n_rep;
-    const int qb = nqb - 1 - (work / p.n_rep) % nqb;   // long (late) query blocks first
+    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.total_q, p.n_docs, BM, true, p.n_rep == 1);   // long query blocks first
     const int kvh = work / (p.n_rep * nqb);
     const int head = kvh * p.n_rep + rep;
 
