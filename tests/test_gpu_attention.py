@@ -25,6 +25,10 @@ CASES = [
     (1, 512, 4, 4, 128, False, (130,)),
     (1, 384, 6, 3, 96, True, (129,)),
     (3, 1, 2, 2, 64, True, ()),                # one token per sequence
+    # equal-length sequences of whole blocks: the kernels hand out blocks across the sequences (longest first) ...
+    (3, 256, 4, 4, 64, True, ()),              # ... forward / dQ (every query head has its own K / V)
+    (2, 256, 4, 2, 128, True, ()),             # ... dK/dV (few workgroups)
+    (1, 512, 4, 4, 64, True, (100,)),          # ... and two documents that only look equal-length from the host
 ]
 
 
