@@ -82,7 +82,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 
     const int nkb = (p.total_k + BNK - 1) / BNK;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
-    const int kb = block_for_rank(work % nkb, nkb, p.total_k, p.n_docs, BNK, false, gridDim.x <= 1024);   // most queries first
+    const int kb = block_for_rank(work % nkb, nkb, p.n_docs, p.across_k, false);   // key blocks with the most queries first
     const int kvh = work / nkb;
     const int key = kb * BNK + kgp * 32 + l32;
 
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     const int nqb = (p.total_q + BM - 1) / BM;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
     const int rep = work % p.n_rep;
-    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.total_q, p.n_docs, BM, true, p.n_rep == 1);
+    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.n_docs, p.across_q, true);
     const int kvh = work / (p.n_rep * nqb);
     const int head = kvh * p.n_rep + rep;
     const int tq = qb * BM + wave * 32 + l32;
@@ -544,6 +544,8 @@ extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
     p.dk_st = b->dk_stride_token; p.dk_sh = b->dk_stride_head;
     p.dv_st = b->dv_stride_token; p.dv_sh = b->dv_stride_head;
     p.delta = (float*)b->workspace;
+    if (p.n_rep == 1) p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 256);                   // dQ: 256-query blocks
+    if (((a->total_k + 127) / 128) * p.nkv <= 1024) p.across_k = mi_blocks_per_doc(a->total_k, a->n_docs, 128);   // dK/dV: 128-key blocks
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
         case 32: return launch_bwd<32>(p, a->flags, st);

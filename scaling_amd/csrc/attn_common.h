@@ -30,6 +30,9 @@ struct AttnParams {
     // dropout on the attention probabilities (0 = off): an element is dropped iff its random byte < drop_thr,
     // kept probabilities are scaled by drop_rscale = 256 / (256 - drop_thr)
     uint32_t drop_thr; float drop_rscale; uint32_t drop_seed;
+    // blocks per document on the query / key axis when the workgroups are to be handed out across documents
+    // (see block_for_rank), 0 for the order along the flattened axis; set by the host entry points
+    int across_q, across_k;
 };
 
 // ---- dropout mask ---------------------------------------------------------------------------------------
@@ -313,20 +316,25 @@ __device__ __forceinline__ void rotate_interleaved(uint4& v, const uint4& c, con
 
 // Block of the token axis that is handed out rank-th: longest first under a causal mask, where a query block has
 // the more work the later it sits in its document (late_first) and a key block the earlier.  By position on the
-// whole axis (exact for one document) or, with `across_docs`, the r-th longest blocks of all documents before the
-// (r + 1)-th longest, assuming n_docs documents of one length that is a multiple of the block size (all that can
-// be told without reading the cumulative lengths; a wrong guess only costs balance).  Handing out across documents
-// balances the tail of the launch but separates blocks of one document that would share operands in L2, so the
-// callers ask for it only where that sharing does not exist or the launch has few workgroups per compute unit
-// (measured on batches of 3 - 16 sequences of 512 - 2048 tokens: 10 - 25 % either way).  Always a permutation.
-__device__ __forceinline__ int block_for_rank(int rank, int n_blocks, int total_tokens, int n_docs, int block, bool late_first,
-                                              bool across_docs) {
-    if (across_docs && n_docs > 1 && total_tokens % n_docs == 0 && (total_tokens / n_docs) % block == 0) {
-        const int per_doc = total_tokens / n_docs / block;
+// whole axis (exact for one document) or, with per_doc != 0, the r-th longest blocks of all documents before the
+// (r + 1)-th longest, for n_docs documents of per_doc blocks each.  Always a permutation of the blocks.
+__device__ __forceinline__ int block_for_rank(int rank, int n_blocks, int n_docs, int per_doc, bool late_first) {
+    if (per_doc != 0) {
         const int pos = rank / n_docs, doc = rank - pos * n_docs;
         return doc * per_doc + (late_first ? per_doc - 1 - pos : pos);
     }
     return late_first ? n_blocks - 1 - rank : rank;
+}
+
+// Host side of the above: blocks per document if the batch looks like n_docs documents of one length that is a
+// multiple of the block size (all that can be told without reading the cumulative lengths; a wrong guess only costs
+// balance), else 0.  Handing out across documents balances the tail of the launch but separates blocks of one
+// document that would share operands in L2, so the entry points ask for it only where that sharing does not exist
+// (forward / dQ: every query head has its own K / V) or the launch has few workgroups per compute unit (dK/dV)
+// (measured on batches of 3 - 16 sequences of 512 - 2048 tokens: 10 - 25 % either way).
+static inline int mi_blocks_per_doc(int64_t total_tokens, int n_docs, int block) {
+    if (n_docs <= 1 || total_tokens % n_docs != 0 || (total_tokens / n_docs) % block != 0) return 0;
+    return (int)(total_tokens / n_docs / block);
 }
 
 // maps the linear workgroup id to a work item so that the workgroups an XCD receives (ids congruent

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     const int nqb = (p.total_q + BM - 1) / BM;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
     const int rep = work % p.n_rep;
-    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.total_q, p.n_docs, BM, true, p.n_rep == 1);   // long query blocks first
+    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.n_docs, p.across_q, true);   // long query blocks first
     const int kvh = work / (p.n_rep * nqb);
     const int head = kvh * p.n_rep + rep;
 
@@ -458,6 +458,7 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     int nw = p.total_q > 128 ? 8 : 4;
     if (a->flags & MI_ATTN_QG1) nw = 4;
     if (a->flags & MI_ATTN_QG2) nw = 8;
+    if (p.n_rep == 1) p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 32 * nw);
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
         case 32: return launch_d<32>(p, rot, nw, st);
