@@ -438,8 +438,10 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
         return mi_fail(MI_E_SHAPE, "rmsnorm: hidden=%lld unsupported", (long long)hidden);
     const int64_t vecs = hidden / Elem<T>::kVec;
     const bool wide = vecs >= 256;
-    // wide rows: 256 threads per row up to 512 vectors (2 rows per block), the whole block per row beyond
-    const int wide_tpr = vecs <= 512 ? 256 : 512;
+    // wide rows: 256 threads per row up to 512 vectors (4 rows per block and step), 512 up to 1024, the whole block
+    // beyond: at most two vectors per thread, so that the next step's rows always fit in registers next to this
+    // step's (four vectors per thread without that prefetch ran at 1.9 TB/s at hidden 12288)
+    const int wide_tpr = vecs <= 512 ? 256 : (vecs <= 1024 ? 512 : 1024);
     // wide rows: a single round of blocks (two per compute unit), each amortising its epilogue over many rows
     const int wide_rpb = kRmsWideBlock / wide_tpr;
     const int64_t wide_blocks = (n_rows + wide_rpb - 1) / wide_rpb;
@@ -454,7 +456,8 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
 #define RMS_WIDE(TPRV, CHV) rmsnorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kRmsWideBlock), lds, st>>>( \
             (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps)
         if (wide_tpr == 256) { if (ch <= 1) RMS_WIDE(256, 1); else RMS_WIDE(256, 2); }
-        else { if (ch <= 2) RMS_WIDE(512, 2); else RMS_WIDE(512, 4); }
+        else if (wide_tpr == 512) RMS_WIDE(512, 2);
+        else RMS_WIDE(1024, 2);
 #undef RMS_WIDE
         int rcw = mi_check_launch("rmsnorm_bwd_wide");
         if (rcw != MI_OK) return rcw;
@@ -954,8 +957,10 @@ int launch_ln_bwd(const void* x, const void* w, const void* dy, const float* mea
     Plan plan;
     if (!make_plan<T>(hidden, &plan)) return mi_fail(MI_E_SHAPE, "layernorm: hidden=%lld unsupported", (long long)hidden);
     const int64_t vecs = hidden / Elem<T>::kVec;
-    const bool wide = vecs >= 256 && vecs <= 1024 && (size_t)3 * hidden * sizeof(float) <= 159 * 1024;
-    const int wide_tpr = vecs <= 512 ? 256 : 512;
+    // rows beyond 1024 vectors take the whole 1024-thread block, which only the saved-statistics kernel has
+    const bool lds_fits = (size_t)3 * hidden * sizeof(float) <= 159 * 1024;
+    const bool wide = vecs >= 256 && lds_fits && (vecs <= 1024 || (vecs <= 2048 && mean != nullptr));
+    const int wide_tpr = vecs <= 512 ? 256 : (vecs <= 1024 ? 512 : 1024);
     // saved statistics (wide rows only; narrower rows recompute them, which costs them nothing measurable)
     const bool stats = wide && mean != nullptr;
     const int wide_rpb = (stats ? kRmsWideBlock : kWideBlock) / wide_tpr;
@@ -974,7 +979,8 @@ int launch_ln_bwd(const void* x, const void* w, const void* dy, const float* mea
 #define LN_STATS(TPRV, CHV) layernorm_bwd_stats_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kRmsWideBlock), lds, st>>>( \
             (const T*)x, (const T*)w, (const T*)dy, mean, rstd, (T*)dx, (float*)ws, n_rows, (int)hidden)
         if (wide_tpr == 256) { if (ch <= 1) LN_STATS(256, 1); else LN_STATS(256, 2); }
-        else LN_STATS(512, 2);
+        else if (wide_tpr == 512) LN_STATS(512, 2);
+        else LN_STATS(1024, 2);
 #undef LN_STATS
     } else if (wide) {
         const int ch = (int)((vecs + wide_tpr - 1) / wide_tpr);
