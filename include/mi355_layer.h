@@ -113,8 +113,11 @@ int mi_gelu_bwd(const void* x, const void* dy, void* dx, int64_t n_elem, int dty
  * row_scale (fp32, NULL = 1) carries loss_weight[r] / sum(loss_weights) times the upstream gradient
  * (cross_entropy.py:30).  A target outside [0, vocab) marks an ignored row (loss 0, zero gradient; -100 is
  * torch's ignore_index).  losses / lse / argmax / dlogits may each be NULL; dlogits may alias logits
- * (in-place gradient for a chunked LM head).  Row strides are in elements.
- * Algorithmic HBM bytes: n_rows*vocab*e read, plus the same written when dlogits is given.
+ * (in-place gradient for a chunked LM head).  Row strides are in elements.  Rows of more than 16384 vectors of
+ * 16 bytes (131072 bf16 logits) with a gradient are served by two launches that hand the log-sum-exp over in `lse`:
+ * pass it (with at most 65535 rows), or such rows fall back to a slow scalar kernel.
+ * Algorithmic HBM bytes: n_rows*vocab*e read, plus the same written when dlogits is given (and read once more
+ * by the two-launch path).
  * ------------------------------------------------------------------------------------------ */
 int mi_cross_entropy(const void* logits, const int64_t* targets, const float* row_scale, float* losses, float* lse,
                      int32_t* argmax, void* dlogits, int64_t n_rows, int64_t vocab, int64_t logits_row_stride,

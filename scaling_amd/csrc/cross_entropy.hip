@@ -364,6 +364,47 @@ __global__ __launch_bounds__(kCeBlock) void ce_stream_kernel(const CeArgs a) {
     }
 }
 
+// Gradient pass for vocabularies whose rows do not fit the registers of one workgroup (more than 16 vectors per
+// thread): an elementwise launch after the streaming forward kernel, which has left the log-sum-exp of every row in
+// a.lse.  dlogits = (softmax - onehot(target)) * scale; in place is fine (a vector is read and written by one thread).
+constexpr int kGradBlock = 256;
+constexpr int kGradUnroll = 2;
+
+template <typename T>
+__global__ __launch_bounds__(kGradBlock) void ce_grad_kernel(const CeArgs a) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t row = blockIdx.y;
+    const int vecs = a.vocab / V;
+    const T* x = reinterpret_cast<const T*>(a.logits) + row * a.logits_stride;
+    T* dx = reinterpret_cast<T*>(a.dlogits) + row * a.dlogits_stride;
+    const int64_t target = a.targets[row];
+    const bool ignored = target < 0 || target >= a.vocab;
+    const float scale = ignored ? 0.f : (a.row_scale != nullptr ? a.row_scale[row] : 1.0f);
+    const float l2 = a.lse[row] * kLog2e;
+    const int v_target = ignored ? -1 : (int)(target / V);
+    const int base = blockIdx.x * (kGradBlock * kGradUnroll) + threadIdx.x;
+    uint4 raw[kGradUnroll];
+#pragma unroll
+    for (int u = 0; u < kGradUnroll; ++u) {
+        const int v = base + u * kGradBlock;
+        if (v < vecs) raw[u] = ldg_nt(reinterpret_cast<const uint4*>(x) + v);
+    }
+#pragma unroll
+    for (int u = 0; u < kGradUnroll; ++u) {
+        const int v = base + u * kGradBlock;
+        if (v < vecs) {
+            float f[V];
+            Elem<T>::unpack(raw[u], f);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const float p = __builtin_amdgcn_exp2f(f[i] * kLog2e - l2);
+                f[i] = (p - ((v == v_target && i == (int)(target - (int64_t)v * V)) ? 1.0f : 0.f)) * scale;
+            }
+            reinterpret_cast<uint4*>(dx)[v] = Elem<T>::pack(f);
+        }
+    }
+}
+
 template <typename T>
 int launch_ce(const CeArgs& a, int64_t n_rows, hipStream_t st) {
     constexpr int V = Elem<T>::kVec;
@@ -383,6 +424,15 @@ int launch_ce(const CeArgs& a, int64_t n_rows, hipStream_t st) {
         else if (nv <= 4) ce_row_kernel<T, 4><<<pgrid, block, 0, st>>>(a, nr);
         else if (nv <= 8) ce_row_kernel<T, 8><<<pgrid, block, 0, st>>>(a, nr);
         else ce_row_kernel<T, 16><<<pgrid, block, 0, st>>>(a, nr);
+    } else if (vec_ok && a.lse != nullptr && n_rows <= 65535) {
+        // rows too long for the register-resident kernel: streaming forward, then an elementwise gradient launch
+        CeArgs f = a;
+        f.dlogits = nullptr;
+        ce_fwd_kernel<T><<<grid, dim3(kFwdBlock), 0, st>>>(f);
+        const int rc = mi_check_launch("cross_entropy");
+        if (rc != MI_OK) return rc;
+        const unsigned gx = (unsigned)((vecs + kGradBlock * kGradUnroll - 1) / (kGradBlock * kGradUnroll));
+        ce_grad_kernel<T><<<dim3(gx, (unsigned)n_rows), dim3(kGradBlock), 0, st>>>(a);
     } else {
         ce_stream_kernel<T><<<grid, block, 0, st>>>(a);
     }
