@@ -113,9 +113,11 @@ int mi_gelu_bwd(const void* x, const void* dy, void* dx, int64_t n_elem, int dty
  * row_scale (fp32, NULL = 1) carries loss_weight[r] / sum(loss_weights) times the upstream gradient
  * (cross_entropy.py:30).  A target outside [0, vocab) marks an ignored row (loss 0, zero gradient; -100 is
  * torch's ignore_index).  losses / lse / argmax / dlogits may each be NULL; dlogits may alias logits
- * (in-place gradient for a chunked LM head).  Row strides are in elements.  Rows of more than 16384 vectors of
- * 16 bytes (131072 bf16 logits) with a gradient are served by two launches that hand the log-sum-exp over in `lse`:
- * pass it (with at most 65535 rows), or such rows fall back to a slow scalar kernel.
+ * (in-place gradient for a chunked LM head).  Row strides are in elements; rows need not be 16-byte aligned nor a
+ * whole number of 16-byte vectors.  With a gradient, rows of more than 16384 vectors (131072 bf16 logits) and rows
+ * that are not aligned whole vectors are served by two launches that hand the log-sum-exp over in `lse`: pass it
+ * (with at most 65535 rows, logits and dlogits rows at the same offset from a 16-byte boundary), or such rows fall
+ * back to a slow scalar kernel.
  * Algorithmic HBM bytes: n_rows*vocab*e read, plus the same written when dlogits is given (and read once more
  * by the two-launch path).
  * ------------------------------------------------------------------------------------------ */

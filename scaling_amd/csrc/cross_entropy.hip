@@ -247,6 +247,28 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
 constexpr int kFwdBlock = 512;
 constexpr int kFwdDepth = 4;        // vectors in flight per thread
 
+// A row as [head scalars][whole aligned 16-byte vectors][tail scalars].
+struct RowSplit {
+    int head, vecs, tail0, vocab;
+    // index of the scalar element thread t takes, -1 for none
+    __device__ __forceinline__ int scalar_index(int t) const {
+        if (t < head) return t;
+        const int i = tail0 + (t - head);
+        return i < vocab ? i : -1;
+    }
+};
+
+template <typename T> __device__ __forceinline__ RowSplit split_row(const T* x, int vocab) {
+    constexpr int V = Elem<T>::kVec;
+    RowSplit r;
+    const int to_boundary = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(x) & 15u)) & 15u) / sizeof(T));
+    r.head = to_boundary < vocab ? to_boundary : vocab;
+    r.vecs = (vocab - r.head) / V;
+    r.tail0 = r.head + r.vecs * V;
+    r.vocab = vocab;
+    return r;
+}
+
 template <typename T>
 __global__ __launch_bounds__(kFwdBlock) void ce_fwd_kernel(const CeArgs a) {
     constexpr int V = Elem<T>::kVec;
@@ -255,11 +277,16 @@ __global__ __launch_bounds__(kFwdBlock) void ce_fwd_kernel(const CeArgs a) {
     __shared__ int lds_i[NW];
     const int64_t row = blockIdx.x;
     const T* x = reinterpret_cast<const T*>(a.logits) + row * a.logits_stride;
-    const uint4* xr = reinterpret_cast<const uint4*>(x);
-    const int vecs = a.vocab / V;
+    // rows need not start on a 16-byte boundary nor hold a whole number of vectors: the elements before the first
+    // aligned vector and after the last whole one (at most V - 1 each) are taken one per thread
+    const RowSplit rs = split_row<T>(x, a.vocab);
+    const uint4* xr = reinterpret_cast<const uint4*>(x + rs.head);
+    const int vecs = rs.vecs;
     const int64_t target = a.targets[row];
     const bool ignored = target < 0 || target >= a.vocab;
     const float x_target = ignored ? 0.f : Elem<T>::load1(x + target);
+    const int sc_idx = rs.scalar_index(threadIdx.x);
+    const float sc = sc_idx >= 0 ? Elem<T>::load1(x + sc_idx) : -INFINITY;
 
     float m = -INFINITY, s = 0.f;     // running maximum (natural units) and sum of exp(x - m)
     uint4 buf[kFwdDepth];
@@ -289,6 +316,11 @@ __global__ __launch_bounds__(kFwdBlock) void ce_fwd_kernel(const CeArgs a) {
             }
         }
     }
+    if (sc > m) {
+        s *= __builtin_amdgcn_exp2f((m - sc) * kLog2e);
+        m = sc;
+    }
+    if (sc_idx >= 0 && m > -INFINITY) s += __builtin_amdgcn_exp2f((sc - m) * kLog2e);
     // merge the (m, s) pairs of the block
     float bm = m;
 #pragma unroll
@@ -311,8 +343,9 @@ __global__ __launch_bounds__(kFwdBlock) void ce_fwd_kernel(const CeArgs a) {
             Elem<T>::unpack(xr[v], f);
 #pragma unroll
             for (int i = V - 1; i >= 0; --i)
-                if (f[i] == bm) arg = v * V + i;
+                if (f[i] == bm) arg = rs.head + v * V + i;
         }
+        if (sc_idx >= 0 && sc == bm) arg = min(arg, sc_idx);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) arg = min(arg, __shfl_xor(arg, off, MI_WAVE));
@@ -374,15 +407,26 @@ template <typename T>
 __global__ __launch_bounds__(kGradBlock) void ce_grad_kernel(const CeArgs a) {
     constexpr int V = Elem<T>::kVec;
     const int64_t row = blockIdx.y;
-    const int vecs = a.vocab / V;
-    const T* x = reinterpret_cast<const T*>(a.logits) + row * a.logits_stride;
-    T* dx = reinterpret_cast<T*>(a.dlogits) + row * a.dlogits_stride;
-    const int64_t target = a.targets[row];
-    const bool ignored = target < 0 || target >= a.vocab;
+    const T* x0 = reinterpret_cast<const T*>(a.logits) + row * a.logits_stride;
+    T* dx0 = reinterpret_cast<T*>(a.dlogits) + row * a.dlogits_stride;
+    const RowSplit rs = split_row<T>(x0, a.vocab);       // dx0 sits at the same offset from a 16-byte boundary (host check)
+    const int vecs = rs.vecs;
+    const T* x = x0 + rs.head;
+    T* dx = dx0 + rs.head;
+    const int64_t target_abs = a.targets[row];
+    const bool ignored = target_abs < 0 || target_abs >= a.vocab;
+    const int64_t target = target_abs - rs.head;         // relative to the first whole vector
     const float scale = ignored ? 0.f : (a.row_scale != nullptr ? a.row_scale[row] : 1.0f);
     const float l2 = a.lse[row] * kLog2e;
-    const int v_target = ignored ? -1 : (int)(target / V);
+    const int v_target = (ignored || target < 0) ? -1 : (int)(target / V);
     const int base = blockIdx.x * (kGradBlock * kGradUnroll) + threadIdx.x;
+    if (blockIdx.x == 0) {                                // the scalar elements of the row
+        const int i = rs.scalar_index(threadIdx.x);
+        if (i >= 0) {
+            const float p = __builtin_amdgcn_exp2f(Elem<T>::load1(x0 + i) * kLog2e - l2);
+            Elem<T>::store1(dx0 + i, (p - ((int64_t)i == target_abs && !ignored ? 1.0f : 0.f)) * scale);
+        }
+    }
     uint4 raw[kGradUnroll];
 #pragma unroll
     for (int u = 0; u < kGradUnroll; ++u) {
@@ -413,7 +457,12 @@ int launch_ce(const CeArgs& a, int64_t n_rows, hipStream_t st) {
     const int64_t vecs = a.vocab / V;
     const int nv = (int)((vecs + kCeBlock - 1) / kCeBlock);
     const dim3 grid((unsigned)n_rows), block(kCeBlock);
-    if (vec_ok && a.dlogits == nullptr) {
+    // the streaming kernels take any row alignment; for the gradient launch logits and dlogits rows have to sit
+    // at the same offset from a 16-byte boundary
+    const bool same_phase = a.dlogits != nullptr &&
+        ((reinterpret_cast<uintptr_t>(a.logits) ^ reinterpret_cast<uintptr_t>(a.dlogits)) & 15u) == 0 &&
+        ((a.logits_stride - a.dlogits_stride) * (int64_t)sizeof(T)) % 16 == 0;
+    if (a.dlogits == nullptr) {
         ce_fwd_kernel<T><<<grid, dim3(kFwdBlock), 0, st>>>(a);
     } else if (vec_ok && nv <= 16) {
         // one resident workgroup per compute unit, each walking its share of the rows
@@ -424,14 +473,15 @@ int launch_ce(const CeArgs& a, int64_t n_rows, hipStream_t st) {
         else if (nv <= 4) ce_row_kernel<T, 4><<<pgrid, block, 0, st>>>(a, nr);
         else if (nv <= 8) ce_row_kernel<T, 8><<<pgrid, block, 0, st>>>(a, nr);
         else ce_row_kernel<T, 16><<<pgrid, block, 0, st>>>(a, nr);
-    } else if (vec_ok && a.lse != nullptr && n_rows <= 65535) {
-        // rows too long for the register-resident kernel: streaming forward, then an elementwise gradient launch
+    } else if (same_phase && a.lse != nullptr && n_rows <= 65535) {
+        // rows too long for the register-resident kernel, not a whole number of vectors or not 16-byte aligned:
+        // streaming forward, then an elementwise gradient launch
         CeArgs f = a;
         f.dlogits = nullptr;
         ce_fwd_kernel<T><<<grid, dim3(kFwdBlock), 0, st>>>(f);
         const int rc = mi_check_launch("cross_entropy");
         if (rc != MI_OK) return rc;
-        const unsigned gx = (unsigned)((vecs + kGradBlock * kGradUnroll - 1) / (kGradBlock * kGradUnroll));
+        const unsigned gx = (unsigned)((vecs + 1 + kGradBlock * kGradUnroll - 1) / (kGradBlock * kGradUnroll));
         ce_grad_kernel<T><<<dim3(gx, (unsigned)n_rows), dim3(kGradBlock), 0, st>>>(a);
     } else {
         ce_stream_kernel<T><<<grid, block, 0, st>>>(a);

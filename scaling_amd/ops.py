@@ -324,8 +324,9 @@ def cross_entropy_forward(logits: torch.Tensor, targets: torch.Tensor, row_scale
     n, v = logits.shape
     losses = torch.empty(n, dtype=torch.float32, device=logits.device)
     argmax = torch.empty(n, dtype=torch.int32, device=logits.device)
-    # with a gradient, rows longer than 16 * 1024 vectors of 16 bytes take two launches that hand the log-sum-exp over
-    need_lse = want_lse or (dlogits is not None and v * logits.element_size() > 16 * 1024 * 16)
+    # with a gradient, rows that are very long, not a whole number of 16-byte vectors or not 16-byte aligned take two
+    # launches that hand the log-sum-exp over: always supply the (rows x 4 bytes) buffer
+    need_lse = want_lse or dlogits is not None
     lse = torch.empty(n, dtype=torch.float32, device=logits.device) if need_lse else None
     check(_lib.load().mi_cross_entropy(ptr(logits), ptr(targets), ptr(row_scale), ptr(losses), ptr(lse), ptr(argmax), ptr(dlogits),
                                        n, v, logits.stride(0), dlogits.stride(0) if dlogits is not None else 0,
