@@ -135,7 +135,8 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
 
     o, lse = ops.attention_forward(q, k, v, cu, None, True, scale)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    ws = torch.empty(nq * T, dtype=torch.float32, device=dev)
+    from scaling_amd import _lib
+    ws = torch.empty(_lib.load().mi_attn_bwd_workspace_bytes_kv(T, T, nq, nkv, d) // 4, dtype=torch.float32, device=dev)
     bufs = (dq, dk, dv, ws)
 
     def fwd():

@@ -251,6 +251,14 @@ typedef struct mi_attn_bwd_args {
 } mi_attn_bwd_args;
 
 size_t mi_attn_bwd_workspace_bytes(int64_t total_q, int32_t n_q_heads, int32_t head_dim);
+/* Workspace that also holds the fp32 partial dK / dV of a launch with fewer than 8 KV heads (multi-query attention,
+ * GQA with 2 or 4 KV heads): with at least this much, the dK/dV kernel splits the query heads of a group over
+ * workgroups (8 x more of them for one KV head) and a second launch sums the partials in a fixed order; with
+ * only mi_attn_bwd_workspace_bytes() it loops over the whole group in one workgroup per key block, which leaves
+ * most compute units idle (6.3 ms against 1.1 ms for 32 query heads on one KV head at 8192 tokens).  Equal to
+ * mi_attn_bwd_workspace_bytes() for 8 or more KV heads. */
+size_t mi_attn_bwd_workspace_bytes_kv(int64_t total_q, int64_t total_k, int32_t n_q_heads, int32_t n_kv_heads,
+                                      int32_t head_dim);
 int mi_attn_bwd(const mi_attn_bwd_args* args);
 
 /* ------------------------------------------------------------------------------------------

@@ -21,7 +21,7 @@ EXPORTS = (
     "mi_rmsnorm_fwd", "mi_add_rmsnorm_fwd", "mi_rmsnorm_bwd_workspace_bytes", "mi_rmsnorm_bwd",
     "mi_layernorm_fwd", "mi_layernorm_bwd_workspace_bytes", "mi_layernorm_bwd", "mi_gelu_fwd", "mi_gelu_bwd", "mi_cross_entropy",
     "mi_swiglu_fwd", "mi_swiglu_bwd", "mi_rotary", "mi_rotary_complex",
-    "mi_attn_fwd", "mi_attn_bwd_workspace_bytes", "mi_attn_bwd",
+    "mi_attn_fwd", "mi_attn_bwd_workspace_bytes", "mi_attn_bwd_workspace_bytes_kv", "mi_attn_bwd",
     "mi_attn_decode_workspace_bytes", "mi_attn_decode",
 )
 
@@ -121,6 +121,8 @@ def _declare(lib):
     lib.mi_attn_fwd.argtypes = [POINTER(MiAttnArgs)]
     lib.mi_attn_bwd_workspace_bytes.restype = c_size_t
     lib.mi_attn_bwd_workspace_bytes.argtypes = [c_int64, c_int32, c_int32]
+    lib.mi_attn_bwd_workspace_bytes_kv.restype = c_size_t
+    lib.mi_attn_bwd_workspace_bytes_kv.argtypes = [c_int64, c_int64, c_int32, c_int32, c_int32]
     lib.mi_attn_bwd.restype = c_int
     lib.mi_attn_bwd.argtypes = [POINTER(MiAttnBwdArgs)]
     lib.mi_attn_decode_workspace_bytes.restype = c_size_t

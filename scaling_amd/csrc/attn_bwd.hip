@@ -83,7 +83,9 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     const int nkb = (p.total_k + BNK - 1) / BNK;
     const int work = xcd_remap(blockIdx.x, gridDim.x);
     const int kb = block_for_rank(work % nkb, nkb, p.n_docs, p.across_k, false);   // key blocks with the most queries first
-    const int kvh = work / nkb;
+    const int hpw = p.n_rep / p.hsplit;   // query heads of this workgroup: hs * hpw .. + hpw of the group
+    const int kvh = (work / nkb) / p.hsplit;
+    const int hs = (work / nkb) - kvh * p.hsplit;
     const int key = kb * BNK + kgp * 32 + l32;
 
     int qlo, qhi;
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     // Query tiles are visited from the last one downwards: under a causal mask every key block of a
     // document needs the document's last queries, so the workgroups that share an XCD start on the same
     // tile and keep streaming the same Q / dO rows through that XCD's L2.
-    const int total_iters = n_tiles * p.n_rep;
+    const int total_iters = n_tiles * hpw;
     const int last_q = p.total_q - 1;
     const __bf16* src_base = q_role ? p.q : p.d_o;
     const int64_t src_head_stride = q_role ? p.q_sh : p.o_sh;
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     float stat = 0.f;
     auto tile_of = [&](int iter, int& head, int& qt) {
         const int rep = iter / n_tiles;
-        head = kvh * p.n_rep + rep;
+        head = kvh * p.n_rep + hs * hpw + rep;
         qt = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ;
     };
     auto issue_tile = [&](int iter) {     // Q / dO tile of iteration `iter` -> stage iter & 1
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             bf16x8_t pf[2], dsf[2];
             uint32_t drop_xb = 0;
             if constexpr (DROP) {
-                const int head_i = kvh * p.n_rep + iter / n_tiles;
+                const int head_i = kvh * p.n_rep + hs * hpw + iter / n_tiles;
                 drop_xb = drop_head_base(p.drop_seed, head_i) + drop_xc + (uint32_t)(qs >> 1) * kDropC1;
             }
 #pragma unroll
@@ -277,7 +279,20 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
         __syncthreads();
     }
 
-    if (sub == 0 && key < p.total_k) {
+    if (sub == 0 && key < p.total_k && p.hsplit > 1) {
+        const int64_t prow = (((int64_t)hs * p.total_k + key) * p.nkv + kvh) * D + 4 * g;
+        const float vs = DROP ? p.drop_rscale : 1.0f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                f32x4_t k4, v4;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) { k4[c] = dk_acc[dt][4 * a + c] * p.scale; v4[c] = dv_acc[dt][4 * a + c] * vs; }
+                *reinterpret_cast<f32x4_t*>(p.dk_part + prow + 32 * dt + 8 * a) = k4;
+                *reinterpret_cast<f32x4_t*>(p.dv_part + prow + 32 * dt + 8 * a) = v4;
+            }
+    } else if (sub == 0 && key < p.total_k) {
         __bf16* dkr = p.dk + (int64_t)key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * g;
         __bf16* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
 #pragma unroll
@@ -293,6 +308,29 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                 *reinterpret_cast<uint2*>(dvr + 32 * dt + 8 * a) = make_uint2(v0, v1);
             }
     }
+}
+
+// Sum of the hsplit partial dK / dV of a split launch, in a fixed order; one thread per (key, KV head, 4 features).
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_reduce_kernel(const AttnParams p) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t n = (int64_t)p.total_k * p.nkv * (D / 4);
+    if (idx >= n) return;
+    const int c = (int)(idx % (D / 4));
+    const int kvh = (int)((idx / (D / 4)) % p.nkv);
+    const int64_t key = idx / ((int64_t)(D / 4) * p.nkv);
+    const int64_t stride = (int64_t)p.total_k * p.nkv * D;
+    const int64_t off = (key * p.nkv + kvh) * D + 4 * c;
+    f32x4_t k4 = *reinterpret_cast<const f32x4_t*>(p.dk_part + off);
+    f32x4_t v4 = *reinterpret_cast<const f32x4_t*>(p.dv_part + off);
+    for (int s = 1; s < p.hsplit; ++s) {
+        k4 += *reinterpret_cast<const f32x4_t*>(p.dk_part + s * stride + off);
+        v4 += *reinterpret_cast<const f32x4_t*>(p.dv_part + s * stride + off);
+    }
+    *reinterpret_cast<uint2*>(p.dk + key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * c) =
+        make_uint2(pack_bf16x2(k4[0], k4[1]), pack_bf16x2(k4[2], k4[3]));
+    *reinterpret_cast<uint2*>(p.dv + key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * c) =
+        make_uint2(pack_bf16x2(v4[0], v4[1]), pack_bf16x2(v4[2], v4[3]));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -322,11 +360,10 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     const int lane = tid & 63, l32 = lane & 31, g = lane >> 5;
 
     const int nqb = (p.total_q + BM - 1) / BM;
-    const int work = xcd_remap(blockIdx.x, gridDim.x);
-    const int rep = work % p.n_rep;
-    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.n_docs, p.across_q, true);
-    const int kvh = work / (p.n_rep * nqb);
-    const int head = kvh * p.n_rep + rep;
+    int head, q_rank;
+    head_and_rank(blockIdx.x, p.nq, head, q_rank);
+    const int kvh = head / p.n_rep;
+    const int qb = block_for_rank(q_rank, nqb, p.n_docs, p.across_q, true);
     const int tq = qb * BM + wave * 32 + l32;
 
     int klo, khi;
@@ -495,11 +532,17 @@ template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) 
         if (rc != MI_OK) return rc;
     }
     if (all || (stages & MI_ATTN_BWD_DKDV)) {
-        const int64_t grid = (((int64_t)p.total_k + 127) / 128) * p.nkv;
+        const int64_t grid = (((int64_t)p.total_k + 127) / 128) * p.nkv * p.hsplit;
         if (p.drop_thr != 0) attn_bwd_dkdv_kernel<D, true><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         else attn_bwd_dkdv_kernel<D, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         int rc = mi_check_launch("attn_bwd_dkdv");
         if (rc != MI_OK) return rc;
+        if (p.hsplit > 1) {
+            const int64_t n = (int64_t)p.total_k * p.nkv * (D / 4);
+            attn_bwd_dkdv_reduce_kernel<D><<<dim3((unsigned)((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, st>>>(p);
+            rc = mi_check_launch("attn_bwd_dkdv_reduce");
+            if (rc != MI_OK) return rc;
+        }
     }
     if (all || (stages & MI_ATTN_BWD_DQ)) {
         const int64_t grid = (((int64_t)p.total_q + 255) / 256) * p.nq;
@@ -519,6 +562,26 @@ extern "C" size_t mi_attn_bwd_workspace_bytes(int64_t total_q, int32_t n_q_heads
     (void)head_dim;
     if (total_q <= 0 || n_q_heads <= 0) return 0;
     return (size_t)total_q * (size_t)n_q_heads * sizeof(float);
+}
+
+namespace {
+// query-head split of the dK/dV launch: enough workgroup groups for the 8 XCDs when there are fewer than 8 KV heads
+int dkdv_head_split(int nq, int nkv) {
+    const int n_rep = nq / nkv;
+    int h = 1;
+    while (nkv * h < 8 && n_rep % (2 * h) == 0) h *= 2;
+    return h;
+}
+size_t delta_bytes_aligned(int64_t total_q, int nq) { return ((size_t)total_q * (size_t)nq * sizeof(float) + 255) & ~(size_t)255; }
+}  // namespace
+
+extern "C" size_t mi_attn_bwd_workspace_bytes_kv(int64_t total_q, int64_t total_k, int32_t n_q_heads, int32_t n_kv_heads,
+                                                 int32_t head_dim) {
+    if (total_q <= 0 || total_k <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || head_dim <= 0)
+        return mi_attn_bwd_workspace_bytes(total_q, n_q_heads, head_dim);
+    const int h = dkdv_head_split(n_q_heads, n_kv_heads);
+    if (h == 1) return mi_attn_bwd_workspace_bytes(total_q, n_q_heads, head_dim);
+    return delta_bytes_aligned(total_q, n_q_heads) + (size_t)2 * h * (size_t)total_k * n_kv_heads * head_dim * sizeof(float);
 }
 
 extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
@@ -544,8 +607,19 @@ extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
     p.dk_st = b->dk_stride_token; p.dk_sh = b->dk_stride_head;
     p.dv_st = b->dv_stride_token; p.dv_sh = b->dv_stride_head;
     p.delta = (float*)b->workspace;
+    p.hsplit = 1;
+    {   // fewer than 8 KV heads: split the query heads of a group over workgroups if the workspace has room for the partials
+        const int h = dkdv_head_split(a->n_q_heads, a->n_kv_heads);
+        const size_t part = (size_t)h * (size_t)a->total_k * a->n_kv_heads * a->head_dim * sizeof(float);
+        const size_t base = delta_bytes_aligned(a->total_q, a->n_q_heads);
+        if (h > 1 && b->workspace_bytes >= base + 2 * part) {
+            p.hsplit = h;
+            p.dk_part = (float*)((char*)b->workspace + base);
+            p.dv_part = (float*)((char*)b->workspace + base + part);
+        }
+    }
     if (p.n_rep == 1) p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 256);                   // dQ: 256-query blocks
-    if (((a->total_k + 127) / 128) * p.nkv <= 1024) p.across_k = mi_blocks_per_doc(a->total_k, a->n_docs, 128);   // dK/dV: 128-key blocks
+    if (((a->total_k + 127) / 128) * p.nkv * p.hsplit <= 1024) p.across_k = mi_blocks_per_doc(a->total_k, a->n_docs, 128);   // dK/dV: 128-key blocks
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
         case 32: return launch_bwd<32>(p, a->flags, st);

@@ -33,6 +33,9 @@ struct AttnParams {
     // blocks per document on the query / key axis when the workgroups are to be handed out across documents
     // (see block_for_rank), 0 for the order along the flattened axis; set by the host entry points
     int across_q, across_k;
+    // dK/dV with fewer than 8 KV heads: the query heads of a group are split over hsplit workgroups per key block,
+    // each writing fp32 partial sums [hsplit][total_k][nkv][head_dim] that a reduce launch adds up (1 = no split)
+    int hsplit; float* dk_part; float* dv_part;
 };
 
 // ---- dropout mask ---------------------------------------------------------------------------------------
@@ -311,6 +314,23 @@ __device__ __forceinline__ void rotate_interleaved(uint4& v, const uint4& c, con
         float x0 = bf16_lo(w[i]), x1 = bf16_hi(w[i]);
         rotate_complex_pair(x0, x1, __uint_as_float(cw[i]), sign * __uint_as_float(sw[i]));
         w[i] = pack_bf16x2(x0, x1);
+    }
+}
+
+// Work item (query head, rank of its query block) of workgroup `linear` in a grid of n_heads * n_blocks workgroups
+// that hands an XCD the workgroups congruent to it modulo 8: every XCD gets whole heads (n_heads / 8 neighbouring
+// ones, which share K / V within a GQA group) with all their blocks, heaviest rank first, so the XCDs carry equal
+// work whatever the number of KV heads.  (Giving an XCD a contiguous slice of a kv-head-major item list, the
+// earlier scheme, coincides with this for 8 or more KV heads and leaves one XCD with all the long blocks for fewer:
+// multi-query attention ran 1.7x slower.)  Without a head count divisible by 8: head fastest, no XCD grouping.
+__device__ __forceinline__ void head_and_rank(int linear, int n_heads, int& head, int& rank) {
+    if ((n_heads & 7) == 0) {
+        const int hpx = n_heads >> 3, j = linear >> 3;
+        rank = j / hpx;
+        head = (linear & 7) * hpx + (j - rank * hpx);
+    } else {
+        rank = linear / n_heads;
+        head = linear - rank * n_heads;
     }
 }
 

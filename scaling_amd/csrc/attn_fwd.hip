@@ -50,11 +50,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
 
     // ---- work item ---------------------------------------------------------------------------
     const int nqb = (p.total_q + BM - 1) / BM;
-    const int work = xcd_remap(blockIdx.x, gridDim.x);
-    const int rep = work % p.n_rep;
-    const int qb = block_for_rank((work / p.n_rep) % nqb, nqb, p.n_docs, p.across_q, true);   // long query blocks first
-    const int kvh = work / (p.n_rep * nqb);
-    const int head = kvh * p.n_rep + rep;
+    int head, q_rank;
+    head_and_rank(blockIdx.x, p.nq, head, q_rank);
+    const int kvh = head / p.n_rep;
+    const int qb = block_for_rank(q_rank, nqb, p.n_docs, p.across_q, true);   // long query blocks first
 
     // ---- per-lane query, mask interval, Q fragment ---------------------------------------------
     const int tq = qb * BM + wave * 32 + l32;

@@ -515,7 +515,7 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
             dq = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
         dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
         dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
-        nbytes = lib.mi_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], q.shape[2])
+        nbytes = lib.mi_attn_bwd_workspace_bytes_kv(q.shape[0], k.shape[0], q.shape[1], k.shape[1], q.shape[2])
         ws = torch.empty(max(nbytes // 4, 4), dtype=torch.float32, device=q.device)
     b = MiAttnBwdArgs()
     b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, None, flags, dropout)

@@ -29,6 +29,10 @@ CASES = [
     (3, 256, 4, 4, 64, True, ()),              # ... forward / dQ (every query head has its own K / V)
     (2, 256, 4, 2, 128, True, ()),             # ... dK/dV (few workgroups)
     (1, 512, 4, 4, 64, True, (100,)),          # ... and two documents that only look equal-length from the host
+    # fewer than 8 KV heads: the dK/dV launch splits the query heads of a group over workgroups and sums partials
+    (2, 256, 8, 1, 128, True, (100, 300)),     # multi-query attention, 8-way split
+    (1, 384, 8, 2, 64, False, (129,)),         # 4-way split, bidirectional
+    (1, 320, 12, 4, 96, True, ()),             # group of 3: no split possible, the unsplit kernel
 ]
 
 
