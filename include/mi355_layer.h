@@ -273,6 +273,8 @@ int mi_attn_bwd(const mi_attn_bwd_args* args);
  * instead of torch.cat); with rotary_cos != NULL it rotates q and k_new by position_ids[b] before
  * use/append (fused rotary; rotary_interleaved selects the pairing and table format as in mi_attn_args).
  * o: [batch, n_q_heads, head_dim] contiguous; q likewise unless q_stride_batch is set.
+ * A workgroup serves up to 16 query heads of one KV head, so every K / V element is read once per 16 heads of its
+ * group (once in all for groups of up to 16; multi-query attention with 32 heads reads the cache twice).
  * The key axis is split into n_splits chunks processed by different workgroups and merged by a
  * second kernel; workspace = mi_attn_decode_workspace_bytes() bytes of fp32 scratch.
  * Algorithmic HBM bytes: 2 * sum_b ctx_len[b] * n_kv_heads * head_dim * e  (K and V read once).

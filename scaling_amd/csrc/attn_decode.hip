@@ -26,6 +26,7 @@ struct DecodeParams {
     const __bf16* cos; const __bf16* sin; const int64_t* pos; int table_rows;
     const float* cos32; const float* sin32;   // interleaved-pair rotary: fp32 tables [table_rows, D / 2]
     int batch, max_ctx, nq, nkv, n_rep, n_splits;
+    int n_hc;      // chunks of up to 16 query heads per KV head (a workgroup serves one chunk)
     int64_t c_sb, c_st, c_sh;
     int64_t q_sb, kn_sb, vn_sb;   // element strides between sequences of q / k_new / v_new
     float scale_log2;
@@ -94,8 +95,13 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     const int wave = tid >> 6, lane = tid & 63, l16 = lane & 15, G = lane >> 4;
 
     const int split = blockIdx.x % p.n_splits;
-    const int kvh = (blockIdx.x / p.n_splits) % p.nkv;
-    const int b = blockIdx.x / (p.n_splits * p.nkv);
+    const int kv_hc = (blockIdx.x / p.n_splits) % (p.nkv * p.n_hc);
+    const int kvh = kv_hc / p.n_hc, hc = kv_hc - kvh * p.n_hc;
+    const int b = blockIdx.x / (p.n_splits * p.nkv * p.n_hc);
+    // this workgroup's query heads: head0 .. head0 + n_heads of the group (groups of more than 16 heads take
+    // several workgroups, each reading the group's K / V once)
+    const int head0 = kvh * p.n_rep + 16 * hc;
+    const int n_heads = min(16, p.n_rep - 16 * hc);
 
     int ctx = p.ctx_len[b];
     ctx = ctx < 0 ? 0 : (ctx > p.max_ctx ? p.max_ctx : ctx);
@@ -109,8 +115,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     // Q^T fragments: column = head slot l16 (valid when < n_rep), contraction = features 32*ks + 8*G + i
     bf16x8_t qf[KS];
     {
-        const int hs = l16 < p.n_rep ? l16 : 0;
-        const __bf16* qr = p.q + (int64_t)b * p.q_sb + (int64_t)(kvh * p.n_rep + hs) * D + 8 * G;
+        const int hs = l16 < n_heads ? l16 : 0;
+        const __bf16* qr = p.q + (int64_t)b * p.q_sb + (int64_t)(head0 + hs) * D + 8 * G;
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qr + 32 * ks);
@@ -135,7 +141,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            if (l16 >= p.n_rep) raw[ks] = make_uint4(0, 0, 0, 0);
+            if (l16 >= n_heads) raw[ks] = make_uint4(0, 0, 0, 0);
             qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
         }
     }
@@ -257,14 +263,14 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     l_i += __shfl_xor(l_i, 32, 64);
     __syncthreads();
     if (G == 0) { wm_lds[wave][l16] = m_i; wl_lds[wave][l16] = l_i; }
-    if (l16 < p.n_rep) {
+    if (l16 < n_heads) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) wo_lds[wave][l16][16 * dt + 4 * G + r] = o_acc[dt][r];
     }
     __syncthreads();
-    for (int idx = tid; idx < p.n_rep * D; idx += kThreads) {
+    for (int idx = tid; idx < n_heads * D; idx += kThreads) {
         const int hs = idx / D, d = idx % D;
         float M = -INFINITY;
 #pragma unroll
@@ -277,7 +283,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
             L += f * wl_lds[w][hs];
             O += f * wo_lds[w][hs][d];
         }
-        const int64_t bh = (int64_t)b * p.nq + kvh * p.n_rep + hs;
+        const int64_t bh = (int64_t)b * p.nq + head0 + hs;
         if (p.n_splits == 1) {
             p.o[bh * D + d] = (__bf16)(L > 0.f ? O / L : 0.f);
         } else {
@@ -328,7 +334,7 @@ int choose_splits(int batch, int nkv, int max_ctx) {
 
 // rot: 0 = none, 1 = rotate-half, 2 = interleaved pairs
 template <int D, int NWV> int launch_split(const DecodeParams& p, int rot, hipStream_t st) {
-    const unsigned grid = (unsigned)p.batch * p.nkv * p.n_splits;
+    const unsigned grid = (unsigned)p.batch * p.nkv * p.n_hc * p.n_splits;
     if (rot == 2) decode_split_kernel<D, 2, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
     else if (rot == 1) decode_split_kernel<D, 1, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
     else decode_split_kernel<D, 0, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
@@ -342,7 +348,7 @@ template <int D> int launch_decode(const DecodeParams& p, bool append, int rot, 
         int rc = mi_check_launch("decode_append");
         if (rc != MI_OK) return rc;
     }
-    const int rc = wide_blocks(p.batch, p.nkv) ? launch_split<D, 8>(p, rot, st) : launch_split<D, 4>(p, rot, st);
+    const int rc = wide_blocks(p.batch, p.nkv * p.n_hc) ? launch_split<D, 8>(p, rot, st) : launch_split<D, 4>(p, rot, st);
     if (rc != MI_OK || p.n_splits == 1) return rc;
     const int64_t n = (int64_t)p.batch * p.nq * D;
     decode_merge_kernel<D><<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st>>>(p);
@@ -362,9 +368,8 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     if (!a->q || !a->k_cache || !a->v_cache || !a->o || !a->ctx_len) return mi_fail(MI_E_NULL, "attn_decode: q, caches, o and ctx_len are required");
     if (a->dtype != MI_BF16) return mi_fail(MI_E_DTYPE, "attn_decode: only bf16 is supported");
     if (a->head_dim != 64 && a->head_dim != 128) return mi_fail(MI_E_SHAPE, "attn_decode: head_dim %d unsupported (64, 128)", a->head_dim);
-    if (a->batch <= 0 || a->max_ctx <= 0 || a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0 ||
-        a->n_q_heads / a->n_kv_heads > 16)
-        return mi_fail(MI_E_SHAPE, "attn_decode: bad batch/head configuration (group size must be <= 16)");
+    if (a->batch <= 0 || a->max_ctx <= 0 || a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0)
+        return mi_fail(MI_E_SHAPE, "attn_decode: bad batch/head configuration");
     if ((a->k_new == nullptr) != (a->v_new == nullptr)) return mi_fail(MI_E_NULL, "attn_decode: k_new and v_new go together");
     const bool rot = a->rotary_cos != nullptr || a->rotary_sin != nullptr;
     if (rot && (!a->rotary_cos || !a->rotary_sin || !a->position_ids || a->rotary_table_rows <= 0))
@@ -381,7 +386,8 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
         (a->v_new_stride_batch && a->v_new_stride_batch < (int64_t)a->n_kv_heads * a->head_dim))
         return mi_fail(MI_E_SHAPE, "attn_decode: a sequence stride is smaller than heads * head_dim");
     if (!(a->softmax_scale > 0.f)) return mi_fail(MI_E_SHAPE, "attn_decode: softmax_scale must be positive");
-    int splits = a->n_splits > 0 ? a->n_splits : choose_splits(a->batch, a->n_kv_heads, a->max_ctx);
+    const int n_hc = (a->n_q_heads / a->n_kv_heads + 15) / 16;
+    int splits = a->n_splits > 0 ? a->n_splits : choose_splits(a->batch, a->n_kv_heads * n_hc, a->max_ctx);
     if (splits > kMaxSplits) splits = kMaxSplits;
     const size_t need = (size_t)a->batch * a->n_q_heads * splits * (size_t)(a->head_dim + 2) * sizeof(float);
     if (!a->workspace || a->workspace_bytes < need || !mi_aligned16(a->workspace))
@@ -397,7 +403,7 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     p.pos = a->position_ids;
     p.table_rows = (int)a->rotary_table_rows;
     p.batch = a->batch; p.max_ctx = a->max_ctx; p.nq = a->n_q_heads; p.nkv = a->n_kv_heads;
-    p.n_rep = a->n_q_heads / a->n_kv_heads; p.n_splits = splits;
+    p.n_rep = a->n_q_heads / a->n_kv_heads; p.n_splits = splits; p.n_hc = n_hc;
     p.c_sb = a->cache_stride_batch; p.c_st = a->cache_stride_token; p.c_sh = a->cache_stride_head;
     p.q_sb = a->q_stride_batch ? a->q_stride_batch : (int64_t)a->n_q_heads * a->head_dim;
     p.kn_sb = a->k_new_stride_batch ? a->k_new_stride_batch : (int64_t)a->n_kv_heads * a->head_dim;

@@ -35,6 +35,9 @@ def _oracle_decode(q, kc, vc, ctx, scale, dtype):
     (2, 4, 4, 64, 128, [128, 5]),
     (4, 32, 8, 128, 1100, [1024, 1025, 33, 1100]),
     (1, 16, 1, 128, 64, [64]),
+    # groups of more than 16 query heads (multi-query attention with 32 heads; 24 = one full and one partial chunk)
+    (2, 32, 1, 128, 300, [300, 17]),
+    (1, 24, 1, 64, 128, [128]),
     # batch x KV heads >= 192: the 8-wavefront workgroups (a single split writes the output directly)
     (24, 16, 8, 128, 300, [300, 1, 257, 31] * 6),
     (48, 8, 4, 64, 520, [520, 256, 255, 7, 300, 513] * 8),
