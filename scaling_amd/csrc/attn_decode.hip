@@ -84,7 +84,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     constexpr int DT = D / 16;          // 16-row tiles of O^T
     constexpr int VSTR = 2 * D + 32;    // bytes per key row of the staged V chunk: transpose reads of 8 rows x 32 bytes hit 256 distinct bytes
     constexpr int V_ITEMS = 8 * (D / 8);  // (key quad, feature group) items of a 32-key chunk
-    constexpr int V_PER_LANE = V_ITEMS / 64;
+    constexpr int V_PER_LANE = (V_ITEMS + 63) / 64;   // head_dim 32 / 96: the last round is partly empty
 
     __shared__ __attribute__((aligned(16))) char v_lds[NWV][kChunk * VSTR];
     __shared__ float wm_lds[NWV][16];
@@ -177,6 +177,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
             const int item = lane + 64 * j;
+            if (V_ITEMS % 64 != 0 && item >= V_ITEMS) break;
             const int quad = item / (D / 8), dg = item % (D / 8);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -230,6 +231,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
             for (int j = 0; j < V_PER_LANE; ++j) {
                 const int item = lane + 64 * j;
+                if (V_ITEMS % 64 != 0 && item >= V_ITEMS) break;
                 const int quad = item / (D / 8), dg = item % (D / 8);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) st128(vt + (4 * quad + r) * VSTR + 16 * dg, c.vraw[j][r]);
@@ -336,8 +338,11 @@ int choose_splits(int batch, int nkv, int max_ctx) {
 template <int D, int NWV> int launch_split(const DecodeParams& p, int rot, hipStream_t st) {
     const unsigned grid = (unsigned)p.batch * p.nkv * p.n_hc * p.n_splits;
     if (rot == 2) decode_split_kernel<D, 2, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
-    else if (rot == 1) decode_split_kernel<D, 1, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
-    else decode_split_kernel<D, 0, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
+    else if (rot == 1) {
+        // rotate-half pairs feature i with i + D / 2: the same lane holds both only when D / 32 is even
+        if constexpr (D == 64 || D == 128) decode_split_kernel<D, 1, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
+        else return mi_fail(MI_E_SHAPE, "attn_decode: fused rotate-half rotary needs head_dim 64 or 128");
+    } else decode_split_kernel<D, 0, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>(p);
     return mi_check_launch("decode_split");
 }
 
@@ -367,13 +372,16 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     if (!a) return mi_fail(MI_E_NULL, "attn_decode: args is null");
     if (!a->q || !a->k_cache || !a->v_cache || !a->o || !a->ctx_len) return mi_fail(MI_E_NULL, "attn_decode: q, caches, o and ctx_len are required");
     if (a->dtype != MI_BF16) return mi_fail(MI_E_DTYPE, "attn_decode: only bf16 is supported");
-    if (a->head_dim != 64 && a->head_dim != 128) return mi_fail(MI_E_SHAPE, "attn_decode: head_dim %d unsupported (64, 128)", a->head_dim);
+    if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 96 && a->head_dim != 128)
+        return mi_fail(MI_E_SHAPE, "attn_decode: head_dim %d unsupported (32, 64, 96, 128)", a->head_dim);
     if (a->batch <= 0 || a->max_ctx <= 0 || a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0)
         return mi_fail(MI_E_SHAPE, "attn_decode: bad batch/head configuration");
     if ((a->k_new == nullptr) != (a->v_new == nullptr)) return mi_fail(MI_E_NULL, "attn_decode: k_new and v_new go together");
     const bool rot = a->rotary_cos != nullptr || a->rotary_sin != nullptr;
     if (rot && (!a->rotary_cos || !a->rotary_sin || !a->position_ids || a->rotary_table_rows <= 0))
         return mi_fail(MI_E_NULL, "attn_decode: fused rotary needs cos, sin, position ids and the table size");
+    if (rot && !a->rotary_interleaved && a->head_dim != 64 && a->head_dim != 128)
+        return mi_fail(MI_E_SHAPE, "attn_decode: fused rotate-half rotary needs head_dim 64 or 128");
     if (!mi_aligned16(a->q) || !mi_aligned16(a->k_cache) || !mi_aligned16(a->v_cache) || !mi_aligned16(a->o) ||
         (a->k_new && (!mi_aligned16(a->k_new) || !mi_aligned16(a->v_new))) ||
         (rot && (!mi_aligned16(a->rotary_cos) || !mi_aligned16(a->rotary_sin))))
@@ -413,6 +421,10 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     p.ws_ml = p.ws_o + (size_t)a->batch * a->n_q_heads * splits * a->head_dim;
     hipStream_t st = (hipStream_t)a->stream;
     const int rot_mode = rot ? (a->rotary_interleaved ? 2 : 1) : 0;
-    if (a->head_dim == 64) return launch_decode<64>(p, a->k_new != nullptr, rot_mode, st);
-    return launch_decode<128>(p, a->k_new != nullptr, rot_mode, st);
+    switch (a->head_dim) {
+        case 32: return launch_decode<32>(p, a->k_new != nullptr, rot_mode, st);
+        case 64: return launch_decode<64>(p, a->k_new != nullptr, rot_mode, st);
+        case 96: return launch_decode<96>(p, a->k_new != nullptr, rot_mode, st);
+        default: return launch_decode<128>(p, a->k_new != nullptr, rot_mode, st);
+    }
 }

@@ -38,6 +38,10 @@ def _oracle_decode(q, kc, vc, ctx, scale, dtype):
     # groups of more than 16 query heads (multi-query attention with 32 heads; 24 = one full and one partial chunk)
     (2, 32, 1, 128, 300, [300, 17]),
     (1, 24, 1, 64, 128, [128]),
+    # the other head sizes of the attention kernels
+    (2, 4, 2, 96, 200, [200, 33]),
+    (3, 8, 8, 32, 100, [100, 1, 64]),
+    (40, 12, 6, 96, 70, [70, 69, 1, 35] * 10),
     # batch x KV heads >= 192: the 8-wavefront workgroups (a single split writes the output directly)
     (24, 16, 8, 128, 300, [300, 1, 257, 31] * 6),
     (48, 8, 4, 64, 520, [520, 256, 255, 7, 300, 513] * 8),

@@ -177,6 +177,19 @@ def test_cached_generation_matches_uncached_and_oracle(rotary):
     assert m["mean_rel"] <= max(1e-3, 1.25 * f["mean_rel"])
 
 
+@pytest.mark.parametrize("hidden,heads", [(384, 4), (128, 4)])
+def test_cached_generation_with_other_head_sizes(hidden, heads):
+    """head_dim 96 and 32: rotary runs as a stand-alone launch (the fused forms need 64 or 128) and the decode kernel
+    takes its other instantiations; the reference's invariant (cached == uncached tokens, logits within 1e-2) holds."""
+    cfg = _arch(hidden_size=hidden, num_attention_heads=heads, attention_num_kv_heads=2)
+    model = TransformerInferenceModule(cfg, device=DEV, init_std=0.2, seed=8)
+    prompt = [7, 3, 55, 20, 9]
+    tok_c, log_c = model.generate(5, prompt, use_cache=True)
+    tok_u, log_u = model.generate(5, prompt, use_cache=False)
+    assert tok_c == tok_u
+    assert torch.allclose(log_c.float(), log_u.float(), rtol=1e-2, atol=1e-2)
+
+
 def test_batched_cached_decode_equals_single_sequences(tmp_path):
     cfg = _arch(attention_num_kv_heads=1, hidden_size=512, num_attention_heads=4)   # head_dim 128, MQA
     model = TransformerInferenceModule(cfg, device=DEV, init_std=0.1, seed=4)
