@@ -180,6 +180,24 @@ def test_attention_with_separate_key_lengths(causal, nq, nkv, d):
         assert torch.count_nonzero(o[a:a + 6]) == 0 and torch.count_nonzero(qg.grad[a:a + 6]) == 0
 
 
+def test_attention_single_token_documents_return_v_exactly():
+    """Every token its own document: each query sees one key, the probability is exactly 1, so O = V (per KV group),
+    dV = dO summed over the group, dQ = dK = 0 up to rounding, whatever the tiling does with 700 documents in a 256-query block."""
+    T, nq, nkv, d = 700, 8, 2, 128
+    g = torch.Generator().manual_seed(21)
+    q, k, v, do = (torch.randn(T, n, d, generator=g).bfloat16().to(DEV) for n in (nq, nkv, nkv, nq))
+    cu = torch.arange(0, T + 1, dtype=torch.int32, device=DEV)
+    qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
+    o = ops.attention(qg, kg, vg, cu, None, True, None)
+    o.backward(do)
+    torch.cuda.synchronize()
+    assert torch.equal(o, v.repeat_interleave(nq // nkv, dim=1))
+    # dS = P * (dP - delta) with dP and delta two fp32 evaluations of the same dot product: rounding noise only
+    assert qg.grad.float().abs().max().item() <= 1e-5 and kg.grad.float().abs().max().item() <= 1e-5
+    dv_ref = do.float().view(T, nkv, nq // nkv, d).sum(dim=2)
+    assert torch.allclose(vg.grad.float(), dv_ref, rtol=1e-2, atol=1e-2)
+
+
 def _complex_tables(d, rows, base):
     """fp32 [rows, d / 2] real / imaginary parts of freqs_cis (core/nn/rotary.py:45-56)."""
     inv_freq = 1.0 / (float(base) ** (torch.arange(0, d, 2)[: d // 2].float() / d))
