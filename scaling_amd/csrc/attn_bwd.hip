@@ -81,11 +81,24 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     const int kgp = wave & 3, sub = wave >> 2;
 
     const int nkb = (p.total_k + BNK - 1) / BNK;
-    const int work = xcd_remap(blockIdx.x, gridDim.x);
-    const int kb = block_for_rank(work % nkb, nkb, p.n_docs, p.across_k, false);   // key blocks with the most queries first
+    // (KV head, head split) groups x key-block ranks.  With a multiple of 8 groups every XCD receives whole groups
+    // with all their key blocks (the same Q / dO stream through its L2, equal work per XCD); otherwise a contiguous
+    // slice per XCD would give one XCD a group's heavy key blocks and another its light ones, so the items go out
+    // rank-major and every XCD sees every rank.
+    const int n_groups = p.nkv * p.hsplit;
+    int kb_rank, group;
+    if ((n_groups & 7) == 0) {
+        const int work = xcd_remap(blockIdx.x, gridDim.x);
+        kb_rank = work % nkb;
+        group = work / nkb;
+    } else {
+        kb_rank = blockIdx.x / n_groups;
+        group = blockIdx.x - kb_rank * n_groups;
+    }
+    const int kb = block_for_rank(kb_rank, nkb, p.n_docs, p.across_k, false);   // key blocks with the most queries first
     const int hpw = p.n_rep / p.hsplit;   // query heads of this workgroup: hs * hpw .. + hpw of the group
-    const int kvh = (work / nkb) / p.hsplit;
-    const int hs = (work / nkb) - kvh * p.hsplit;
+    const int kvh = group / p.hsplit;
+    const int hs = group - kvh * p.hsplit;
     const int key = kb * BNK + kgp * 32 + l32;
 
     int qlo, qhi;
