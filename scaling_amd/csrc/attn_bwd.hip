@@ -1,11 +1,13 @@
 // Attention backward for gfx950 (bf16 MFMA, fp32 softmax recomputation from the saved log-sum-exp).
 //
-// Three kernels, no atomics, fixed summation order (bit-reproducible):
+// Three kernels (four with fewer than 8 KV heads), no atomics, fixed summation order (bit-reproducible):
 //   1. delta[h][t] = sum_d dO[t][h][d] * O[t][h][d]
 //   2. dK/dV: a workgroup owns 128 keys of one KV head (K and V rows stay in LDS), loops over the query
 //      heads of the group and over 64-query tiles staged in LDS:
 //          S = Q K^T,  P = exp2(S*c - lse),  dP = dO V^T,  dS = P * (dP - delta)
 //          dV^T += dO^T P        dK^T += Q^T dS         (P / dS feed the MFMA straight from registers)
+//      With fewer than 8 KV heads the query heads of a group are split over workgroups, which write fp32 partial
+//      dK / dV that a small reduce kernel sums in a fixed order (enough workgroups for all compute units).
 //   3. dQ: a workgroup owns 256 queries of one head (32 per wavefront, Q and dO fragments in registers),
 //      loops over 64-key tiles:  S^T = K Q^T, dP^T = V dO^T, dS^T, dQ^T += K^T dS^T.
 // Tiles whose rows are needed both as row operands and transposed (Q / dO in kernel 2, K in kernel 3) are
