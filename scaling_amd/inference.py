@@ -176,6 +176,10 @@ class TransformerInferenceModule(torch.nn.Module):
         fuse_add_norm = all(isinstance(n, RMSNorm) for layer in layers for n in (layer.input_layernorm, layer.post_attention_layernorm)) \
             and isinstance(final_norm, RMSNorm)
 
+        # arg-max over the vocabulary by the streaming cross-entropy kernel (first index of the maximum, as
+        # torch.argmax): ~8 us for [32, 128256] against ~48 us for torch's reduction
+        no_target = torch.zeros(b, dtype=torch.int64, device=self.device)
+
         def one_step():
             h = self._layers[0](tok)
             shared_ctx.add_(1)
@@ -193,7 +197,7 @@ class TransformerInferenceModule(torch.nn.Module):
                 for layer in layers:
                     h = layer.decode_step(h, pos, advance=False)
                 lg = self._layers[-1].linear(final_norm(h))
-            nxt = torch.argmax(lg, dim=-1)                                # [b, 1]
+            nxt = ops.cross_entropy_forward(lg.view(b, -1), no_target)[1].to(torch.int64).view(b, 1)
             out.index_copy_(1, step, nxt)
             tok.copy_(nxt)
             pos.add_(1)
