@@ -312,6 +312,18 @@ typedef struct mi_decode_args {
 size_t mi_attn_decode_workspace_bytes(int32_t batch, int32_t n_q_heads, int32_t head_dim, int32_t max_ctx);
 int mi_attn_decode(const mi_decode_args* args);
 
+/* mi_attn_decode for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, kernels and results
+ * as mi_attn_decode, except that `workspace` / `workspace_bytes` are ignored: the per-split partial results go to
+ * a static device array inside the library (mi_attn_decode_static_scratch_bytes() bytes, 8 MiB, held by every GPU
+ * the library runs on until the process ends).  The call allocates and frees nothing.  It returns MI_E_WORKSPACE
+ * when batch * n_q_heads * n_splits * (head_dim + 2) * 4 bytes exceed the array (n_splits as chosen by the library
+ * or given, at most 32).  All calls on one GPU share that GPU's array: calls that may overlap on one GPU (different
+ * streams, different threads) race and must be serialised by the caller; nothing in the array has to be cleared
+ * between calls (every slot a call reads was written by the same call). */
+size_t mi_attn_decode_static_scratch_bytes(void);
+int mi_attn_decode_static(const mi_decode_args* args);
+
 #ifdef __cplusplus
 }
 #endif

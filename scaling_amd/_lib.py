@@ -22,7 +22,7 @@ EXPORTS = (
     "mi_layernorm_fwd", "mi_layernorm_bwd_workspace_bytes", "mi_layernorm_bwd", "mi_gelu_fwd", "mi_gelu_bwd", "mi_cross_entropy",
     "mi_swiglu_fwd", "mi_swiglu_bwd", "mi_rotary", "mi_rotary_complex",
     "mi_attn_fwd", "mi_attn_bwd_workspace_bytes", "mi_attn_bwd_workspace_bytes_kv", "mi_attn_bwd",
-    "mi_attn_decode_workspace_bytes", "mi_attn_decode",
+    "mi_attn_decode_workspace_bytes", "mi_attn_decode", "mi_attn_decode_static_scratch_bytes", "mi_attn_decode_static",
 )
 
 
@@ -129,6 +129,10 @@ def _declare(lib):
     lib.mi_attn_decode_workspace_bytes.argtypes = [c_int32, c_int32, c_int32, c_int32]
     lib.mi_attn_decode.restype = c_int
     lib.mi_attn_decode.argtypes = [POINTER(MiDecodeArgs)]
+    lib.mi_attn_decode_static_scratch_bytes.restype = c_size_t
+    lib.mi_attn_decode_static_scratch_bytes.argtypes = []
+    lib.mi_attn_decode_static.restype = c_int
+    lib.mi_attn_decode_static.argtypes = [POINTER(MiDecodeArgs)]
 
 
 def load(path: str = LIB_PATH):

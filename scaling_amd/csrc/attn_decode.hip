@@ -12,6 +12,8 @@
 // applies rotary to it; the query is rotated while its fragments are loaded.
 #include "attn_common.h"
 
+#include <mutex>
+
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 namespace {
@@ -368,7 +370,10 @@ extern "C" size_t mi_attn_decode_workspace_bytes(int32_t batch, int32_t n_q_head
     return (size_t)batch * n_q_heads * kMaxSplits * (size_t)(head_dim + 2) * sizeof(float);
 }
 
-extern "C" int mi_attn_decode(const mi_decode_args* a) {
+namespace {
+// Validation and launches shared by the two entry points; `ws` / `ws_bytes` is the scratch for the per-split partial
+// results (the caller's workspace, or the library's own static array for mi_attn_decode_static).
+int decode_entry(const mi_decode_args* a, void* ws, size_t ws_bytes, bool static_ws) {
     if (!a) return mi_fail(MI_E_NULL, "attn_decode: args is null");
     if (!a->q || !a->k_cache || !a->v_cache || !a->o || !a->ctx_len) return mi_fail(MI_E_NULL, "attn_decode: q, caches, o and ctx_len are required");
     if (a->dtype != MI_BF16) return mi_fail(MI_E_DTYPE, "attn_decode: only bf16 is supported");
@@ -398,8 +403,12 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     int splits = a->n_splits > 0 ? a->n_splits : choose_splits(a->batch, a->n_kv_heads * n_hc, a->max_ctx);
     if (splits > kMaxSplits) splits = kMaxSplits;
     const size_t need = (size_t)a->batch * a->n_q_heads * splits * (size_t)(a->head_dim + 2) * sizeof(float);
-    if (!a->workspace || a->workspace_bytes < need || !mi_aligned16(a->workspace))
-        return mi_fail(MI_E_WORKSPACE, "attn_decode: workspace needs %zu bytes (16-byte aligned), got %zu", need, a->workspace_bytes);
+    if (static_ws && need > ws_bytes)
+        return mi_fail(MI_E_WORKSPACE, "attn_decode_static: batch %d x %d query heads x %d key splits x head_dim %d needs %zu bytes of "
+                       "scratch, the library's static array holds %zu; use mi_attn_decode with a caller workspace",
+                       a->batch, a->n_q_heads, splits, a->head_dim, need, ws_bytes);
+    if (!ws || ws_bytes < need || !mi_aligned16(ws))
+        return mi_fail(MI_E_WORKSPACE, "attn_decode: workspace needs %zu bytes (16-byte aligned), got %zu", need, ws_bytes);
     DecodeParams p{};
     p.q = (const __bf16*)a->q; p.kc = (__bf16*)a->k_cache; p.vc = (__bf16*)a->v_cache; p.o = (__bf16*)a->o;
     p.ctx_len = a->ctx_len; p.k_new = (const __bf16*)a->k_new; p.v_new = (const __bf16*)a->v_new;
@@ -417,7 +426,7 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
     p.kn_sb = a->k_new_stride_batch ? a->k_new_stride_batch : (int64_t)a->n_kv_heads * a->head_dim;
     p.vn_sb = a->v_new_stride_batch ? a->v_new_stride_batch : (int64_t)a->n_kv_heads * a->head_dim;
     p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
-    p.ws_o = (float*)a->workspace;
+    p.ws_o = (float*)ws;
     p.ws_ml = p.ws_o + (size_t)a->batch * a->n_q_heads * splits * a->head_dim;
     hipStream_t st = (hipStream_t)a->stream;
     const int rot_mode = rot ? (a->rotary_interleaved ? 2 : 1) : 0;
@@ -427,4 +436,50 @@ extern "C" int mi_attn_decode(const mi_decode_args* a) {
         case 96: return launch_decode<96>(p, a->k_new != nullptr, rot_mode, st);
         default: return launch_decode<128>(p, a->k_new != nullptr, rot_mode, st);
     }
+}
+}  // namespace
+
+extern "C" int mi_attn_decode(const mi_decode_args* a) {
+    if (!a) return mi_fail(MI_E_NULL, "attn_decode: args is null");
+    return decode_entry(a, a->workspace, a->workspace_bytes, false);
+}
+
+// ---- entry point that allocates nothing ------------------------------------------------------------------------
+// The per-split partial results live in a file-scope device array instead of a caller workspace.  Every GPU the
+// library's code object is loaded on holds its own copy of the array at its own address, obtained once per device with
+// hipGetSymbolAddress (the array's name is only a host-side handle, not a device address) and kept in g_scratch_ptr.
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];        // per device; written once, under g_scratch_mutex
+std::mutex g_scratch_mutex;
+
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return mi_fail(MI_E_LAUNCH, "attn_decode_static: hipGetDevice failed or device index %d out of range (%s)", dev, hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return mi_fail(MI_E_LAUNCH, "attn_decode_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return MI_OK;
+}
+}  // namespace
+
+extern "C" size_t mi_attn_decode_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int mi_attn_decode_static(const mi_decode_args* a) {
+    if (!a) return mi_fail(MI_E_NULL, "attn_decode_static: args is null");
+    void* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != MI_OK) return rc;
+    return decode_entry(a, ws, kStaticScratchBytes, true);
 }

@@ -21,6 +21,12 @@ def get_cumulative_seq_lengths(input_token_ids: torch.Tensor, reset_attention_ma
     return torch.cat((torch.zeros(1, dtype=torch.int32, device=dev), ends.to(torch.int32)))
 
 
+def get_max_seq_length(cumulative_seq_lengths: torch.Tensor) -> int:
+    """core/nn/attention/attention.py:72-73: length of the longest document (a host integer; the reference hands it
+    to its flash-attention call, the hip kernels size their loops from the cumulative lengths themselves)."""
+    return int(torch.diff(cumulative_seq_lengths).max().item())
+
+
 def get_position_ids(input_token_ids: torch.Tensor, reset_position_ids: bool = True,
                      eod_token: int = EOD_TOKEN) -> torch.Tensor:
     b, s = input_token_ids.shape

@@ -17,7 +17,6 @@ from pathlib import Path
 from typing import Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
-import torch.nn.functional as F
 
 from .config import TransformerArchitectureConfig, architecture_from_config_file
 from .data import get_cumulative_seq_lengths, get_position_ids
@@ -73,6 +72,9 @@ class TransformerInferenceModule(torch.nn.Module):
             self._layers[-1].linear.weight = self._layers[0].embedding.weight
         else:
             init(self._layers[-1].linear.weight)
+        # core/nn/parallel_module/inference_module.py:98: an inference module is in eval mode from construction, so the
+        # dropouts of a training config (after attention, after the MLP, on the attention probabilities) are off
+        self.eval()
 
     # ---- checkpoint files ------------------------------------------------------------------------------
     def load_checkpoint(self, checkpoint_dir: Union[str, Path]) -> None:

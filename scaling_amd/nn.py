@@ -28,6 +28,22 @@ def _default_device(device, topology=None) -> torch.device:
     return torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available() else torch.device("cpu")
 
 
+_CHECKED: Dict[str, tuple] = {}
+
+
+def _checked_once(kind: str, t: torch.Tensor, extra: tuple, compute: Callable[[], bool]) -> bool:
+    """Result of a device-side validation of tensor `t` that needs a host read-back: computed once per tensor and
+    kind, so the layers of one forward share it.  The tensor is identified by address, layout and version counter,
+    and the last validated one is kept alive here, so its memory cannot be handed to another tensor meanwhile."""
+    key = (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t._version, t.device, extra)
+    hit = _CHECKED.get(kind)
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    ok = compute()
+    _CHECKED[kind] = (key, ok, t)
+    return ok
+
+
 class _Linear(torch.nn.Module):
     """weight [out, in] (+ bias [out]): the parameter layout of the reference's Column/RowParallelLinear
     at model-parallel size 1 (core/nn/linear/column_parallel_linear.py:109-116, row_parallel_linear.py:117-124)."""
@@ -216,6 +232,81 @@ class ParallelMLP(torch.nn.Module):
         return self.dense_out(ops.gelu(self.dense_in(x)))
 
 
+class MaskedSoftmax(torch.nn.Module):
+    """Mirror of core/nn/masked_softmax/masked_softmax.py:37-52: holds the config and resolves the kernel.  As for the
+    reference's fused flash-attention kernel, `kernel` is None for `hip` (the softmax runs inside the attention
+    kernels, always in fp32, with `config.scale` folded into the score scale) and calling the module asserts;
+    any other kernel raises NotImplementedError at construction."""
+
+    def __init__(self, config: MaskedSoftmaxConfig) -> None:
+        super().__init__()
+        self.config = config
+        self.kernel: Optional[torch.nn.Module]
+        if self.config.kernel == MaskedSoftmaxKernel.HIP:
+            self.kernel = None
+        else:
+            raise NotImplementedError(f"kernel {self.config.kernel} not implemented (this package provides masked_softmax.kernel = 'hip' only)")
+
+    def forward(self, x: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+        assert self.kernel is not None
+        return self.kernel(x=x, mask=mask)
+
+
+class ScaledDotProductAttention(torch.nn.Module):
+    """Mirror of core/nn/attention/attention.py:280-395 backed by the fused kernels: same constructor, attributes
+    (`head_dim`, `dropout_p`, `softmax_fn`, `dropout_fn`, `masked_softmax_config`, `query_key_scaling_factor`,
+    `causal`, `use_matmul`) and forward signature.  `forward` takes the reference's layout (query [s_q, b, n, d],
+    key / value [s_k, b, n_kv, d]; the KV heads need not be repeated) and returns [(b n), s_q, d];
+    `forward_tokens` is the copy-free form on token-major tensors that ParallelSelfAttention uses."""
+
+    def __init__(self, head_dim: int, dropout_p: float, masked_softmax_config: MaskedSoftmaxConfig, causal: bool,
+                 use_matmul: bool = False, umup_mult: Optional[float] = None):
+        super().__init__()
+        if umup_mult is not None:
+            raise NotImplementedError("u-muP scaling is outside the hip kernel's scope")
+        self.head_dim = head_dim
+        self.dropout_p = dropout_p
+        self.softmax_fn = MaskedSoftmax(masked_softmax_config)
+        self.dropout_fn = torch.nn.Dropout(p=dropout_p)   # kept for the module tree; the kernels draw their own mask
+        self.masked_softmax_config = masked_softmax_config
+        self.query_key_scaling_factor: float = 1 / (head_dim ** 0.5)
+        self.causal = causal
+        self.use_matmul = use_matmul
+        self.umup_mult = None
+        self._use_umup = False
+
+    @property
+    def softmax_scale(self) -> float:
+        """alpha of the score product times masked_softmax.scale (attention.py:154-160 with masked_softmax.py:21-22)."""
+        return self.query_key_scaling_factor * self.masked_softmax_config.scale
+
+    def forward_tokens(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cumulative_seq_lengths: torch.Tensor,
+                       cumulative_seq_lengths_key: Optional[torch.Tensor] = None, rotary=None) -> torch.Tensor:
+        """q [tokens, n, d], k / v [tokens_k, n_kv, d] (views with contiguous features) -> [tokens, n, d]."""
+        return ops.attention(q, k, v, cumulative_seq_lengths, cumulative_seq_lengths_key, self.causal, self.softmax_scale,
+                             dropout_p=self.dropout_p if self.training else 0.0, rotary=rotary,
+                             deterministic=self.masked_softmax_config.deterministic_flash_attn_bwd)
+
+    def forward(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, cumulative_seq_lengths: torch.Tensor,
+                attention_scores_manipulation: Optional[torch.Tensor] = None,
+                attentions_score_manipulation_log_additive=True) -> torch.Tensor:
+        if attention_scores_manipulation is not None:
+            raise NotImplementedError("attention_scores_manipulation is not available with the hip kernel")
+        s_q, b, n, d = query.shape
+
+        def tokens(x):
+            return x.permute(1, 0, 2, 3).reshape(b * x.shape[0], x.shape[2], d)
+
+        cu = cumulative_seq_lengths.to(torch.int32)
+        if key.shape[0] != s_q:   # cached decoding in the reference's layout: every row is one document with its own key length
+            assert cu.numel() == b + 1, "differing query and key lengths need one document per batch row"
+            cu_k = torch.arange(0, b * key.shape[0] + 1, key.shape[0], dtype=torch.int32, device=cu.device)
+        else:
+            cu_k = None
+        out = self.forward_tokens(tokens(query), tokens(key), tokens(value), cu, cu_k)
+        return out.view(b, s_q, n, d).permute(0, 2, 1, 3).reshape(b * n, s_q, d)
+
+
 class KVCache:
     """Pre-allocated cache of post-rotary K and un-repeated V, indexed [batch, token, kv head, d], replacing
     the reference's per-step torch.cat (core/nn/attention/attention.py:862-869).  Storage is head-major
@@ -259,12 +350,12 @@ class ParallelSelfAttention(torch.nn.Module):
         self._device = _default_device(device, topology)
         assert hidden_size % num_attention_heads == 0, \
             f"hidden size ({hidden_size}) must be divisible by num_attention_heads ({num_attention_heads})"
-        if masked_softmax_config.kernel != MaskedSoftmaxKernel.HIP:
-            raise NotImplementedError(
-                f"this module implements masked_softmax.kernel = 'hip' only (got '{masked_softmax_config.kernel.value}'); "
-                "the other kernels live in the reference implementation")
         assert 0.0 <= dropout_attention_probs < 1.0, "dropout_attention_probs must be in [0, 1)"
         self.dropout_attention_probs = float(dropout_attention_probs)   # applied in training mode only
+        # attention.py:734-743; raises NotImplementedError for any masked_softmax.kernel other than `hip`
+        self.scaled_dot_product_attention = ScaledDotProductAttention(
+            head_dim=hidden_size // num_attention_heads, dropout_p=self.dropout_attention_probs,
+            masked_softmax_config=masked_softmax_config, causal=causal, use_matmul=use_matmul)
         if num_local_attention_heads > 0 or lora_config is not None or fp8_config is not None or \
                 fp8_config_dense_out is not None or bitfit_bias_name is not None:
             raise NotImplementedError("local attention, LoRA, fp8 and bitfit are outside the hip kernel's scope")
@@ -319,15 +410,11 @@ class ParallelSelfAttention(torch.nn.Module):
             self.norm_key = get_norm(norm_type, layernorm_config, d, self._device, dtype)
 
         # softmax_fn scale: alpha * masked_softmax.scale (attention.py:297 with masked_softmax.py:21-22)
-        self.query_key_scaling_factor = 1.0 / math.sqrt(d)
-        self.softmax_scale = self.query_key_scaling_factor * masked_softmax_config.scale
+        self.query_key_scaling_factor = self.scaled_dot_product_attention.query_key_scaling_factor
+        self.softmax_scale = self.scaled_dot_product_attention.softmax_scale
         self.dense = _Linear(hidden_size, hidden_size, bias, self._device, dtype, init_method)
         self.cache: Dict[int, Optional[KVCache]] = dict()
         self.max_cache_length = max_cache_length
-
-    # ---- reference API that callers of every ParallelSelfAttention instance use ---------------------
-    def merge_lora_weights(self) -> None:  # core/trainer/trainer.py:87-92 calls this unconditionally
-        return None
 
     # ---- helpers --------------------------------------------------------------------------------
     def _project(self, x: torch.Tensor):
@@ -336,8 +423,9 @@ class ParallelSelfAttention(torch.nn.Module):
         if self.qkv_in_one:
             qkv = self.query_key_value(x).view(b * s, nq, 3 * d)       # per head: q then k then v (attention.py:790-796)
             return qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:]
-        if not torch.is_grad_enabled():
-            # inference: one projection GEMM over the row-stacked weights; q, k, v are column slices of its output
+        if not torch.is_grad_enabled() and not self.training:
+            # inference (eval mode, so that a no-grad forward that activation checkpointing recomputes with grad takes
+            # the same GEMMs both times): one projection GEMM over the row-stacked weights; q, k, v are column slices
             w, bias = self._fused_qkv()
             out = F.linear(x, w, bias).view(b * s, (nq + 2 * nkv) * d)
             return (out[:, :nq * d].view(b * s, nq, d), out[:, nq * d:(nq + nkv) * d].view(b * s, nkv, d),
@@ -378,9 +466,26 @@ class ParallelSelfAttention(torch.nn.Module):
         ok = t.stride(2) == 1 and t.stride(1) == t.shape[2] and t.stride(0) % 8 == 0
         return t if ok else t.contiguous()
 
-    @staticmethod
-    def _rows_are_single_documents(cu: torch.Tensor, b: int, s: int) -> bool:
-        return cu.numel() == b + 1 and bool(torch.equal(cu.cpu(), torch.arange(0, b * s + 1, s, dtype=cu.dtype)))
+    def _rows_are_single_documents(self, cu: torch.Tensor, b: int, s: int) -> bool:
+        """True when every batch row is one document.  A decode step (s == 1) needs the shape only: b + 1 strictly
+        increasing offsets that end at b are 0..b.  A prefill compares on the device and reads the answer back once
+        per cumulative-lengths tensor (all layers of a forward receive the same one), not once per layer."""
+        if cu.numel() != b + 1:
+            return False
+        if s == 1:
+            return True
+        return _checked_once("single_documents", cu, (b, s),
+                             lambda: bool(torch.equal(cu, torch.arange(0, b * s + 1, s, dtype=cu.dtype, device=cu.device))))
+
+    def _check_positions(self, pos: Optional[torch.Tensor]) -> None:
+        """The reference gathers cos / sin rows by position id (rotary.py:128-131) and raises on an id outside the
+        table; the kernels would clamp instead, so the ids are validated here, once per position-id tensor."""
+        if pos is None or self.rotary_embedding is None or pos.numel() == 0:
+            return
+        rows = self.rotary_embedding.max_seq_length
+        ok = _checked_once("positions", pos, (rows,), lambda: bool(((pos >= 0) & (pos < rows)).all()))
+        if not ok:
+            raise IndexError(f"position ids outside the rotary table of {rows} rows")
 
     def forward(self, x: torch.Tensor, cumulative_seq_lengths: torch.Tensor, position_ids: Optional[torch.Tensor],
                 cumulative_seq_lengths_key: Optional[torch.Tensor] = None, use_cache: bool = False,
@@ -396,6 +501,7 @@ class ParallelSelfAttention(torch.nn.Module):
             k = self.norm_key(k)
         pos = None if position_ids is None else position_ids.reshape(-1).contiguous()
         cu = cumulative_seq_lengths.to(torch.int32)
+        sdpa = self.scaled_dot_product_attention
 
         if use_cache:
             if not self.causal:
@@ -405,21 +511,20 @@ class ParallelSelfAttention(torch.nn.Module):
                 return self.dense(self._decode_step(q, k, v, pos, b, s, cache_index).view(b, s, nq * d))
         elif reset_cache:
             self.cache[cache_index] = None
+        self._check_positions(pos)
+        cu_k = None if cumulative_seq_lengths_key is None else cumulative_seq_lengths_key.to(torch.int32)
 
-        if self._fusable_rotary and not use_cache and not torch.is_grad_enabled() and pos is not None:
-            # inference without cache: rotary is applied while the kernel loads Q and K
+        if self._fusable_rotary and pos is not None and not use_cache:
+            # rotary is applied while the kernels load Q and K (forward and backward); nothing rotated is stored
             cos, sin = self.rotary_embedding.tables()
-            cu_k = None if cumulative_seq_lengths_key is None else cumulative_seq_lengths_key.to(torch.int32)
-            ctx, _ = ops.attention_forward(q, k, v, cu, cu_k, self.causal, self.softmax_scale, rotary=(cos, sin, pos, pos))
+            ctx = sdpa.forward_tokens(q, k, v, cu, cu_k, rotary=(cos, sin, pos, pos))
             return self.dense(ctx.view(b, s, nq * d))
         if self.rotary_embedding is not None:
             q = self.rotary_embedding.rotate_tokens(q, pos, s)
             k = self.rotary_embedding.rotate_tokens(k, pos, s)
         if use_cache:  # prefill: keep post-rotary K and V (attention.py:861-862)
             self._fill_cache(k, v, b, s, cache_index)
-        ctx = ops.attention(q, k, v, cu, None if cumulative_seq_lengths_key is None else cumulative_seq_lengths_key.to(torch.int32),
-                            self.causal, self.softmax_scale,
-                            dropout_p=self.dropout_attention_probs if self.training else 0.0)
+        ctx = sdpa.forward_tokens(q, k, v, cu, cu_k)
         return self.dense(ctx.view(b, s, nq * d))
 
     # ---- KV cache ----------------------------------------------------------------------------------
@@ -484,6 +589,8 @@ class ParallelSelfAttention(torch.nn.Module):
         cache.ctx_len.add_(1)
         rotary = None
         if self.rotary_embedding is not None:
+            if cache.length > self.rotary_embedding.max_seq_length:
+                raise IndexError(f"position {cache.length - 1} is outside the rotary table of {self.rotary_embedding.max_seq_length} rows")
             if pos is None:
                 pos = torch.full((b,), cache.length - 1, dtype=torch.int64, device=q.device)
             if self._fusable_rotary:

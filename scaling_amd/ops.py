@@ -556,18 +556,30 @@ def next_dropout_seed(device: torch.device) -> int:
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
               cu_seqlens_k: Optional[torch.Tensor] = None, causal: bool = True,
               softmax_scale: Optional[float] = None, dropout_p: float = 0.0,
-              dropout_seed: Optional[int] = None) -> torch.Tensor:
+              dropout_seed: Optional[int] = None, rotary=None, deterministic: bool = False) -> torch.Tensor:
     """Differentiable attention core on q [tokens, n_q, d], k/v [tokens_k, n_kv, d] (bf16).
 
     Tokens are the flattened (batch seq) axis; cu_seqlens are int32 offsets on it.  Returns
     o [tokens, n_q, d].  dropout_p > 0 drops attention probabilities (attention.py:204-207) with a mask that
     is a function of (dropout_seed, head, query, key); without a seed one is drawn from the device generator.
     The drop probability is quantised to round(256 p) / 256.
+
+    rotary = (cos, sin, position_ids_q, position_ids_k) applies the rotary embedding of the whole head to q and k
+    (attention.py:836-845; table formats as for attention_forward) and differentiates through it.
+    deterministic mirrors masked_softmax.deterministic_flash_attn_bwd of the reference.
     """
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
     if dropout_p > 0.0 and dropout_seed is None:
         dropout_seed = next_dropout_seed(q.device)
+    if rotary is not None:
+        cos, sin, pos_q, pos_k = rotary
+        interleaved = _fused_rotary_kind(cos, sin, q.shape[2], q.dtype)
+        needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
+        if not needs_grad and dropout_p == 0.0:
+            return attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary=rotary)[0]
+        rot = rotary_embedding_complex if interleaved else rotary_embedding
+        q, k = rot(q, cos, sin, pos_q), rot(k, cos, sin, pos_k)
     return _Attention.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, float(softmax_scale), float(dropout_p),
                             int(dropout_seed) if dropout_seed is not None else 0)
 
@@ -584,12 +596,14 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
                      rotary: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None,
                      softmax_scale: Optional[float] = None, workspace: Optional[torch.Tensor] = None,
-                     n_splits: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     n_splits: int = 0, out: Optional[torch.Tensor] = None, static_scratch: bool = False) -> torch.Tensor:
     """One decode step.  q [B, n_q, d]; caches [B, max_ctx, n_kv, d]; ctx_len int32 [B] counts the valid
     keys INCLUDING the token appended by this call (k_new/v_new [B, n_kv, d], written at ctx_len-1).
     rotary = (cos, sin, position_ids[B]) rotates q and k_new inside the kernels (table formats as for
     attention_forward: rotate-half or interleaved pairs).  q, k_new and v_new may be
-    column slices of one projection output: only their [heads, d] part has to be contiguous."""
+    column slices of one projection output: only their [heads, d] part has to be contiguous.
+    static_scratch=True calls the entry point that allocates nothing (partial results in the library's static
+    device array; `out` should be given too, and calls on one GPU must not overlap)."""
     _need_cuda(q, k_cache, v_cache, ctx_len)
     B, nq, d = q.shape
 
@@ -602,7 +616,7 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     assert ctx_len.dtype == torch.int32 and ctx_len.numel() == B
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
-    if workspace is None:
+    if workspace is None and not static_scratch:
         workspace = decode_workspace(B, nq, d, k_cache.shape[1], q.device)
     if out is None:
         out = torch.empty((B, nq, d), dtype=q.dtype, device=q.device)
@@ -624,7 +638,10 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     a.cache_stride_batch, a.cache_stride_token, a.cache_stride_head = k_cache.stride(0), k_cache.stride(1), k_cache.stride(2)
     a.softmax_scale = float(softmax_scale)
     a.n_splits = int(n_splits)
-    a.workspace, a.workspace_bytes = ptr(workspace), workspace.numel() * 4
     a.stream = stream_ptr()
+    if static_scratch:
+        check(_lib.load().mi_attn_decode_static(ctypes.byref(a)), "mi_attn_decode_static")
+        return out
+    a.workspace, a.workspace_bytes = ptr(workspace), workspace.numel() * 4
     check(_lib.load().mi_attn_decode(ctypes.byref(a)), "mi_attn_decode")
     return out

@@ -27,3 +27,10 @@ def pytest_collection_modifyitems(config, items):
 @pytest.fixture(scope="session")
 def golden_dir():
     return GOLDEN
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Which clause of the parity gates every checked tensor passed by (tests/parity.py)."""
+    from tests import parity
+    for line in parity.summary_lines():
+        terminalreporter.write_line(line)

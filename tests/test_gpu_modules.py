@@ -13,6 +13,9 @@ from tests.parity import check, metrics
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
+# parameter gradients and logits sum over all tokens; they are held to this fraction of the error that the reference's
+# own bf16 operation order shows against the same fp32 target (measured: 0.3 - 0.8)
+PARAM_GRAD_FLOOR_FRAC = 1.0
 
 
 def _arch(**kw):
@@ -103,7 +106,7 @@ def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
             # shift invariant): both sides hold rounding noise only, so bound its size instead of its relative error
             assert m["finite"] and m["max_abs"] <= 2.0 * f["max_abs"] + 1e-3, (k, m, f)
             continue
-        assert m["finite"] and m["mean_rel"] <= max(1e-3, 1.25 * f["mean_rel"]), (k, m, f)
+        assert m["finite"] and m["mean_rel"] <= max(1e-3, PARAM_GRAD_FLOOR_FRAC * f["mean_rel"]), (k, m, f)
 
 
 def test_layer_full_size_properties():
@@ -174,7 +177,7 @@ def test_cached_generation_matches_uncached_and_oracle(rotary):
     m, f = metrics(log_c[0], ref), metrics(ref_o, ref, torch.bfloat16)
     print(f"[parity] generate.logits: max_abs={m['max_abs']:.3e} mean_rel={m['mean_rel']:.3e} | reference bf16 order: "
           f"max_abs={f['max_abs']:.3e} mean_rel={f['mean_rel']:.3e}", flush=True)
-    assert m["mean_rel"] <= max(1e-3, 1.25 * f["mean_rel"])
+    assert m["mean_rel"] <= max(1e-3, PARAM_GRAD_FLOOR_FRAC * f["mean_rel"])
 
 
 @pytest.mark.parametrize("hidden,heads", [(384, 4), (128, 4)])
@@ -275,3 +278,64 @@ def test_layer_with_attention_dropout_train_eval_and_recompute():
         out.float().square().mean().backward()
         grads.append((xin.grad.clone(), layer.self_attention.dense.weight.grad.clone()))
     assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
+
+
+def test_inference_module_is_in_eval_mode_with_a_training_config():
+    """A config with every dropout at 0.1 (what from_checkpoint reads from a training run's config.yml): the module
+    is in eval mode from construction (inference_module.py:98), so cached, uncached and graph-captured generation
+    agree token for token."""
+    print("case inference module dropout config", flush=True)
+    cfg = _arch(attention_num_kv_heads=2, dropout_after_attention=0.1, dropout_after_mlp=0.1, dropout_attention_probs=0.1,
+                dropout_embedding=0.1)
+    model = TransformerInferenceModule(cfg, device=DEV, init_std=0.2, seed=3)
+    assert not model.training and not any(m.training for m in model.modules())
+    prompt = [5, 17, 3, 90, 41, 8, 63]
+    tok_c, _ = model.generate(6, prompt, use_cache=True)
+    tok_u, _ = model.generate(6, prompt, use_cache=False)
+    tok_g = model.generate_graph(6, prompt)
+    assert tok_c == tok_u == tok_g
+    plain = TransformerInferenceModule(_arch(attention_num_kv_heads=2), device=DEV, init_std=0.2, seed=3)
+    assert plain.generate(6, prompt)[0] == tok_c
+
+
+def test_reentrant_checkpoint_with_attention_dropout_matches_plain_training_step():
+    """Reentrant activation checkpointing runs the forward under no_grad and recomputes it with grad: in training mode
+    both passes must take the same path (same dropout mask, same GEMMs), so outputs and gradients equal those of the
+    non-checkpointed layer at the same seed."""
+    print("case reentrant checkpoint + dropout", flush=True)
+    from torch.utils.checkpoint import checkpoint
+    cfg = _arch(dropout_attention_probs=0.1, attention_num_kv_heads=2)     # whole-head rotary: the fused-rotary path
+    layer = _seeded_layer(cfg, 5)
+    layer.train()
+    b, s = 2, 96
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(b, s, cfg.hidden_size, generator=g).bfloat16().to(DEV)
+    ids = torch.ones(b, s, dtype=torch.int64)
+    cu = D.get_cumulative_seq_lengths(ids).to(DEV)
+    pos = D.get_position_ids(ids).to(DEV)
+
+    def run(t):
+        return layer(TransformerLayerIO(activations=t, position_ids=pos, cumulative_seq_lengths=cu)).activations
+
+    res = []
+    for use_ckpt in (False, True):
+        torch.manual_seed(11)
+        xin = x.clone().requires_grad_()
+        layer.zero_grad()
+        out = checkpoint(run, xin, use_reentrant=True) if use_ckpt else run(xin)
+        out.float().square().mean().backward()
+        res.append((out.detach().clone(), xin.grad.clone(), layer.self_attention.query.weight.grad.clone()))
+    assert all(torch.equal(a, c) for a, c in zip(res[0], res[1]))
+
+
+def test_position_ids_outside_the_rotary_table_raise():
+    """The reference's table gather raises on an out-of-range id (rotary.py:128-131); so does the module."""
+    cfg = _arch(attention_num_kv_heads=2, sequence_length=32)
+    layer = _seeded_layer(cfg, 1)
+    x = torch.randn(1, 16, cfg.hidden_size).bfloat16().to(DEV)
+    cu = torch.tensor([0, 16], dtype=torch.int32, device=DEV)
+    ok = torch.arange(16, device=DEV).view(1, 16)
+    with torch.no_grad():
+        layer(TransformerLayerIO(activations=x, position_ids=ok, cumulative_seq_lengths=cu))
+        with pytest.raises(IndexError, match="rotary table"):
+            layer(TransformerLayerIO(activations=x, position_ids=ok + 20, cumulative_seq_lengths=cu))

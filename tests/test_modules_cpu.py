@@ -98,6 +98,34 @@ def test_data_utils_bit_exact_against_oracle():
             assert a.dtype == o.dtype and torch.equal(a, o)
 
 
+def test_get_max_seq_length_matches_oracle():
+    cu = torch.tensor(KA.CU_WITH_RESET, dtype=torch.int32)
+    assert D.get_max_seq_length(cu) == oracle.get_max_seq_length(cu) == max(b - a for a, b in zip(KA.CU_WITH_RESET[:-1], KA.CU_WITH_RESET[1:]))
+
+
+def test_scaled_dot_product_attention_and_masked_softmax_mirror_the_reference_classes():
+    """attention.py:280-304 and masked_softmax.py:37-52: attribute names, the module tree under
+    `scaled_dot_product_attention`, NotImplementedError for a kernel this package does not provide, and the
+    assert of a fused kernel's softmax module when it is called directly."""
+    from scaling_amd.nn import MaskedSoftmax, ScaledDotProductAttention
+    hip = C.MaskedSoftmaxConfig(kernel="hip", scale=2.0, deterministic_flash_attn_bwd=True)
+    sdpa = ScaledDotProductAttention(head_dim=64, dropout_p=0.1, masked_softmax_config=hip, causal=True)
+    assert sdpa.head_dim == 64 and sdpa.dropout_p == 0.1 and sdpa.causal and not sdpa.use_matmul
+    assert sdpa.query_key_scaling_factor == 1 / 8 and sdpa.softmax_scale == 0.25 and sdpa.masked_softmax_config is hip
+    assert isinstance(sdpa.softmax_fn, MaskedSoftmax) and isinstance(sdpa.dropout_fn, torch.nn.Dropout)
+    assert sdpa.softmax_fn.kernel is None and sdpa.softmax_fn.config is hip
+    with pytest.raises(AssertionError):
+        sdpa.softmax_fn(torch.zeros(1, 1, 2, 2), torch.zeros(1, 1, 2, 2, dtype=torch.bool))
+    for kernel in ("torch", "flash_attention"):
+        with pytest.raises(NotImplementedError, match="not implemented"):
+            MaskedSoftmax(C.MaskedSoftmaxConfig(kernel=kernel))
+    att = ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, rotary_config=C.RotaryConfig(dimensions=64))
+    names = dict(att.named_modules())
+    assert "scaled_dot_product_attention" in names and "scaled_dot_product_attention.softmax_fn" in names
+    assert att.softmax_scale == sdpa.softmax_scale
+    assert not any(k.startswith("scaled_dot_product_attention") for k in att.state_dict())   # no parameters: checkpoints unchanged
+
+
 # ---- module / checkpoint contract ---------------------------------------------------------------------------
 def test_layer_parameter_names_match_reference_checkpoint(golden_dir):
     legacy = torch.load(os.path.join(golden_dir, "legacy_layer_state.pt"), weights_only=True)
