@@ -154,6 +154,7 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
 
     res = {"pairs_per_head": pairs}
     res["ms_step"] = time_gpu(step, steps, warmup)
+    res["ms_step_graph"] = time_gpu_graph(step, steps, warmup)
     res["ms_fwd"] = time_gpu(fwd, steps, warmup)
     res["ms_bwd_delta"] = time_gpu(lambda: bwd(16), steps, 1)
     res["ms_bwd_dkdv"] = time_gpu(lambda: bwd(32), steps, 1)
@@ -177,6 +178,7 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
     flops_unit = d * nq * pairs
     res["tflops_fwd"] = 4 * flops_unit / (res["ms_fwd"] * 1e-3) / 1e12
     res["tflops_step"] = 14 * flops_unit / (res["ms_step"] * 1e-3) / 1e12
+    res["tflops_step_graph"] = 14 * flops_unit / (res["ms_step_graph"] * 1e-3) / 1e12
     res["frac_of_bf16_peak_step"] = res["tflops_step"] / PEAK_BF16_TFLOPS
     return res
 
@@ -425,7 +427,7 @@ def main():
     dom_ms, dom_mult = kernels[dom]
     achieved = dom_mult * flops_unit / (dom_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_KIB[dom] * 1024.0, "traffic_unit": "bytes per launch",
+                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
                 "avg_launch_ms": dom_ms}
 
     extra = {"headline": main_res}

@@ -495,7 +495,8 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
 
 def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None,
                        flags=0, buffers=None, dropout=None):
-    """Returns (dq, dk, dv) for already rotated q/k.
+    """Returns (dq, dk, dv) for already rotated q/k.  The summation order is fixed: results are bit-reproducible
+    (what masked_softmax.deterministic_flash_attn_bwd asks of the reference's fused kernel holds always).
 
     flags: 0 runs the whole backward; 16 / 32 / 64 run only the delta / dK-dV / dQ kernel (timing aid).
     buffers: optional (dq, dk, dv, workspace) to reuse across calls."""
@@ -566,7 +567,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
 
     rotary = (cos, sin, position_ids_q, position_ids_k) applies the rotary embedding of the whole head to q and k
     (attention.py:836-845; table formats as for attention_forward) and differentiates through it.
-    deterministic mirrors masked_softmax.deterministic_flash_attn_bwd of the reference.
+    deterministic mirrors masked_softmax.deterministic_flash_attn_bwd of the reference; the kernels sum in a fixed
+    order whatever its value.
     """
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])

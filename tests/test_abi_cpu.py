@@ -83,6 +83,8 @@ def test_null_and_shape_errors_are_status_codes(lib):
     # 8 or more KV heads: nothing to split; one KV head: room for 8 fp32 partial dK and dV next to delta
     assert lib.mi_attn_bwd_workspace_bytes_kv(8192, 8192, 32, 8, 128) == 8192 * 32 * 4
     assert lib.mi_attn_bwd_workspace_bytes_kv(8192, 4096, 32, 1, 128) == 8192 * 32 * 4 + 2 * 8 * 4096 * 128 * 4
+    assert lib.mi_attn_decode_static_scratch_bytes() == 8 << 20
+    assert lib.mi_attn_decode_static(None) == -1
     assert lib.mi_rmsnorm_bwd_workspace_bytes(8192, 4096) >= 4096 * 4
     assert lib.mi_attn_decode_workspace_bytes(32, 32, 128, 4352) > 0
 
