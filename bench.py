@@ -161,17 +161,15 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
     res["ms_bwd_dq"] = time_gpu(lambda: bwd(64), steps, 1)
     if rot is not None:
         res["ms_fwd_fused_rotary"] = time_gpu(fwd_rot, steps, warmup)
-        # training step with the rotary embedding: rotate q and k (one launch each), attention forward and
-        # backward on the rotated tensors, inverse rotation of dq and dk (the rotary backward)
+        # training step with the rotary embedding as ops.attention runs it: k rotated by one stand-alone launch, q
+        # while the forward kernel loads it (the rotated q is written out for the backward), dq and dk rotated back
+        # inside the backward kernels
         cos_t, sin_t, pos_t, _ = rot
 
         def step_rotary():
-            qr = ops._rotary_launch(q, cos_t, sin_t, pos_t, 0, False)
             kr = ops._rotary_launch(k, cos_t, sin_t, pos_t, 0, False)
-            o2, lse2 = ops.attention_forward(qr, kr, v, cu, None, True, scale)
-            ops.attention_backward(do, qr, kr, v, o2, lse2, cu, None, True, scale, buffers=bufs)
-            ops._rotary_launch(dq, cos_t, sin_t, pos_t, 0, True, out=dq)
-            ops._rotary_launch(dk, cos_t, sin_t, pos_t, 0, True, out=dk)
+            o2, lse2, qr = ops.attention_forward(q, kr, v, cu, None, True, scale, rotary=(cos_t, sin_t, pos_t, None), return_rotated_q=True)
+            ops.attention_backward(do, qr, kr, v, o2, lse2, cu, None, True, scale, buffers=bufs, rotary=rot)
 
         res["ms_step_with_rotary"] = time_gpu(step_rotary, steps, warmup)
         res["tflops_step_with_rotary"] = 14 * d * nq * pairs / (res["ms_step_with_rotary"] * 1e-3) / 1e12

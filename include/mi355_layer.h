@@ -177,7 +177,10 @@ int mi_rotary_complex(const void* x, void* out, const float* cos, const float* s
  *
  * Fused rotary (optional): if rotary_cos != NULL, q and k are rotated on load (rotate-half, the
  * whole head_dim; tables [rotary_table_rows, head_dim] in the I/O dtype; position ids int64 per
- * token, required).  With rotary_interleaved != 0 the rotation is the interleaved-pair ("complex")
+ * token).  position_ids_k == NULL means that k is rotated already and only q is rotated here: the cheaper
+ * arrangement whenever k can be rotated once beforehand (mi_rotary), because a K tile is loaded by every query
+ * block of every query head of its group and a Q row only once; it is also the only one that combines with
+ * dropout.  q_rot_out receives the rotated q for the backward.  With rotary_interleaved != 0 the rotation is the interleaved-pair ("complex")
  * one of core/nn/rotary.py:59-90 instead: pairs (2i, 2i+1), fp32 tables [rotary_table_rows,
  * head_dim / 2] (real and imaginary part of freqs_cis), fp32 arithmetic, one rounding -- the same
  * bits as mi_rotary_complex followed by the plain call.  Supported: dtype MI_BF16, head_dim in {64, 128}.
@@ -225,17 +228,21 @@ typedef struct mi_attn_args {
      *                  >> (16 * (query & 1) + 8 * (key & 1))) < T,  T = round(256 * dropout_p) clamped to 1..255,
      * head_base = lowbias32(seed32 ^ lowbias32(head * 0x9E3779B9 + 0x7F4A7C15)), seed32 = low ^ high word of
      * dropout_seed; query / key are token indices on the flattened axes.  The effective drop probability is
-     * T / 256 and kept probabilities are scaled by 256 / (256 - T).  The backward call must pass the same values.
-     * Not available together with the fused rotary of the forward. */
+     * T / 256 and kept probabilities are scaled by 256 / (256 - T).  The backward call must pass the same values. */
     float dropout_p;
     uint64_t dropout_seed;
     int32_t rotary_interleaved;    /* fused rotary: 0 = rotate-half, 1 = interleaved pairs with fp32 tables */
+    void* q_rot_out;               /* forward with fused rotary: optional copy of the rotated q (strides of q), what
+                                      mi_attn_bwd takes as q; NULL = not stored */
 } mi_attn_args;
 
 int mi_attn_fwd(const mi_attn_args* args);
 
 /* Backward of mi_attn_fwd.  Extra inputs: o and lse from the forward, d_o (layout/strides of o).
- * Outputs dq (strides of q), dk, dv (strides given).  GQA: dk/dv are summed over the query heads of
+ * Outputs dq (strides of q), dk, dv (strides given).  With rotary (fwd.rotary_cos != NULL; both position id arrays
+ * required): fwd.q and fwd.k are the ROTATED tensors the forward attended with (its q_rot_out, and the rotated k), and
+ * dq / dk are the gradients of the unrotated ones: each row is rotated back (by minus its position's angles, what
+ * autograd derives from core/nn/rotary.py:117-139 / :59-90) in fp32 before its single rounding.  GQA: dk/dv are summed over the query heads of
  * each group inside the kernel, in a fixed order (no atomics; bit-reproducible).
  * workspace: fp32 scratch of mi_attn_bwd_workspace_bytes() bytes (row sums of d_o * o). */
 typedef struct mi_attn_bwd_args {

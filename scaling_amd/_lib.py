@@ -43,6 +43,7 @@ class MiAttnArgs(Structure):
         ("rotary_table_rows", c_int64),
         ("stream", c_void_p),
         ("dropout_p", c_float), ("dropout_seed", c_uint64), ("rotary_interleaved", c_int32),
+        ("q_rot_out", c_void_p),
     ]
 
 

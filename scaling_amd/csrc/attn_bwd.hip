@@ -308,14 +308,21 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                 *reinterpret_cast<f32x4_t*>(p.dv_part + prow + 32 * dt + 8 * a) = v4;
             }
     } else if (sub == 0 && key < p.total_k) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dk_acc[dt][r] *= p.scale;
+        if constexpr (D == 64 || D == 128) {
+            if (p.unrotate != 0) unrotate_acc<D>(dk_acc, p, p.pos_k[key], g);   // k was the rotated tensor
+        }
         __bf16* dkr = p.dk + (int64_t)key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * g;
         __bf16* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const uint32_t k0 = pack_bf16x2(dk_acc[dt][4 * a] * p.scale, dk_acc[dt][4 * a + 1] * p.scale);
-                const uint32_t k1 = pack_bf16x2(dk_acc[dt][4 * a + 2] * p.scale, dk_acc[dt][4 * a + 3] * p.scale);
+                const uint32_t k0 = pack_bf16x2(dk_acc[dt][4 * a], dk_acc[dt][4 * a + 1]);
+                const uint32_t k1 = pack_bf16x2(dk_acc[dt][4 * a + 2], dk_acc[dt][4 * a + 3]);
                 *reinterpret_cast<uint2*>(dkr + 32 * dt + 8 * a) = make_uint2(k0, k1);
                 const float vs = DROP ? p.drop_rscale : 1.0f;   // dV = (P * mask / (1 - p))^T dO
                 const uint32_t v0 = pack_bf16x2(dv_acc[dt][4 * a] * vs, dv_acc[dt][4 * a + 1] * vs);
@@ -325,27 +332,61 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     }
 }
 
-// Sum of the hsplit partial dK / dV of a split launch, in a fixed order; one thread per (key, KV head, 4 features).
+// Sum of the hsplit partial dK / dV of a split launch, in a fixed order; one thread per (key, KV head) and two groups
+// of 4 features, D / 2 apart (the two halves of rotate-half pairs), so that the summed dK can be rotated back in place.
 template <int D>
 __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_reduce_kernel(const AttnParams p) {
     const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    const int64_t n = (int64_t)p.total_k * p.nkv * (D / 4);
+    const int64_t n = (int64_t)p.total_k * p.nkv * (D / 8);
     if (idx >= n) return;
-    const int c = (int)(idx % (D / 4));
-    const int kvh = (int)((idx / (D / 4)) % p.nkv);
-    const int64_t key = idx / ((int64_t)(D / 4) * p.nkv);
+    const int c = (int)(idx % (D / 8));
+    const int kvh = (int)((idx / (D / 8)) % p.nkv);
+    const int64_t key = idx / ((int64_t)(D / 8) * p.nkv);
     const int64_t stride = (int64_t)p.total_k * p.nkv * D;
     const int64_t off = (key * p.nkv + kvh) * D + 4 * c;
-    f32x4_t k4 = *reinterpret_cast<const f32x4_t*>(p.dk_part + off);
-    f32x4_t v4 = *reinterpret_cast<const f32x4_t*>(p.dv_part + off);
-    for (int s = 1; s < p.hsplit; ++s) {
-        k4 += *reinterpret_cast<const f32x4_t*>(p.dk_part + s * stride + off);
-        v4 += *reinterpret_cast<const f32x4_t*>(p.dv_part + s * stride + off);
+    f32x4_t k4[2], v4[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        k4[h] = *reinterpret_cast<const f32x4_t*>(p.dk_part + off + h * (D / 2));
+        v4[h] = *reinterpret_cast<const f32x4_t*>(p.dv_part + off + h * (D / 2));
     }
-    *reinterpret_cast<uint2*>(p.dk + key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * c) =
-        make_uint2(pack_bf16x2(k4[0], k4[1]), pack_bf16x2(k4[2], k4[3]));
-    *reinterpret_cast<uint2*>(p.dv + key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * c) =
-        make_uint2(pack_bf16x2(v4[0], v4[1]), pack_bf16x2(v4[2], v4[3]));
+    for (int s = 1; s < p.hsplit; ++s)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            k4[h] += *reinterpret_cast<const f32x4_t*>(p.dk_part + s * stride + off + h * (D / 2));
+            v4[h] += *reinterpret_cast<const f32x4_t*>(p.dv_part + s * stride + off + h * (D / 2));
+        }
+    if (p.unrotate != 0) {
+        int64_t pos = p.pos_k[key];
+        pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+        if (p.unrotate == 1) {               // features 4 c + i pair with 4 c + i + D / 2
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float cs = (float)p.cos[pos * D + 4 * c + i], sn = (float)p.sin[pos * D + 4 * c + i];
+                const float x0 = k4[0][i], x1 = k4[1][i];
+                k4[0][i] = x0 * cs + x1 * sn;
+                k4[1][i] = x1 * cs - x0 * sn;
+            }
+        } else {                             // pairs (4 c, 4 c + 1), (4 c + 2, 4 c + 3) of either half
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int pair = (4 * c + h * (D / 2)) / 2 + i;
+                    float x0 = k4[h][2 * i], x1 = k4[h][2 * i + 1];
+                    rotate_complex_pair(x0, x1, p.cos32[pos * (D / 2) + pair], -p.sin32[pos * (D / 2) + pair]);
+                    k4[h][2 * i] = x0;
+                    k4[h][2 * i + 1] = x1;
+                }
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        *reinterpret_cast<uint2*>(p.dk + key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * c + h * (D / 2)) =
+            make_uint2(pack_bf16x2(k4[h][0], k4[h][1]), pack_bf16x2(k4[h][2], k4[h][3]));
+        *reinterpret_cast<uint2*>(p.dv + key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * c + h * (D / 2)) =
+            make_uint2(pack_bf16x2(v4[h][0], v4[h][1]), pack_bf16x2(v4[h][2], v4[h][3]));
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -523,13 +564,21 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     }
 
     if (tq < p.total_q) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dq_acc[dt][r] *= p.scale;
+        if constexpr (D == 64 || D == 128) {
+            // q was the rotated tensor: the gradient of the unrotated one is the row rotated back (rotary.py:117-139)
+            if (p.unrotate != 0) unrotate_acc<D>(dq_acc, p, p.pos_q[tq], g);
+        }
         __bf16* dqr = p.dq + (int64_t)tq * p.q_st + (int64_t)head * p.q_sh + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const uint32_t w0 = pack_bf16x2(dq_acc[dt][4 * a] * p.scale, dq_acc[dt][4 * a + 1] * p.scale);
-                const uint32_t w1 = pack_bf16x2(dq_acc[dt][4 * a + 2] * p.scale, dq_acc[dt][4 * a + 3] * p.scale);
+                const uint32_t w0 = pack_bf16x2(dq_acc[dt][4 * a], dq_acc[dt][4 * a + 1]);
+                const uint32_t w1 = pack_bf16x2(dq_acc[dt][4 * a + 2], dq_acc[dt][4 * a + 3]);
                 *reinterpret_cast<uint2*>(dqr + 32 * dt + 8 * a) = make_uint2(w0, w1);
             }
     }
@@ -553,7 +602,7 @@ template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) 
         int rc = mi_check_launch("attn_bwd_dkdv");
         if (rc != MI_OK) return rc;
         if (p.hsplit > 1) {
-            const int64_t n = (int64_t)p.total_k * p.nkv * (D / 4);
+            const int64_t n = (int64_t)p.total_k * p.nkv * (D / 8);
             attn_bwd_dkdv_reduce_kernel<D><<<dim3((unsigned)((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, st>>>(p);
             rc = mi_check_launch("attn_bwd_dkdv_reduce");
             if (rc != MI_OK) return rc;
@@ -604,7 +653,7 @@ extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
     const mi_attn_args* a = &b->fwd;
     int rc = mi_attn_validate(a, "attn_bwd");
     if (rc != MI_OK) return rc;
-    if (a->rotary_cos) return mi_fail(MI_E_SHAPE, "attn_bwd: takes already rotated q/k (rotary is not fused into the backward)");
+    if (a->rotary_cos && !a->position_ids_k) return mi_fail(MI_E_NULL, "attn_bwd: rotary needs the position ids of q and k");
     if (!a->o || !a->lse || !b->d_o || !b->dq || !b->dk || !b->dv)
         return mi_fail(MI_E_NULL, "attn_bwd: o, lse, d_o, dq, dk, dv are required");
     if (!mi_aligned16(a->o) || !mi_aligned16(b->d_o) || !mi_aligned16(b->dq) || !mi_aligned16(b->dk) || !mi_aligned16(b->dv))
@@ -622,6 +671,7 @@ extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
     p.dk_st = b->dk_stride_token; p.dk_sh = b->dk_stride_head;
     p.dv_st = b->dv_stride_token; p.dv_sh = b->dv_stride_head;
     p.delta = (float*)b->workspace;
+    p.unrotate = a->rotary_cos == nullptr ? 0 : (a->rotary_interleaved ? 2 : 1);
     p.hsplit = 1;
     {   // fewer than 8 KV heads: split the query heads of a group over workgroups if the workspace has room for the partials
         const int h = dkdv_head_split(a->n_q_heads, a->n_kv_heads);

@@ -36,6 +36,11 @@ struct AttnParams {
     // dK/dV with fewer than 8 KV heads: the query heads of a group are split over hsplit workgroups per key block,
     // each writing fp32 partial sums [hsplit][total_k][nkv][head_dim] that a reduce launch adds up (1 = no split)
     int hsplit; float* dk_part; float* dv_part;
+    // forward: optional copy of the rotated q (fused rotary), same strides as q
+    __bf16* q_rot;
+    // backward with rotary: q / k are the rotated tensors; dq / dk leave the kernels rotated back (0 = no rotary,
+    // 1 = rotate-half with tables in the I/O dtype, 2 = interleaved pairs with fp32 tables)
+    int unrotate;
 };
 
 // ---- dropout mask ---------------------------------------------------------------------------------------
@@ -314,6 +319,50 @@ __device__ __forceinline__ void rotate_interleaved(uint4& v, const uint4& c, con
         float x0 = bf16_lo(w[i]), x1 = bf16_hi(w[i]);
         rotate_complex_pair(x0, x1, __uint_as_float(cw[i]), sign * __uint_as_float(sw[i]));
         w[i] = pack_bf16x2(x0, x1);
+    }
+}
+
+// Inverse rotary (rotation by minus the position's angles) of one token's gradient row held in accumulator layout:
+// acc[dt][4 a + c] is feature 32 dt + 8 a + 4 g + c of the lane's token.  Rotate-half pairs feature f with f + D / 2
+// (accumulators dt and dt + D / 64, same register), the interleaved form pairs registers (4 a, 4 a + 1) and
+// (4 a + 2, 4 a + 3).  fp32 throughout; the caller rounds once afterwards.
+template <int D>
+__device__ __forceinline__ void unrotate_acc(f32x16_t (&acc)[D / 32], const AttnParams& p, int64_t pos, int g) {
+    static_assert(D == 64 || D == 128, "fused rotary covers head_dim 64 and 128");
+    constexpr int DT = D / 32;
+    pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+    if (p.unrotate == 1) {
+        const __bf16* cr = p.cos + pos * D + 4 * g;
+        const __bf16* sr = p.sin + pos * D + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT / 2; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const uint2 cw = *reinterpret_cast<const uint2*>(cr + 32 * dt + 8 * a);
+                const uint2 sw = *reinterpret_cast<const uint2*>(sr + 32 * dt + 8 * a);
+                const float c4[4] = {bf16_lo(cw.x), bf16_hi(cw.x), bf16_lo(cw.y), bf16_hi(cw.y)};
+                const float s4[4] = {bf16_lo(sw.x), bf16_hi(sw.x), bf16_lo(sw.y), bf16_hi(sw.y)};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float x0 = acc[dt][4 * a + c], x1 = acc[dt + DT / 2][4 * a + c];
+                    acc[dt][4 * a + c] = x0 * c4[c] + x1 * s4[c];
+                    acc[dt + DT / 2][4 * a + c] = x1 * c4[c] - x0 * s4[c];
+                }
+            }
+    } else {
+        const float* cr = p.cos32 + pos * (D / 2) + 2 * g;
+        const float* sr = p.sin32 + pos * (D / 2) + 2 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const float2 c2 = *reinterpret_cast<const float2*>(cr + 16 * dt + 4 * a);
+                const float2 s2 = *reinterpret_cast<const float2*>(sr + 16 * dt + 4 * a);
+                float x0 = acc[dt][4 * a], x1 = acc[dt][4 * a + 1], y0 = acc[dt][4 * a + 2], y1 = acc[dt][4 * a + 3];
+                rotate_complex_pair(x0, x1, c2.x, -s2.x);
+                rotate_complex_pair(y0, y1, c2.y, -s2.y);
+                acc[dt][4 * a] = x0; acc[dt][4 * a + 1] = x1; acc[dt][4 * a + 2] = y0; acc[dt][4 * a + 3] = y1;
+            }
     }
 }
 

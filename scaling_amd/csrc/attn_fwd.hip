@@ -24,10 +24,15 @@ namespace {
 constexpr int BN = 64;               // keys per tile
 constexpr float kRescaleGap = 8.0f;  // log2 units by which a row max may lag before O is rescaled
 
-// ROT: 0 = q / k are used as they are, 1 = rotate-half rotary applied on load (tables in the I/O dtype),
-// 2 = interleaved-pair rotary applied on load (fp32 tables)
-template <int D, int NW, int ROT, bool DROP>
+// ROTM: 0 = q / k are used as they are; 1 = rotate-half rotary applied to q and k on load (tables in the I/O dtype),
+// 2 = interleaved-pair rotary applied to q and k on load (fp32 tables); 3 / 4 = the same two rotations applied to q
+// only (k arrives rotated: the training path rotates it once with the stand-alone kernel, because every K tile is
+// loaded by each query block of each head of its group and would be rotated a few hundred times over in here, whereas
+// a Q row is loaded exactly once).  With p.q_rot the rotated q is also written out (the backward kernels stream it).
+template <int D, int NW, int ROTM, bool DROP>
 __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p) {
+    constexpr int ROT = (ROTM == 1 || ROTM == 2) ? ROTM : 0;        // rotation of K inside the tile loaders
+    constexpr int QROT = ROTM == 0 ? 0 : ((ROTM & 1) ? 1 : 2);      // rotation of the Q fragment
     constexpr int BM = 32 * NW;
     constexpr int KS = D / 16;            // contraction steps of Q K^T
     constexpr int DT = D / 32;            // 32-row tiles of O^T
@@ -67,7 +72,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qrow + 16 * ks);
-        if constexpr (ROT == 1) {
+        if constexpr (QROT == 1) {
             int64_t pos = p.pos_q[tl];
             pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
             const __bf16* cr = p.cos + pos * D + 8 * g;
@@ -78,7 +83,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 const uint4 s = *reinterpret_cast<const uint4*>(sr + 16 * ks);
                 rotate_pair(raw[ks], raw[ks + KS / 2], c, s, 1.0f);
             }
-        } else if constexpr (ROT == 2) {
+        } else if constexpr (QROT == 2) {
             int64_t pos = p.pos_q[tl];
             pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
             const float* cr = p.cos32 + pos * (D / 2) + 4 * g;   // features 16 ks + 8 g .. + 8 = pairs 8 ks + 4 g .. + 4
@@ -89,6 +94,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
+        if constexpr (QROT != 0) {
+            if (p.q_rot != nullptr && tq < p.total_q) {
+                __bf16* qo = p.q_rot + (int64_t)tq * p.q_st + (int64_t)head * p.q_sh + 8 * g;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) st128(qo + 16 * ks, raw[ks]);
+            }
+        }
     }
     // Consume the Q registers here: otherwise their loads count as possibly outstanding at the loop
     // entry, and every use inside the loop waits for the K/V prefetch issued just before it.
@@ -419,20 +431,25 @@ template <int D, int NW, int ROT, bool DROP> int launch(const AttnParams& p, hip
     return mi_check_launch("attn_fwd");
 }
 
-// rot: 0 = none, 1 = rotate-half, 2 = interleaved pairs
-template <int D> int launch_d(const AttnParams& p, int rot, int nw, hipStream_t st) {
-    if (p.drop_thr != 0) {               // dropout: one tiling per head_dim (256-query workgroups), no fused rotary
-        if (rot) return mi_fail(MI_E_SHAPE, "attn_fwd: dropout and fused rotary cannot be combined");
-        return launch<D, 8, 0, true>(p, st);
-    }
+// rot: 0 = none, 1 = rotate-half, 2 = interleaved pairs; q_only: k arrives rotated
+template <int D> int launch_d(const AttnParams& p, int rot, bool q_only, int nw, hipStream_t st) {
     if (rot) {
         if constexpr (D == 64 || D == 128) {
+            if (p.drop_thr != 0) {           // dropout: one tiling per head_dim (256-query workgroups), rotary on q only
+                if (!q_only) return mi_fail(MI_E_SHAPE, "attn_fwd: with dropout the fused rotary covers q only (pass rotated k and position_ids_k = NULL)");
+                return rot == 2 ? launch<D, 8, 4, true>(p, st) : launch<D, 8, 3, true>(p, st);
+            }
+            if (q_only) {
+                if (rot == 2) return nw == 8 ? launch<D, 8, 4, false>(p, st) : launch<D, 4, 4, false>(p, st);
+                return nw == 8 ? launch<D, 8, 3, false>(p, st) : launch<D, 4, 3, false>(p, st);
+            }
             if (rot == 2) return nw == 8 ? launch<D, 8, 2, false>(p, st) : launch<D, 4, 2, false>(p, st);
             return nw == 8 ? launch<D, 8, 1, false>(p, st) : launch<D, 4, 1, false>(p, st);
         } else {
             return mi_fail(MI_E_SHAPE, "attn_fwd: fused rotary needs head_dim 64 or 128");
         }
     }
+    if (p.drop_thr != 0) return launch<D, 8, 0, true>(p, st);
     return nw == 8 ? launch<D, 8, 0, false>(p, st) : launch<D, 4, 0, false>(p, st);
 }
 
@@ -451,6 +468,12 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     AttnParams p;
     mi_attn_fill_params(a, &p);
     const int rot = a->rotary_cos == nullptr ? 0 : (a->rotary_interleaved ? 2 : 1);
+    const bool q_only = a->position_ids_k == nullptr;
+    if (a->q_rot_out) {
+        if (!rot) return mi_fail(MI_E_NULL, "attn_fwd: q_rot_out needs the fused rotary");
+        if (!mi_aligned16(a->q_rot_out)) return mi_fail(MI_E_ALIGN, "attn_fwd: q_rot_out must be 16-byte aligned");
+        p.q_rot = (__bf16*)a->q_rot_out;
+    }
     // 256-query workgroups (two groups of wavefronts a phase apart) beat 128-query ones at every size measured,
     // also when they leave most compute units without work (1 x 512 tokens x 32 heads: 22 against 25 us,
     // 1 x 2048: 65 against 93 us); the smaller tiling only serves inputs that do not fill one workgroup
@@ -460,10 +483,10 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     if (p.n_rep == 1) p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 32 * nw);
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
-        case 32: return launch_d<32>(p, rot, nw, st);
-        case 64: return launch_d<64>(p, rot, nw, st);
-        case 96: return launch_d<96>(p, rot, nw, st);
-        case 128: return launch_d<128>(p, rot, nw, st);
+        case 32: return launch_d<32>(p, rot, q_only, nw, st);
+        case 64: return launch_d<64>(p, rot, q_only, nw, st);
+        case 96: return launch_d<96>(p, rot, q_only, nw, st);
+        case 128: return launch_d<128>(p, rot, q_only, nw, st);
         default: return mi_fail(MI_E_SHAPE, "attn_fwd: head_dim %d unsupported (32, 64, 96, 128)", a->head_dim);
     }
 }

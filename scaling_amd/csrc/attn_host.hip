@@ -20,14 +20,13 @@ int mi_attn_validate(const mi_attn_args* a, const char* who) {
         return mi_fail(MI_E_ALIGN, "%s: strides must be multiples of 8 elements", who);
     if (!(a->softmax_scale > 0.f)) return mi_fail(MI_E_SHAPE, "%s: softmax_scale must be positive", who);
     if (a->rotary_cos || a->rotary_sin) {
-        if (!a->rotary_cos || !a->rotary_sin || !a->position_ids_q || !a->position_ids_k)
-            return mi_fail(MI_E_NULL, "%s: fused rotary needs cos, sin and both position id arrays", who);
+        if (!a->rotary_cos || !a->rotary_sin || !a->position_ids_q)
+            return mi_fail(MI_E_NULL, "%s: fused rotary needs cos, sin and the query position ids", who);
         if (a->head_dim != 64 && a->head_dim != 128) return mi_fail(MI_E_SHAPE, "%s: fused rotary needs head_dim 64 or 128", who);
         if (a->rotary_table_rows <= 0 || a->rotary_table_rows > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "%s: bad rotary table size", who);
         if (!mi_aligned16(a->rotary_cos) || !mi_aligned16(a->rotary_sin)) return mi_fail(MI_E_ALIGN, "%s: rotary tables must be 16-byte aligned", who);
     }
     if (!(a->dropout_p >= 0.f) || a->dropout_p >= 1.f) return mi_fail(MI_E_SHAPE, "%s: dropout_p must be in [0, 1)", who);
-    if (a->dropout_p > 0.f && a->rotary_cos) return mi_fail(MI_E_SHAPE, "%s: dropout and fused rotary cannot be combined", who);
     return MI_OK;
 }
 

@@ -431,7 +431,7 @@ def _fused_rotary_kind(cos: torch.Tensor, sin: torch.Tensor, head_dim: int, dtyp
     return False
 
 
-def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, flags=0, dropout=None) -> MiAttnArgs:
+def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, flags=0, dropout=None, q_rot=None) -> MiAttnArgs:
     a = MiAttnArgs()
     a.flags = int(flags)
     a.q, a.k, a.v, a.o, a.lse = ptr(q), ptr(k), ptr(v), ptr(o), ptr(lse)
@@ -452,6 +452,7 @@ def _fill_attn_args(q, k, v, o, lse, cu_q, cu_k, causal, scale, rotary=None, fla
         a.position_ids_q, a.position_ids_k = ptr(pos_q), ptr(pos_k)
         a.rotary_table_rows = cos.shape[0]
         a.rotary_interleaved = int(_fused_rotary_kind(cos, sin, q.shape[2], q.dtype))
+        a.q_rot_out = ptr(q_rot)
     if dropout is not None and dropout[0] > 0.0:
         a.dropout_p, a.dropout_seed = float(dropout[0]), int(dropout[1]) & 0xFFFFFFFFFFFFFFFF
     a.stream = stream_ptr()
@@ -469,11 +470,13 @@ def _check_qkv(q, k, v, cu_q, cu_k):
 
 
 def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None, rotary=None, flags=0,
-                      dropout=None):
-    """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens]).
+                      dropout=None, return_rotated_q=False):
+    """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens]) (+ the rotated q if asked).
 
     rotary: optional (cos, sin, position_ids_q, position_ids_k), q and k are rotated while they are loaded:
     rotate-half with [rows, head_dim] tables in q's dtype, interleaved pairs with fp32 [rows, head_dim / 2] tables.
+    position_ids_k = None: k is rotated already, only q is rotated in the kernel (the cheaper arrangement, see
+    include/mi355_layer.h); return_rotated_q then also returns the rotated q (strides of q) for the backward.
 
     dropout: optional (p, seed) for dropout on the attention probabilities; the backward needs the same pair.
 
@@ -481,22 +484,30 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
+    q_rot = None
     if rotary is not None:
         cos, sin, pos_q, pos_k = rotary
         _fused_rotary_kind(cos, sin, q.shape[2], q.dtype)
         assert pos_q.dtype == torch.int64 and pos_q.is_contiguous() and pos_q.numel() == q.shape[0]
-        assert pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0]
+        assert pos_k is None or (pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0])
+        if return_rotated_q:
+            q_rot = torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
+    else:
+        assert not return_rotated_q
     o = torch.empty((q.shape[0], q.shape[1], q.shape[2]), dtype=q.dtype, device=q.device)
     lse = torch.empty((q.shape[1], q.shape[0]), dtype=torch.float32, device=q.device)
-    a = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary, flags, dropout)
+    a = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary, flags, dropout, q_rot)
     check(_lib.load().mi_attn_fwd(ctypes.byref(a)), "mi_attn_fwd")
-    return o, lse
+    return (o, lse, q_rot) if return_rotated_q else (o, lse)
 
 
 def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None,
-                       flags=0, buffers=None, dropout=None):
-    """Returns (dq, dk, dv) for already rotated q/k.  The summation order is fixed: results are bit-reproducible
+                       flags=0, buffers=None, dropout=None, rotary=None):
+    """Returns (dq, dk, dv).  The summation order is fixed: results are bit-reproducible
     (what masked_softmax.deterministic_flash_attn_bwd asks of the reference's fused kernel holds always).
+
+    rotary = (cos, sin, position_ids_q, position_ids_k): q and k are the ROTATED tensors the forward attended with, and
+    dq / dk come back as gradients of the unrotated ones (rotated back inside the kernels, one rounding).
 
     flags: 0 runs the whole backward; 16 / 32 / 64 run only the delta / dK-dV / dQ kernel (timing aid).
     buffers: optional (dq, dk, dv, workspace) to reuse across calls."""
@@ -519,7 +530,7 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
         nbytes = lib.mi_attn_bwd_workspace_bytes_kv(q.shape[0], k.shape[0], q.shape[1], k.shape[1], q.shape[2])
         ws = torch.empty(max(nbytes // 4, 4), dtype=torch.float32, device=q.device)
     b = MiAttnBwdArgs()
-    b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, None, flags, dropout)
+    b.fwd = _fill_attn_args(q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary, flags, dropout)
     b.d_o, b.dq, b.dk, b.dv = ptr(do), ptr(dq), ptr(dk), ptr(dv)
     b.dk_stride_token, b.dk_stride_head = dk.stride(0), dk.stride(1)
     b.dv_stride_token, b.dv_stride_head = dv.stride(0), dv.stride(1)
@@ -530,18 +541,31 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
 
 class _Attention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, cu_q, cu_k, causal, scale, dropout_p, dropout_seed):
+    def forward(ctx, q, k, v, cu_q, cu_k, causal, scale, dropout_p, dropout_seed, cos, sin, pos_q, pos_k):
         dropout = (dropout_p, dropout_seed) if dropout_p > 0.0 else None
-        o, lse = attention_forward(q, k, v, cu_q, cu_k, causal, scale, dropout=dropout)
-        ctx.save_for_backward(q, k, v, o, lse, cu_q, cu_k if cu_k is not None else cu_q)
-        ctx.causal, ctx.scale, ctx.dropout = causal, scale, dropout
+        if cos is None:
+            o, lse = attention_forward(q, k, v, cu_q, cu_k, causal, scale, dropout=dropout)
+            ctx.save_for_backward(q, k, v, o, lse, cu_q, cu_k if cu_k is not None else cu_q)
+        else:
+            # rotary: k is rotated once by the stand-alone kernel, q while the attention kernel loads it; the rotated
+            # tensors are what the backward kernels stream, so they are kept instead of q and k
+            interleaved = _fused_rotary_kind(cos, sin, q.shape[2], q.dtype)
+            k_rot = (_rotary_complex_launch if interleaved else _rotary_launch)(k, cos, sin, pos_k, 0, False)
+            if any(ctx.needs_input_grad[:3]):
+                o, lse, q_rot = attention_forward(q, k_rot, v, cu_q, cu_k, causal, scale, rotary=(cos, sin, pos_q, None),
+                                                  dropout=dropout, return_rotated_q=True)
+                ctx.save_for_backward(q_rot, k_rot, v, o, lse, cu_q, cu_k if cu_k is not None else cu_q, cos, sin, pos_q, pos_k)
+            else:   # nothing to differentiate: the rotated q is not written out
+                o, lse = attention_forward(q, k_rot, v, cu_q, cu_k, causal, scale, rotary=(cos, sin, pos_q, None), dropout=dropout)
+        ctx.causal, ctx.scale, ctx.dropout, ctx.rotary = causal, scale, dropout, cos is not None
         return o
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, o, lse, cu_q, cu_k = ctx.saved_tensors
-        dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale, dropout=ctx.dropout)
-        return dq, dk, dv, None, None, None, None, None, None
+        q, k, v, o, lse, cu_q, cu_k = ctx.saved_tensors[:7]
+        rotary = tuple(ctx.saved_tensors[7:11]) if ctx.rotary else None
+        dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale, dropout=ctx.dropout, rotary=rotary)
+        return (dq, dk, dv) + (None,) * 10
 
 
 def next_dropout_seed(device: torch.device) -> int:
@@ -566,7 +590,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
     The drop probability is quantised to round(256 p) / 256.
 
     rotary = (cos, sin, position_ids_q, position_ids_k) applies the rotary embedding of the whole head to q and k
-    (attention.py:836-845; table formats as for attention_forward) and differentiates through it.
+    (attention.py:836-845; table formats as for attention_forward) and differentiates through it: q is rotated while
+    the forward kernel loads it, k by one stand-alone launch, and the backward kernels rotate dq / dk back in their
+    epilogues, with or without autograd, with or without dropout.
     deterministic mirrors masked_softmax.deterministic_flash_attn_bwd of the reference; the kernels sum in a fixed
     order whatever its value.
     """
@@ -574,16 +600,14 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
     if dropout_p > 0.0 and dropout_seed is None:
         dropout_seed = next_dropout_seed(q.device)
+    cos = sin = pos_q = pos_k = None
     if rotary is not None:
         cos, sin, pos_q, pos_k = rotary
-        interleaved = _fused_rotary_kind(cos, sin, q.shape[2], q.dtype)
-        needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
-        if not needs_grad and dropout_p == 0.0:
-            return attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, softmax_scale, rotary=rotary)[0]
-        rot = rotary_embedding_complex if interleaved else rotary_embedding
-        q, k = rot(q, cos, sin, pos_q), rot(k, cos, sin, pos_k)
+        _fused_rotary_kind(cos, sin, q.shape[2], q.dtype)
+        assert pos_q.dtype == torch.int64 and pos_q.is_contiguous() and pos_q.numel() == q.shape[0]
+        assert pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0]
     return _Attention.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, float(softmax_scale), float(dropout_p),
-                            int(dropout_seed) if dropout_seed is not None else 0)
+                            int(dropout_seed) if dropout_seed is not None else 0, cos, sin, pos_q, pos_k)
 
 
 # ------------------------------------------------------------------------------------------------

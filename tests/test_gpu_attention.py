@@ -119,6 +119,70 @@ def test_attention_fused_rotary_matches_separate_rotary():
     assert float(diff.max()) <= 2e-2 and float((diff > 0).float().mean()) < 0.02
 
 
+def _complex_tables(d, rows, base):
+    """fp32 [rows, d / 2] real / imaginary parts of freqs_cis (core/nn/rotary.py:45-56)."""
+    inv_freq = 1.0 / (float(base) ** (torch.arange(0, d, 2)[: d // 2].float() / d))
+    ang = torch.outer(torch.arange(rows).float(), inv_freq).float()
+    return ang.cos().contiguous(), ang.sin().contiguous()
+
+
+@pytest.mark.parametrize("kind,b,s,nq,nkv,d,cuts,p_drop", [
+    ("half", 2, 192, 4, 2, 128, (50, 250), 0.0),
+    ("half", 1, 320, 8, 1, 128, (100,), 0.0),          # one KV head: dK goes through the partial-sum reduce kernel
+    ("half", 2, 96, 4, 4, 64, (), 0.0),
+    ("interleaved", 2, 160, 4, 2, 128, (70,), 0.0),
+    ("interleaved", 1, 200, 8, 2, 64, (33, 34), 0.0),  # 4-way head split
+    ("half", 1, 256, 4, 2, 128, (77,), 0.1),           # rotary together with dropout
+])
+def test_attention_with_rotary_fwd_bwd_parity(kind, b, s, nq, nkv, d, cuts, p_drop):
+    """ops.attention(rotary=...) is rotary -> attention of the reference (attention.py:836-845, 876-888): q is rotated
+    inside the forward kernel, k by the stand-alone kernel, and dq / dk are rotated back inside the backward kernels.
+    Output and the gradients of the UNROTATED q, k, v against the oracle's rotary followed by its attention."""
+    print(f"case attn rotary {kind} b={b} s={s} nq={nq} nkv={nkv} d={d} cuts={cuts} dropout={p_drop}", flush=True)
+    q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=s + d + nq)
+    cu = U.make_cu(b, s, cuts)
+    pos = U.position_ids_from_cu(cu, b * s)
+    ids = pos.view(b, s).transpose(0, 1)
+    scale, n_rep = 1 / math.sqrt(d), nq // nkv
+    seed = 1234567 + s
+    drop = None
+    if p_drop > 0:
+        keep, p_eff = U.dropout_keep_mask(seed, nq, b * s, b * s, p_drop)
+        drop = dict(dropout_p=p_eff, dropout_keep=torch.stack([keep[:, i * s:(i + 1) * s, i * s:(i + 1) * s] for i in range(b)]))
+    if kind == "half":
+        tabs = oracle.rotary_tables(d, s, 500000, torch.bfloat16)
+        dev_tabs = (tabs.cos.to(DEV), tabs.sin.to(DEV))
+    else:
+        dev_tabs = tuple(t.to(DEV) for t in _complex_tables(d, s, 10000.0))
+
+    def reference(dtype):
+        qq, kk, vv = (t.to(dtype).clone().requires_grad_() for t in (q, k, v))
+        q4, k4, v4 = U.to_sbnd(qq, b, s), U.to_sbnd(kk, b, s), U.to_sbnd(vv, b, s)
+        if kind == "half":    # table values as stored (bf16), arithmetic in `dtype`
+            q4, k4 = oracle.apply_rotary(q4, k4, oracle.RotaryTables(tabs.cos.to(dtype), tabs.sin.to(dtype), d), ids, ids)
+        else:
+            q4, k4 = oracle.apply_rotary_complex(q4, k4, d, s, 10000.0, ids, ids)
+        out = oracle.multi_head_attention(q4, oracle.repeat_kv(k4, n_rep), oracle.repeat_kv(v4, n_rep), cu, True, scale,
+                                          softmax_in_fp32=True, **(drop or {}))
+        o = U.from_bn_s_d(out, b, nq)
+        o.backward(do.to(dtype))
+        return o.detach(), qq.grad, kk.grad, vv.grad
+
+    ref, ref_o = reference(torch.float32), reference(torch.bfloat16)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    posd = pos.to(DEV)
+    o = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale, rotary=(*dev_tabs, posd, posd), dropout_p=p_drop, dropout_seed=seed)
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    for name, got, r, ro in (("o", o, ref[0], ref_o[0]), ("dq", qg.grad, ref[1], ref_o[1]),
+                             ("dk", kg.grad, ref[2], ref_o[2]), ("dv", vg.grad, ref[3], ref_o[3])):
+        check(f"attn.rotary[{kind}].{name}", got, r, ro)
+    # without autograd the same kernels run (minus the copy of the rotated q): same output bits
+    with torch.no_grad():
+        o2 = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale, rotary=(*dev_tabs, posd, posd), dropout_p=p_drop, dropout_seed=seed)
+    assert torch.equal(o2, o.detach())
+
+
 def _cross_length_reference(q, k, v, do, cu_q, cu_k, causal, scale, dtype=torch.float32):
     """Brute force from the mask predicate of the C header, one document at a time: query t of document j may
     attend key u of the same document iff (not causal) or u_local <= t_local + (len_k - len_q); rows without any
@@ -196,13 +260,6 @@ def test_attention_single_token_documents_return_v_exactly():
     assert qg.grad.float().abs().max().item() <= 1e-5 and kg.grad.float().abs().max().item() <= 1e-5
     dv_ref = do.float().view(T, nkv, nq // nkv, d).sum(dim=2)
     assert torch.allclose(vg.grad.float(), dv_ref, rtol=1e-2, atol=1e-2)
-
-
-def _complex_tables(d, rows, base):
-    """fp32 [rows, d / 2] real / imaginary parts of freqs_cis (core/nn/rotary.py:45-56)."""
-    inv_freq = 1.0 / (float(base) ** (torch.arange(0, d, 2)[: d // 2].float() / d))
-    ang = torch.outer(torch.arange(rows).float(), inv_freq).float()
-    return ang.cos().contiguous(), ang.sin().contiguous()
 
 
 @pytest.mark.parametrize("d", [64, 128])
