@@ -562,8 +562,9 @@ class _Attention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, o, lse, cu_q, cu_k = ctx.saved_tensors[:7]
-        rotary = tuple(ctx.saved_tensors[7:11]) if ctx.rotary else None
+        saved = ctx.saved_tensors           # read once: saved-tensor hooks (activation checkpointing) unpack on access
+        q, k, v, o, lse, cu_q, cu_k = saved[:7]
+        rotary = tuple(saved[7:11]) if ctx.rotary else None
         dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale, dropout=ctx.dropout, rotary=rotary)
         return (dq, dk, dv) + (None,) * 10
 
