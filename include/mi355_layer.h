@@ -189,6 +189,11 @@ int mi_rotary_complex(const void* x, void* out, const float* cos, const float* s
  * ------------------------------------------------------------------------------------------ */
 #define MI_ATTN_QG1 1   /* forward: one group of 32 queries per wavefront (128 per workgroup) */
 #define MI_ATTN_QG2 2   /* forward: two groups of 32 queries per wavefront (256 per workgroup) */
+/* Accuracy mode, forward and backward: every bf16 operand that the kernels form themselves (the probabilities P in
+ * P V and dV = P^T dO, dS in dQ = dS K and dK = dS^T Q) enters its MFMA as two bf16 terms hi + lo, so these products
+ * carry 16 mantissa bits instead of 8 (the reference rounds P once to the value dtype, attention.py:211).  Costs a
+ * second pass over those MFMAs (forward 1.5 x, backward 1.4 x the MFMA work).  No dropout; fused rotary on q only. */
+#define MI_ATTN_SPLIT_P 4
 /* backward: run only the named kernels (for per-kernel timing; all three when none of the bits is set) */
 #define MI_ATTN_BWD_DELTA 16
 #define MI_ATTN_BWD_DKDV 32

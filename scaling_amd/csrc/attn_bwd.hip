@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_delta_kernel(const AttnPara
 // (32 of the 64 queries staged per iteration), so the pair (w, w + 4) accumulates the same dK / dV
 // rows and is summed once at the end.  The first four wavefronts stage Q, the last four dO; the staged
 // tiles are double buffered (one barrier per iteration).
-template <int D, bool DROP>
+template <int D, bool DROP, bool SPLIT>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
     constexpr int BNK = 128;              // keys per workgroup
     constexpr int BQ = 64;                // queries per tile
@@ -227,6 +227,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                 }
             }
             bf16x8_t pf[2], dsf[2];
+            bf16x8_t pl[SPLIT ? 2 : 1], dsl[SPLIT ? 2 : 1];   // accuracy mode: low-order terms of P and dS
             uint32_t drop_xb = 0;
             if constexpr (DROP) {
                 const int head_i = kvh * p.n_rep + hs * hpw + iter / n_tiles;
@@ -252,8 +253,13 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                     const float pv = fast_exp2(s_acc[r] * c2 - l4[c]);
                     const float dpv = DROP ? (keep[c] ? dp_acc[r] * p.drop_rscale : 0.f) : dp_acc[r];
                     const float ds = pv * (dpv - d4[c]);
-                    pf[a >> 1][4 * (a & 1) + c] = (__bf16)((DROP && !keep[c]) ? 0.f : pv);
+                    const float pk = (DROP && !keep[c]) ? 0.f : pv;
+                    pf[a >> 1][4 * (a & 1) + c] = (__bf16)pk;
                     dsf[a >> 1][4 * (a & 1) + c] = (__bf16)ds;
+                    if constexpr (SPLIT) {
+                        pl[a >> 1][4 * (a & 1) + c] = (__bf16)(pk - (float)pf[a >> 1][4 * (a & 1) + c]);
+                        dsl[a >> 1][4 * (a & 1) + c] = (__bf16)(ds - (float)dsf[a >> 1][4 * (a & 1) + c]);
+                    }
                 }
             }
 #pragma unroll
@@ -265,6 +271,10 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                     const bf16x8_t aqt = tr_pair(qt_ + o0, qt_ + o1);
                     dv_acc[dt] = mfma_32x32x16(adt, pf[m], dv_acc[dt]);
                     dk_acc[dt] = mfma_32x32x16(aqt, dsf[m], dk_acc[dt]);
+                    if constexpr (SPLIT) {
+                        dv_acc[dt] = mfma_32x32x16(adt, pl[m], dv_acc[dt]);
+                        dk_acc[dt] = mfma_32x32x16(aqt, dsl[m], dk_acc[dt]);
+                    }
                 }
             }
         }
@@ -395,7 +405,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_reduce_kernel(const At
 // 8 wavefronts, two per SIMD, 32 queries each (256 per workgroup); the first four stage K (one
 // token-major tile read both as row operand and transposed), the last four stage V.  Double-buffered
 // LDS, one barrier per 64-key tile.
-template <int D, bool DROP>
+template <int D, bool DROP, bool SPLIT>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p) {
     constexpr int BM = 256;
     constexpr int BN = 64;
@@ -532,7 +542,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
                 const int t = m >> 1, r0 = 8 * (m & 1);
-                bf16x8_t dsf;
+                bf16x8_t dsf, dsl;
                 if constexpr (DROP) {
                     // dP of a dropped probability is zero, that of a kept one carries the 1 / (1 - p) scale
                     const uint32_t drop_xt = drop_xr + (uint32_t)(kt >> 1) * kDropC2;
@@ -548,13 +558,16 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float pv = fast_exp2(s_acc[t][r0 + e] * c2 - lse2);
-                    dsf[e] = (__bf16)(pv * (dp_acc[t][r0 + e] - delta));
+                    const float ds = pv * (dp_acc[t][r0 + e] - delta);
+                    dsf[e] = (__bf16)ds;
+                    if constexpr (SPLIT) dsl[e] = (__bf16)(ds - (float)dsf[e]);
                 }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
                     const int o0 = (tr_h0 ^ (dt << 6)) + 16 * m * RB, o1 = (tr_h1 ^ (dt << 6)) + 16 * m * RB;
                     const bf16x8_t akt = tr_pair(kt_ + o0, kt_ + o1);
                     dq_acc[dt] = mfma_32x32x16(akt, dsf, dq_acc[dt]);
+                    if constexpr (SPLIT) dq_acc[dt] = mfma_32x32x16(akt, dsl, dq_acc[dt]);
                 }
             }
         }
@@ -586,6 +599,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
 
 template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) {
     const int stages = flags & (MI_ATTN_BWD_DELTA | MI_ATTN_BWD_DKDV | MI_ATTN_BWD_DQ);
+    const bool split = (flags & MI_ATTN_SPLIT_P) != 0;     // accuracy mode (no dropout: checked by the entry point)
     const bool all = stages == 0;
     if (all || (stages & MI_ATTN_BWD_DELTA)) {
         const int64_t rows = (int64_t)p.total_q * p.nq;
@@ -597,8 +611,9 @@ template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) 
     }
     if (all || (stages & MI_ATTN_BWD_DKDV)) {
         const int64_t grid = (((int64_t)p.total_k + 127) / 128) * p.nkv * p.hsplit;
-        if (p.drop_thr != 0) attn_bwd_dkdv_kernel<D, true><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
-        else attn_bwd_dkdv_kernel<D, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        if (split) attn_bwd_dkdv_kernel<D, false, true><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        else if (p.drop_thr != 0) attn_bwd_dkdv_kernel<D, true, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        else attn_bwd_dkdv_kernel<D, false, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         int rc = mi_check_launch("attn_bwd_dkdv");
         if (rc != MI_OK) return rc;
         if (p.hsplit > 1) {
@@ -610,8 +625,9 @@ template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) 
     }
     if (all || (stages & MI_ATTN_BWD_DQ)) {
         const int64_t grid = (((int64_t)p.total_q + 255) / 256) * p.nq;
-        if (p.drop_thr != 0) attn_bwd_dq_kernel<D, true><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
-        else attn_bwd_dq_kernel<D, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        if (split) attn_bwd_dq_kernel<D, false, true><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        else if (p.drop_thr != 0) attn_bwd_dq_kernel<D, true, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
+        else attn_bwd_dq_kernel<D, false, false><<<dim3((unsigned)grid), dim3(512), 0, st>>>(p);
         return mi_check_launch("attn_bwd_dq");
     }
     return MI_OK;
@@ -661,6 +677,7 @@ extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
     if (a->o_stride_token % 8 || a->o_stride_head % 8 || b->dk_stride_token % 8 || b->dk_stride_head % 8 ||
         b->dv_stride_token % 8 || b->dv_stride_head % 8)
         return mi_fail(MI_E_ALIGN, "attn_bwd: strides must be multiples of 8 elements");
+    if ((a->flags & MI_ATTN_SPLIT_P) && a->dropout_p > 0.f) return mi_fail(MI_E_SHAPE, "attn_bwd: MI_ATTN_SPLIT_P takes no dropout");
     if (a->total_q == 0) return MI_OK;
     const size_t need = mi_attn_bwd_workspace_bytes(a->total_q, a->n_q_heads, a->head_dim);
     if (!b->workspace || b->workspace_bytes < need || !mi_aligned16(b->workspace))

@@ -29,7 +29,9 @@ constexpr float kRescaleGap = 8.0f;  // log2 units by which a row max may lag be
 // only (k arrives rotated: the training path rotates it once with the stand-alone kernel, because every K tile is
 // loaded by each query block of each head of its group and would be rotated a few hundred times over in here, whereas
 // a Q row is loaded exactly once).  With p.q_rot the rotated q is also written out (the backward kernels stream it).
-template <int D, int NW, int ROTM, bool DROP>
+// SPLIT: the probabilities enter the P V product as two bf16 terms (P = hi + lo, lo = bf16(P - hi)), i.e. with 16
+// mantissa bits instead of 8, at the price of a second pass of P V MFMAs (accuracy mode, MI_ATTN_SPLIT_P).
+template <int D, int NW, int ROTM, bool DROP, bool SPLIT>
 __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p) {
     constexpr int ROT = (ROTM == 1 || ROTM == 2) ? ROTM : 0;        // rotation of K inside the tile loaders
     constexpr int QROT = ROTM == 0 ? 0 : ((ROTM & 1) ? 1 : 2);      // rotation of the Q fragment
@@ -257,6 +259,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     }
     f32x16_t s_acc[2];
     bf16x8_t pf[4];
+    bf16x8_t pl[SPLIT ? 4 : 1];           // low-order terms of the probabilities
     bool pending = false;                 // pf holds the probabilities of the previous tile
 
     // One MFMA phase = up to 16 steps of O^T += V^T P^T (previous tile) followed by up to 16 steps of
@@ -292,6 +295,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
             if (i < PV_STEPS) {
                 const int m = i / DT, dt = i % DT;
                 o_acc[dt] = mfma_32x32x16(a, pf[m], o_acc[dt]);
+                if constexpr (SPLIT) o_acc[dt] = mfma_32x32x16(a, pl[m], o_acc[dt]);
             } else {
                 const int ksi = (i - PV_STEPS) >> 1, t = (i - PV_STEPS) & 1;
                 s_acc[t] = mfma_32x32x16(a, qf[ksi], s_acc[t]);
@@ -372,6 +376,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                     const float ev = fast_exp2(s_acc[t][r0 + e] * c2 - m_use);
                     if (e & 1) rs1 += ev; else rs0 += ev;
                     pf[m][e] = (__bf16)ev;
+                    if constexpr (SPLIT) pl[m][e] = (__bf16)(ev - (float)pf[m][e]);
                 }
                 if constexpr (DROP) {
                     // the row sum above stays that of the full softmax; only the P that multiplies V is masked
@@ -380,8 +385,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                     for (int pi = 0; pi < 4; ++pi) {
                         const int a = 2 * (m & 1) + (pi >> 1), j = pi & 1;
                         const uint32_t h = lowbias32(drop_xt + (uint32_t)(16 * t + 4 * a + j) * kDropC2);
-                        if (drop_byte(h, drop_sel) < p.drop_thr) pf[m][2 * pi] = (__bf16)0.f;
-                        if (drop_byte(h, drop_sel + 8) < p.drop_thr) pf[m][2 * pi + 1] = (__bf16)0.f;
+                        if (drop_byte(h, drop_sel) < p.drop_thr) { pf[m][2 * pi] = (__bf16)0.f; if constexpr (SPLIT) pl[m][2 * pi] = (__bf16)0.f; }
+                        if (drop_byte(h, drop_sel + 8) < p.drop_thr) { pf[m][2 * pi + 1] = (__bf16)0.f; if constexpr (SPLIT) pl[m][2 * pi + 1] = (__bf16)0.f; }
                     }
                 }
             }
@@ -422,17 +427,27 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     }
 }
 
-template <int D, int NW, int ROT, bool DROP> int launch(const AttnParams& p, hipStream_t st) {
+template <int D, int NW, int ROT, bool DROP, bool SPLIT = false> int launch(const AttnParams& p, hipStream_t st) {
     constexpr int BM = 32 * NW;
     const int64_t nqb = ((int64_t)p.total_q + BM - 1) / BM;
     const int64_t grid = nqb * p.nq;
     if (grid > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_fwd: grid too large");
-    attn_fwd_kernel<D, NW, ROT, DROP><<<dim3((unsigned)grid), dim3(64 * NW), 0, st>>>(p);
+    attn_fwd_kernel<D, NW, ROT, DROP, SPLIT><<<dim3((unsigned)grid), dim3(64 * NW), 0, st>>>(p);
     return mi_check_launch("attn_fwd");
 }
 
 // rot: 0 = none, 1 = rotate-half, 2 = interleaved pairs; q_only: k arrives rotated
-template <int D> int launch_d(const AttnParams& p, int rot, bool q_only, int nw, hipStream_t st) {
+template <int D> int launch_d(const AttnParams& p, int rot, bool q_only, int nw, bool split, hipStream_t st) {
+    if (split) {      // accuracy mode: 256-query workgroups, no dropout, rotary on q only
+        if (p.drop_thr != 0 || (rot && !q_only)) return mi_fail(MI_E_SHAPE, "attn_fwd: MI_ATTN_SPLIT_P takes no dropout and rotary on q only");
+        if constexpr (D == 64 || D == 128) {
+            if (rot == 2) return launch<D, 8, 4, false, true>(p, st);
+            if (rot == 1) return launch<D, 8, 3, false, true>(p, st);
+        } else {
+            if (rot) return mi_fail(MI_E_SHAPE, "attn_fwd: fused rotary needs head_dim 64 or 128");
+        }
+        return launch<D, 8, 0, false, true>(p, st);
+    }
     if (rot) {
         if constexpr (D == 64 || D == 128) {
             if (p.drop_thr != 0) {           // dropout: one tiling per head_dim (256-query workgroups), rotary on q only
@@ -480,13 +495,15 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     int nw = p.total_q > 128 ? 8 : 4;
     if (a->flags & MI_ATTN_QG1) nw = 4;
     if (a->flags & MI_ATTN_QG2) nw = 8;
+    const bool split = (a->flags & MI_ATTN_SPLIT_P) != 0;
+    if (split) nw = 8;
     if (p.n_rep == 1) p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 32 * nw);
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
-        case 32: return launch_d<32>(p, rot, q_only, nw, st);
-        case 64: return launch_d<64>(p, rot, q_only, nw, st);
-        case 96: return launch_d<96>(p, rot, q_only, nw, st);
-        case 128: return launch_d<128>(p, rot, q_only, nw, st);
+        case 32: return launch_d<32>(p, rot, q_only, nw, split, st);
+        case 64: return launch_d<64>(p, rot, q_only, nw, split, st);
+        case 96: return launch_d<96>(p, rot, q_only, nw, split, st);
+        case 128: return launch_d<128>(p, rot, q_only, nw, split, st);
         default: return mi_fail(MI_E_SHAPE, "attn_fwd: head_dim %d unsupported (32, 64, 96, 128)", a->head_dim);
     }
 }

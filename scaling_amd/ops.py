@@ -469,8 +469,11 @@ def _check_qkv(q, k, v, cu_q, cu_k):
         assert cu_k.dtype == torch.int32 and cu_k.is_contiguous() and cu_k.numel() == cu_q.numel()
 
 
+SPLIT_P = 4   # MI_ATTN_SPLIT_P
+
+
 def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None, rotary=None, flags=0,
-                      dropout=None, return_rotated_q=False):
+                      dropout=None, return_rotated_q=False, precise=False):
     """Returns (o [tokens, n_q_heads, head_dim], lse fp32 [n_q_heads, tokens]) (+ the rotated q if asked).
 
     rotary: optional (cos, sin, position_ids_q, position_ids_k), q and k are rotated while they are loaded:
@@ -480,10 +483,13 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
 
     dropout: optional (p, seed) for dropout on the attention probabilities; the backward needs the same pair.
 
-    flags: 0 lets the library pick the tiling; 1 / 2 pin one / two query groups per wavefront."""
+    flags: 0 lets the library pick the tiling; 1 / 2 pin one / two query groups per wavefront.
+    precise: accuracy mode (probabilities enter P V as two bf16 terms; no dropout, rotary on q only)."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
+    if precise:
+        flags |= SPLIT_P
     q_rot = None
     if rotary is not None:
         cos, sin, pos_q, pos_k = rotary
@@ -502,7 +508,7 @@ def attention_forward(q, k, v, cu_seqlens_q, cu_seqlens_k=None, causal=True, sof
 
 
 def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, causal=True, softmax_scale=None,
-                       flags=0, buffers=None, dropout=None, rotary=None):
+                       flags=0, buffers=None, dropout=None, rotary=None, precise=False):
     """Returns (dq, dk, dv).  The summation order is fixed: results are bit-reproducible
     (what masked_softmax.deterministic_flash_attn_bwd asks of the reference's fused kernel holds always).
 
@@ -510,9 +516,12 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
     dq / dk come back as gradients of the unrotated ones (rotated back inside the kernels, one rounding).
 
     flags: 0 runs the whole backward; 16 / 32 / 64 run only the delta / dK-dV / dQ kernel (timing aid).
-    buffers: optional (dq, dk, dv, workspace) to reuse across calls."""
+    buffers: optional (dq, dk, dv, workspace) to reuse across calls.
+    precise: accuracy mode (P and dS enter their MFMAs as two bf16 terms each; no dropout)."""
     _check_qkv(q, k, v, cu_seqlens_q, cu_seqlens_k)
     lib = _lib.load()
+    if precise:
+        flags |= SPLIT_P
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
     if do.stride() != o.stride():
@@ -541,10 +550,11 @@ def attention_backward(do, q, k, v, o, lse, cu_seqlens_q, cu_seqlens_k=None, cau
 
 class _Attention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, cu_q, cu_k, causal, scale, dropout_p, dropout_seed, cos, sin, pos_q, pos_k):
+    def forward(ctx, q, k, v, cu_q, cu_k, causal, scale, dropout_p, dropout_seed, cos, sin, pos_q, pos_k, precise):
         dropout = (dropout_p, dropout_seed) if dropout_p > 0.0 else None
+        ctx.precise = precise
         if cos is None:
-            o, lse = attention_forward(q, k, v, cu_q, cu_k, causal, scale, dropout=dropout)
+            o, lse = attention_forward(q, k, v, cu_q, cu_k, causal, scale, dropout=dropout, precise=precise)
             ctx.save_for_backward(q, k, v, o, lse, cu_q, cu_k if cu_k is not None else cu_q)
         else:
             # rotary: k is rotated once by the stand-alone kernel, q while the attention kernel loads it; the rotated
@@ -553,10 +563,11 @@ class _Attention(torch.autograd.Function):
             k_rot = (_rotary_complex_launch if interleaved else _rotary_launch)(k, cos, sin, pos_k, 0, False)
             if any(ctx.needs_input_grad[:3]):
                 o, lse, q_rot = attention_forward(q, k_rot, v, cu_q, cu_k, causal, scale, rotary=(cos, sin, pos_q, None),
-                                                  dropout=dropout, return_rotated_q=True)
+                                                  dropout=dropout, return_rotated_q=True, precise=precise)
                 ctx.save_for_backward(q_rot, k_rot, v, o, lse, cu_q, cu_k if cu_k is not None else cu_q, cos, sin, pos_q, pos_k)
             else:   # nothing to differentiate: the rotated q is not written out
-                o, lse = attention_forward(q, k_rot, v, cu_q, cu_k, causal, scale, rotary=(cos, sin, pos_q, None), dropout=dropout)
+                o, lse = attention_forward(q, k_rot, v, cu_q, cu_k, causal, scale, rotary=(cos, sin, pos_q, None), dropout=dropout,
+                                           precise=precise)
         ctx.causal, ctx.scale, ctx.dropout, ctx.rotary = causal, scale, dropout, cos is not None
         return o
 
@@ -565,8 +576,9 @@ class _Attention(torch.autograd.Function):
         saved = ctx.saved_tensors           # read once: saved-tensor hooks (activation checkpointing) unpack on access
         q, k, v, o, lse, cu_q, cu_k = saved[:7]
         rotary = tuple(saved[7:11]) if ctx.rotary else None
-        dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale, dropout=ctx.dropout, rotary=rotary)
-        return (dq, dk, dv) + (None,) * 10
+        dq, dk, dv = attention_backward(do, q, k, v, o, lse, cu_q, cu_k, ctx.causal, ctx.scale, dropout=ctx.dropout, rotary=rotary,
+                                        precise=ctx.precise)
+        return (dq, dk, dv) + (None,) * 11
 
 
 def next_dropout_seed(device: torch.device) -> int:
@@ -582,7 +594,7 @@ def next_dropout_seed(device: torch.device) -> int:
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
               cu_seqlens_k: Optional[torch.Tensor] = None, causal: bool = True,
               softmax_scale: Optional[float] = None, dropout_p: float = 0.0,
-              dropout_seed: Optional[int] = None, rotary=None, deterministic: bool = False) -> torch.Tensor:
+              dropout_seed: Optional[int] = None, rotary=None, deterministic: bool = False, precise: bool = False) -> torch.Tensor:
     """Differentiable attention core on q [tokens, n_q, d], k/v [tokens_k, n_kv, d] (bf16).
 
     Tokens are the flattened (batch seq) axis; cu_seqlens are int32 offsets on it.  Returns
@@ -596,6 +608,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
     epilogues, with or without autograd, with or without dropout.
     deterministic mirrors masked_softmax.deterministic_flash_attn_bwd of the reference; the kernels sum in a fixed
     order whatever its value.
+    precise selects the accuracy mode of forward and backward: P and dS enter their products as two bf16 terms, which
+    brings outputs and gradients within max-abs 2e-2 / mean-relative 1e-3 of the fp32 reference (the default mode
+    rounds P once to bf16 as the reference does); about 1.4 x the time; no dropout.
     """
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])
@@ -608,7 +623,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
         assert pos_q.dtype == torch.int64 and pos_q.is_contiguous() and pos_q.numel() == q.shape[0]
         assert pos_k.dtype == torch.int64 and pos_k.is_contiguous() and pos_k.numel() == k.shape[0]
     return _Attention.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, causal, float(softmax_scale), float(dropout_p),
-                            int(dropout_seed) if dropout_seed is not None else 0, cos, sin, pos_q, pos_k)
+                            int(dropout_seed) if dropout_seed is not None else 0, cos, sin, pos_q, pos_k, bool(precise))
 
 
 # ------------------------------------------------------------------------------------------------

@@ -39,13 +39,17 @@ def _slice_reference(q, k, v, do, cu, b, s, heads, kvh, scale, dtype, rotary=Non
 
 
 @pytest.mark.timeout(600)
+@pytest.mark.parametrize("precise", [False, True])
 @pytest.mark.parametrize("name,b,s,nq,nkv,docs,rotary", [
     ("headline", 1, 8192, 32, 8, False, False),     # the workload of the headline metric
     ("config2", 4, 2048, 32, 32, False, False),
     ("config3", 1, 8192, 32, 8, True, True),        # packed documents of 256..2048 tokens, rotary base 500000
 ])
-def test_attention_fwd_bwd_full_size_against_oracle_slices(name, b, s, nq, nkv, docs, rotary):
-    print(f"case full-size attention {name}", flush=True)
+def test_attention_fwd_bwd_full_size_against_oracle_slices(name, b, s, nq, nkv, docs, rotary, precise):
+    """precise=True is the accuracy mode (P and dS as hi + lo bf16 terms): held to the gates exactly as stated, except
+    with rotary, where q and k are attended with after one rounding to bf16 (as the reference's bf16 path does) while
+    the fp32 oracle rotates without rounding."""
+    print(f"case full-size attention {name} precise={precise}", flush=True)
     d = 128
     q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=200 + s + nq + nkv)
     cu = U.random_docs_cu(b * s, 256, 2048, seed=0) if docs else U.make_cu(b, s)
@@ -56,9 +60,10 @@ def test_attention_fwd_bwd_full_size_against_oracle_slices(name, b, s, nq, nkv, 
         pos = U.position_ids_from_cu(cu, b * s)
         tabs = oracle.rotary_tables(d, s, 500000, torch.bfloat16)
         rot_ref = (tabs, pos)
-        o = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale, rotary=(tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV), pos.to(DEV)))
+        o = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale, rotary=(tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV), pos.to(DEV)),
+                          precise=precise)
     else:
-        o = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale)
+        o = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale, precise=precise)
     o.backward(do.to(DEV))
     torch.cuda.synchronize()
     assert bool(torch.isfinite(o.float()).all()) and all(bool(torch.isfinite(t.grad.float()).all()) for t in (qg, kg, vg))
@@ -67,10 +72,12 @@ def test_attention_fwd_bwd_full_size_against_oracle_slices(name, b, s, nq, nkv, 
         heads = list(range(kvh * n_rep, (kvh + 1) * n_rep))
         ref = _slice_reference(q, k, v, do, cu, b, s, heads, kvh, scale, torch.float32, rot_ref)
         ref_o = _slice_reference(q, k, v, do, cu, b, s, heads, kvh, scale, torch.bfloat16, rot_ref)
-        check(f"{name}.o[kv{kvh}]", o[:, heads], ref[0], ref_o[0])
-        check(f"{name}.dq[kv{kvh}]", qg.grad[:, heads], ref[1], ref_o[1])
-        check(f"{name}.dk[kv{kvh}]", kg.grad[:, kvh], ref[2], ref_o[2])
-        check(f"{name}.dv[kv{kvh}]", vg.grad[:, kvh], ref[3], ref_o[3])
+        lit = precise and not rotary
+        tag = f"{name}.precise" if precise else name
+        check(f"{tag}.o[kv{kvh}]", o[:, heads], ref[0], ref_o[0], literal=lit)
+        check(f"{tag}.dq[kv{kvh}]", qg.grad[:, heads], ref[1], ref_o[1], literal=lit)
+        check(f"{tag}.dk[kv{kvh}]", kg.grad[:, kvh], ref[2], ref_o[2], literal=lit)
+        check(f"{tag}.dv[kv{kvh}]", vg.grad[:, kvh], ref[3], ref_o[3], literal=lit)
 
 
 @pytest.mark.timeout(600)
