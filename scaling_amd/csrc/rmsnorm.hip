@@ -237,18 +237,16 @@ __global__ __launch_bounds__(kRmsWideBlock) void rmsnorm_bwd_wide_kernel(const T
             gv[c] = ok ? gr[v] : make_uint4(0, 0, 0, 0);
         }
     };
-    constexpr bool kPrefetch = CH <= 2;   // beyond that the second register set would spill
-    if (iters > 0) fetch(0, xraw, graw);
-    for (int64_t it = 0; it < iters; ++it) {
+    // one row step: reduce the two row sums over the row's wavefronts (one barrier), write dx, add to dweight
+    auto process = [&](int64_t it, const uint4 (&xv)[CH], const uint4 (&gv)[CH]) {
         const int64_t row = it * row_step + (int64_t)blockIdx.x * RPB + rg;
         const bool row_ok = row < n_rows;
-        if (kPrefetch) { if (it + 1 < iters) fetch(it + 1, xnext, gnext); }
         float ss = 0.f, dot = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             float xf[V], gf[V], wf[V];
-            Elem<T>::unpack(xraw[c], xf);
-            Elem<T>::unpack(graw[c], gf);
+            Elem<T>::unpack(xv[c], xf);
+            Elem<T>::unpack(gv[c], gf);
             const int v0 = (c * TPR + tr < vecs ? c * TPR + tr : 0) * V;
 #pragma unroll
             for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v0 + i);
@@ -280,8 +278,8 @@ __global__ __launch_bounds__(kRmsWideBlock) void rmsnorm_bwd_wide_kernel(const T
                 const int v = c * TPR + tr;
                 if (v < vecs) {
                     float xf[V], gf[V], wf[V], o[V];
-                    Elem<T>::unpack(xraw[c], xf);
-                    Elem<T>::unpack(graw[c], gf);
+                    Elem<T>::unpack(xv[c], xf);
+                    Elem<T>::unpack(gv[c], gf);
 #pragma unroll
                     for (int i = 0; i < V; i += 4) *reinterpret_cast<f32x4_t*>(wf + i) = *reinterpret_cast<const f32x4_t*>(w_lds + v * V + i);
 #pragma unroll
@@ -293,11 +291,42 @@ __global__ __launch_bounds__(kRmsWideBlock) void rmsnorm_bwd_wide_kernel(const T
                 }
             }
         }
-        if (kPrefetch) {
-#pragma unroll
-            for (int c = 0; c < CH; ++c) { xraw[c] = xnext[c]; graw[c] = gnext[c]; }
-        } else if (it + 1 < iters) {
-            fetch(it + 1, xraw, graw);
+    };
+    // Three register sets rotate: the rows of steps it + 1 and it + 2 are in flight while step it is reduced (two
+    // steps of loads outstanding per compute unit cover the memory latency; with one, the block-wide barrier
+    // made every wavefront issue its loads at the same moment and the memory pipe ran dry in between).  The loop
+    // is unrolled by three so that every set is addressed statically; `iters` is the same for the whole block.
+    constexpr bool kDeep = CH == 1;       // three register sets fit without spilling only for one vector per thread
+    if constexpr (kDeep) {
+        uint4 x2[CH], g2[CH];
+        if (iters > 0) fetch(0, xraw, graw);
+        if (iters > 1) fetch(1, xnext, gnext);
+        for (int64_t it = 0; it < iters; it += 3) {
+            if (it + 2 < iters) fetch(it + 2, x2, g2);
+            process(it, xraw, graw);
+            if (it + 1 < iters) {
+                if (it + 3 < iters) fetch(it + 3, xraw, graw);
+                process(it + 1, xnext, gnext);
+            }
+            if (it + 2 < iters) {
+                if (it + 4 < iters) fetch(it + 4, xnext, gnext);
+                process(it + 2, x2, g2);
+            }
+        }
+    } else if constexpr (CH <= 2) {       // two sets: the rows of step it + 1 are in flight while step it is reduced
+        if (iters > 0) fetch(0, xraw, graw);
+        for (int64_t it = 0; it < iters; it += 2) {
+            if (it + 1 < iters) fetch(it + 1, xnext, gnext);
+            process(it, xraw, graw);
+            if (it + 1 < iters) {
+                if (it + 2 < iters) fetch(it + 2, xraw, graw);
+                process(it + 1, xnext, gnext);
+            }
+        }
+    } else {
+        for (int64_t it = 0; it < iters; ++it) {
+            fetch(it, xraw, graw);
+            process(it, xraw, graw);
         }
     }
     for (int i = threadIdx.x; i < hidden; i += kRmsWideBlock) dw_lds[i] = 0.f;
@@ -441,7 +470,7 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
     // wide rows: 256 threads per row up to 512 vectors (4 rows per block and step), 512 up to 1024, the whole block
     // beyond: at most two vectors per thread, so that the next step's rows always fit in registers next to this
     // step's (four vectors per thread without that prefetch ran at 1.9 TB/s at hidden 12288)
-    const int wide_tpr = vecs <= 512 ? 256 : (vecs <= 1024 ? 512 : 1024);
+    const int wide_tpr = vecs <= 256 ? 256 : (vecs <= 1024 ? 512 : 1024);
     // wide rows: a single round of blocks (two per compute unit), each amortising its epilogue over many rows
     const int wide_rpb = kRmsWideBlock / wide_tpr;
     const int64_t wide_blocks = (n_rows + wide_rpb - 1) / wide_rpb;
@@ -456,7 +485,7 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
 #define RMS_WIDE(TPRV, CHV) rmsnorm_bwd_wide_kernel<T, TPRV, CHV><<<dim3(blocks), dim3(kRmsWideBlock), lds, st>>>( \
             (const T*)x, (const T*)w, (const T*)dy, (T*)dx, (float*)ws, n_rows, (int)hidden, eps)
         if (wide_tpr == 256) { if (ch <= 1) RMS_WIDE(256, 1); else RMS_WIDE(256, 2); }
-        else if (wide_tpr == 512) RMS_WIDE(512, 2);
+        else if (wide_tpr == 512) { if (ch <= 1) RMS_WIDE(512, 1); else RMS_WIDE(512, 2); }
         else RMS_WIDE(1024, 2);
 #undef RMS_WIDE
         int rcw = mi_check_launch("rmsnorm_bwd_wide");
