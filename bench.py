@@ -29,14 +29,36 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, vendor figure
 
-# HBM bytes per launch of the attention kernels on the headline workload: rocprofv3 FETCH_SIZE and WRITE_SIZE
-# (KiB per dispatch, one counter per run), scaled by what the same counters read for a plain 1 GiB device copy
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Summary and commands: profiles/attention_fwd_bwd_gqa32x8_d128_s8192_hbm_traffic.md
-MEASURED_TRAFFIC_KIB = {
-    "attn_fwd_kernel": 2.0 * 72101 + 66560,
-    "attn_bwd_dkdv_kernel": 2.0 * 703245 + 32788,
-    "attn_bwd_dq_kernel": 2.0 * 106432 + 65536,
-}
+# HBM bytes per launch of the attention kernels on the headline workload come from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+# whose figures are kept in this file together with a hash of the kernel sources they were measured on; the figure is
+# reported only while the sources are unchanged.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "attention_fwd_bwd_gqa32x8_d128_s8192_hbm_traffic.json")
+ATTENTION_SOURCES = ("attn_common.h", "attn_fwd.hip", "attn_bwd.hip", "attn_host.hip", "common.h")
+
+
+def attention_sources_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for name in ATTENTION_SOURCES:
+        with open(os.path.join(ROOT, "scaling_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic_bytes(kernel):
+    """HBM bytes per launch of `kernel` from the counter runs, or (None, reason) when there is no current measurement."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            data = json.load(f)
+    except (OSError, ValueError):
+        return None, "no counter measurement on file"
+    if data.get("sources_sha256") != attention_sources_hash():
+        return None, "the kernel sources changed after the counters were taken"
+    k = data.get("kernels", {}).get(kernel)
+    if not k:
+        return None, "kernel not in the counter file"
+    cal = data["calibration"]
+    return 1024.0 * (cal["fetch_scale"] * k["fetch_size_kib"] + cal["write_scale"] * k["write_size_kib"]), None
 
 
 def causal_pairs(cu):
@@ -92,6 +114,23 @@ def time_gpu_graph(fn, steps, warmup):
         return time_gpu(fn, steps, warmup)
 
 
+def time_rotating(make_call, n_sets, steps, warmup):
+    """Average milliseconds per call over a HIP-graph replay that cycles through n_sets distinct sets of input buffers
+    (and keeps n_sets results alive, so the outputs land in distinct buffers too): with the sets totalling more than
+    twice the 256 MB Infinity Cache every call streams from and to HBM, which replaying one set of 134 - 201 MB does
+    not guarantee.  make_call(k) returns the zero-argument call for buffer set k."""
+    calls = [make_call(k) for k in range(n_sets)]
+    keep = [None] * n_sets
+    counter = [0]
+
+    def one():
+        k = counter[0] % n_sets
+        counter[0] += 1
+        keep[k] = calls[k]()
+
+    return time_gpu_graph(one, max(steps, 2 * n_sets), max(warmup, n_sets))
+
+
 def random_docs_cu(total, lo, hi, seed):
     """Cumulative document lengths: lengths uniform in [lo, hi], the last one truncated so they sum to `total`."""
     import torch
@@ -108,6 +147,37 @@ def _rotary_tables(dim, max_seq, base, device):
     from scaling_amd.config import RotaryConfig
     from scaling_amd.nn import RotaryEmbedding
     return RotaryEmbedding(RotaryConfig(dimensions=dim, max_seq_length=max_seq, base=base), torch.device(device), torch.bfloat16).tables()
+
+
+def _check_sampled_rows(q, k, v, do, o, lse, dq, dk, dv, cu_list, scale):
+    """Finite outputs plus one sampled row per stage against plain fp32 torch arithmetic on that row."""
+    import torch
+    for name, t in (("o", o), ("lse", lse), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert bool(torch.isfinite(t.float()).all()), f"attention {name} has non-finite values"
+    n_rep = q.shape[1] // k.shape[1]
+    qf, kf, vf, dof, of = (t.float() for t in (q, k, v, do, o))
+
+    def close(name, got, want):
+        err = (got.float() - want).abs().max().item()
+        tol = 0.03 * max(1.0, want.abs().max().item())
+        assert err <= tol, f"attention {name}: sampled row off by {err:.3e} (tolerance {tol:.3e})"
+
+    # last query of the last document, head 0: attends keys [lo, t]
+    t, lo, h = cu_list[-1] - 1, cu_list[-2], 0
+    p = torch.softmax((kf[lo:t + 1, 0] @ qf[t, h]) * scale, 0)
+    close("o row", o[t, h], p @ vf[lo:t + 1, 0])
+    ds = p * (vf[lo:t + 1, 0] @ dof[t, h] - (dof[t, h] * of[t, h]).sum())
+    close("dq row", dq[t, h], scale * (ds @ kf[lo:t + 1, 0]))
+    # first key of the first document, KV head 0: every query of that document and of the group's heads attends it
+    hi = cu_list[1]
+    dk_row, dv_row = torch.zeros_like(kf[0, 0]), torch.zeros_like(vf[0, 0])
+    for hh in range(n_rep):
+        pj = torch.exp((qf[:hi, hh] @ kf[0, 0]) * scale - lse[hh, :hi])              # P[:, key 0] from the saved log-sum-exp
+        dsj = pj * (dof[:hi, hh] @ vf[0, 0] - (dof[:hi, hh] * of[:hi, hh]).sum(-1))
+        dv_row += pj @ dof[:hi, hh]
+        dk_row += scale * (dsj @ qf[:hi, hh])
+    close("dv row", dv[0, 0], dv_row)
+    close("dk row", dk[0, 0], dk_row)
 
 
 def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=False):
@@ -138,6 +208,10 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
     from scaling_amd import _lib
     ws = torch.empty(_lib.load().mi_attn_bwd_workspace_bytes_kv(T, T, nq, nkv, d) // 4, dtype=torch.float32, device=dev)
     bufs = (dq, dk, dv, ws)
+    # before anything is timed: every output finite, and one row of each (the last query's o and dq, the first key's
+    # dk and dv) equal to a plain fp32 evaluation of that row (the full comparison with the oracle is tests/'s job)
+    ops.attention_backward(do, q, k, v, o, lse, cu, None, True, scale, buffers=bufs)
+    _check_sampled_rows(q, k, v, do, o, lse, dq, dk, dv, cu_list, scale)
 
     def fwd():
         ops.attention_forward(q, k, v, cu, None, True, scale)
@@ -189,19 +263,30 @@ def bandwidth_cases(steps, warmup):
     out = {}
     g = torch.Generator().manual_seed(1)
     N, H, I = 8192, 4096, 14336
-    x = torch.randn(N, H, generator=g).bfloat16().to(dev)
     w = torch.ones(H, dtype=torch.bfloat16, device=dev)
-    dy = torch.randn(N, H, generator=g).bfloat16().to(dev)
-    ms = time_gpu_graph(lambda: ops.rms_norm_forward(x, w, 1e-5), steps, warmup)
-    out["rmsnorm_fwd"] = {"ms": ms, "GBs": 2 * N * H * 2 / ms / 1e6}
-    ms = time_gpu_graph(lambda: ops.rms_norm_backward(x, w, dy, 1e-5), steps, warmup)
-    out["rmsnorm_bwd"] = {"ms": ms, "GBs": 3 * N * H * 2 / ms / 1e6}
     bias = torch.zeros(H, dtype=torch.bfloat16, device=dev)
-    ms = time_gpu_graph(lambda: ops.layer_norm_forward(x, w, bias, 1e-5), steps, warmup)
-    out["layernorm_fwd"] = {"ms": ms, "GBs": 2 * N * H * 2 / ms / 1e6}
+    # The norm and rotary working sets (134 - 201 MB) fit the 256 MB Infinity Cache: "GBs" cycles through 8 distinct
+    # buffer sets (0.5 - 1.1 GB of inputs), "GBs_same_buffers" replays one set (part of its traffic can be cache hits)
+    n_sets = 8
+    xs = [torch.randn(N, H, generator=g).bfloat16().to(dev) for _ in range(n_sets)]
+    dys = [torch.randn(N, H, generator=g).bfloat16().to(dev) for _ in range(n_sets)]
+    x, dy = xs[0], dys[0]
     _, ln_stats = ops.layer_norm_forward(x, w, bias, 1e-5, save_stats=True)   # as the autograd function runs it
-    ms = time_gpu_graph(lambda: ops.layer_norm_backward(x, w, dy, 1e-5, True, ln_stats), steps, warmup)
-    out["layernorm_bwd"] = {"ms": ms, "GBs": 3 * N * H * 2 / ms / 1e6}
+    stats = [ops.layer_norm_forward(xi, w, bias, 1e-5, save_stats=True)[1] for xi in xs]
+
+    def both(name, nbytes, rotating, same):
+        ms = time_rotating(rotating, n_sets, steps, warmup)
+        ms_same = time_gpu_graph(same, steps, warmup)
+        out[name] = {"ms": ms, "GBs": nbytes / ms / 1e6, "ms_same_buffers": ms_same, "GBs_same_buffers": nbytes / ms_same / 1e6}
+
+    both("rmsnorm_fwd", 2 * N * H * 2, lambda k: (lambda: ops.rms_norm_forward(xs[k], w, 1e-5)), lambda: ops.rms_norm_forward(x, w, 1e-5))
+    both("rmsnorm_bwd", 3 * N * H * 2, lambda k: (lambda: ops.rms_norm_backward(xs[k], w, dys[k], 1e-5)),
+         lambda: ops.rms_norm_backward(x, w, dy, 1e-5))
+    both("layernorm_fwd", 2 * N * H * 2, lambda k: (lambda: ops.layer_norm_forward(xs[k], w, bias, 1e-5)),
+         lambda: ops.layer_norm_forward(x, w, bias, 1e-5))
+    both("layernorm_bwd", 3 * N * H * 2, lambda k: (lambda: ops.layer_norm_backward(xs[k], w, dys[k], 1e-5, True, stats[k])),
+         lambda: ops.layer_norm_backward(x, w, dy, 1e-5, True, ln_stats))
+    del xs, dys, stats
     a = torch.randn(N, I, generator=g).bfloat16().to(dev)
     gate = torch.randn(N, I, generator=g).bfloat16().to(dev)
     dout = torch.randn(N, I, generator=g).bfloat16().to(dev)
@@ -225,12 +310,12 @@ def bandwidth_cases(steps, warmup):
     out["cross_entropy_fwd_bwd"] = {"ms": ms, "GBs": 2 * rows * vocab * 2 / ms / 1e6}
     del logits, dlogits
     nq, nkv, d = 32, 8, 128
-    qk = torch.randn(N, nq + nkv, d, generator=g).bfloat16().to(dev)
+    qks = [torch.randn(N, nq + nkv, d, generator=g).bfloat16().to(dev) for _ in range(n_sets)]
     cos, sin = _rotary_tables(d, 8192, 500000, dev)
     pos = torch.arange(N, dtype=torch.int64, device=dev) % 4096
-    ms = time_gpu_graph(lambda: ops.rotary_embedding(qk, cos, sin, pos), steps, warmup)
-    out["rotary"] = {"ms": ms, "GBs": (2 * N * (nq + nkv) * d * 2 + 8 * N) / ms / 1e6}
-    del qk
+    both("rotary", 2 * N * (nq + nkv) * d * 2 + 8 * N, lambda k: (lambda: ops.rotary_embedding(qks[k], cos, sin, pos)),
+         lambda: ops.rotary_embedding(qks[0], cos, sin, pos))
+    del qks
     B, ctx, max_ctx = 32, 4096, 4352
     # head-major storage viewed as [batch, token, kv head, d]: the layout scaling_amd.nn.KVCache allocates
     kc = torch.randn(B, nkv, max_ctx, d, generator=g).bfloat16().to(dev).transpose(1, 2)
@@ -241,6 +326,12 @@ def bandwidth_cases(steps, warmup):
     od = torch.empty_like(q1)
     ms = time_gpu_graph(lambda: ops.decode_attention(q1, kc, vc, ctx_len, workspace=wsd, out=od), steps, warmup)
     out["decode_attention"] = {"ms": ms, "GBs": 2 * B * ctx * nkv * d * 2 / ms / 1e6, "batch": B, "ctx": ctx}
+    # what a plain device copy of 1 GiB reaches on this box: the practical ceiling of a one-in one-out stream
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    ms = time_gpu_graph(lambda: dst.copy_(src), max(5, steps // 2), 2)
+    out["device_copy_1GiB"] = {"ms": ms, "GBs": 2 * (1 << 30) / ms / 1e6}
+    del src, dst
     for v_ in out.values():
         v_["frac_of_hbm_peak"] = v_["GBs"] / PEAK_HBM_GBS
     return out
@@ -342,13 +433,34 @@ def decode_case(steps, layers=32, batch=32, prompt=4096):
     return out
 
 
+def _cpu_info():
+    model, physical = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name") and model == "unknown":
+                model = line.split(":", 1)[1].strip()
+            elif line.startswith("physical id"):
+                phys = line.split(":", 1)[1].strip()
+            elif line.startswith("core id"):
+                core = line.split(":", 1)[1].strip()
+                physical.add((phys, core))
+    except OSError:
+        pass
+    return model, os.cpu_count() or 1, len(physical) or None
+
+
 def cpu_baseline(seconds_budget=25.0):
-    """The reference's operation order (CPU oracle) on a bounded sample of the headline workload:
-    same head_dim / GQA ratio / causal mask / bf16 with fp32 softmax, fewer heads and a shorter sequence."""
+    """The reference's operation order (CPU oracle, plain torch) on the host cores, two bounded samples:
+    the headline workload's attention (same head_dim / GQA ratio / causal mask / bf16 with fp32 softmax, fewer heads and
+    a shorter sequence), which gives `value` in the metric's unit, and config 1 (the reference's own CPU-runnable case:
+    one transformer layer forward + backward, fp32) at full size."""
     import torch
     import oracle
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
+    model, logical, physical = _cpu_info()
+    # the CPU share of a one-GPU box is what OMP_NUM_THREADS announces (16 here), whatever the machine has in total
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or logical
+    cores = max(1, min(cores, logical))
     torch.set_num_threads(cores)
     s, nq, nkv, d = 2048, 4, 1, 128
     g = torch.Generator().manual_seed(0)
@@ -364,18 +476,50 @@ def cpu_baseline(seconds_budget=25.0):
         out.backward(do)
         q.grad = k.grad = v.grad = None
 
-    step()
-    times = []
-    t_all = time.time()
-    while len(times) < 3 or (time.time() - t_all < seconds_budget / 2 and len(times) < 10):
-        t0 = time.time()
-        step()
-        times.append(time.time() - t0)
-    med = sorted(times)[len(times) // 2]
+    def median_time(fn, budget, min_runs=3, max_runs=10):
+        fn()
+        times, t_all = [], time.time()
+        while len(times) < min_runs or (time.time() - t_all < budget and len(times) < max_runs):
+            t0 = time.time()
+            fn()
+            times.append(time.time() - t0)
+        return sorted(times)[len(times) // 2], len(times)
+
+    med, n_runs = median_time(step, seconds_budget / 3)
     flops = 14 * d * nq * (s * (s + 1) // 2)
+
+    # config 1: hidden 256, 4 heads x 64, SwiGLU 688, RMSNorm, rotary base 10000, causal, batch 2 x seq 128, fp32
+    spec = oracle.LayerSpec(hidden_size=256, num_attention_heads=4, qkv_in_one=False, norm_type="rms", mlp_type="swiglu",
+                            layernorm_epsilon=1e-5, rotary_base=10000, sequence_length=128, causal=True, softmax_in_fp32=True,
+                            dtype=torch.float32)
+    g1 = torch.Generator().manual_seed(0)
+    shapes = {"self_attention.query.weight": (256, 256), "self_attention.key.weight": (256, 256), "self_attention.value.weight": (256, 256),
+              "self_attention.dense.weight": (256, 256), "mlp.dense_in.weight": (688, 256), "mlp.siglu_weight.weight": (688, 256),
+              "mlp.dense_out.weight": (256, 688)}
+    w1 = {name: (torch.randn(shape, generator=g1) * 0.02).requires_grad_() for name, shape in shapes.items()}
+    w1["input_layernorm.weight"] = torch.ones(256, requires_grad=True)
+    w1["post_attention_layernorm.weight"] = torch.ones(256, requires_grad=True)
+    x1 = torch.randn(2, 128, 256, generator=g1).requires_grad_()
+    dy1 = torch.randn(2, 128, 256, generator=g1)
+    cu1 = torch.tensor([0, 128, 256], dtype=torch.int32)
+    pos1 = torch.arange(128).repeat(2, 1)
+    tables = spec.tables()
+
+    def step_c1():
+        y = oracle.transformer_layer(spec, w1, x1, cu1, pos1, tables=tables)
+        y.backward(dy1)
+        x1.grad = None
+        for t in w1.values():
+            t.grad = None
+
+    med1, n1 = median_time(step_c1, seconds_budget / 3, min_runs=5, max_runs=200)
     return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "cpu_model": model, "logical_cpus": logical, "physical_cores": physical,
             "sample": f"oracle (reference op order, bf16 + fp32 softmax) attention fwd+bwd, b1 s{s} {nq}q/{nkv}kv d{d} causal, "
-                      f"median of {len(times)} runs = {med * 1e3:.1f} ms"}
+                      f"median of {n_runs} runs = {med * 1e3:.1f} ms; config 1 (one layer fwd+bwd, fp32, hidden 256, 4 heads x 64, "
+                      f"SwiGLU 688, batch 2 x seq 128) at full size: median of {n1} runs = {med1 * 1e3:.2f} ms "
+                      f"({256 / med1:.0f} tokens/s)",
+            "config1_layer_ms": med1 * 1e3, "config1_tokens_per_s": 256 / med1}
 
 
 def main():
@@ -424,8 +568,9 @@ def main():
     dom = max(kernels, key=lambda n: kernels[n][0])
     dom_ms, dom_mult = kernels[dom]
     achieved = dom_mult * flops_unit / (dom_ms * 1e-3) / 1e12
+    traffic, traffic_note = measured_traffic_bytes(dom)
     roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic, "traffic_unit": "bytes per launch", "traffic_note": traffic_note,
                 "avg_launch_ms": dom_ms}
 
     extra = {"headline": main_res}
