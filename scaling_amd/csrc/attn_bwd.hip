@@ -16,6 +16,8 @@
 // accumulator layout.
 #include "attn_common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int kThreads = 256;
@@ -72,10 +74,12 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     __shared__ __attribute__((aligned(16))) float lse_lds[2][BQ];
     __shared__ __attribute__((aligned(16))) float delta_lds[2][BQ];
     __shared__ int range_lds[16];
-    char* k_t = smem;                     // [2 tiles of 64 keys]
-    char* v_t = smem + 2 * TILE;
-    char* q_t = smem + 4 * TILE;          // [2 stages]
-    char* do_t = smem + 6 * TILE;         // [2 stages]
+    // The streamed tiles come first: with the stage index a compile-time constant (the tile loop is unrolled by two)
+    // their LDS addresses are a per-lane register plus an immediate offset, which reaches 64 KB.
+    char* q_t = smem;                     // [2 stages]
+    char* do_t = smem + 2 * TILE;         // [2 stages]
+    char* k_t = smem + 4 * TILE;          // [2 tiles of 64 keys]
+    char* v_t = smem + 6 * TILE;
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -139,9 +143,9 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk_acc[dt][r] = 0.f; dv_acc[dt][r] = 0.f; }
 
-    // Query tiles are visited from the last one downwards: under a causal mask every key block of a
-    // document needs the document's last queries, so the workgroups that share an XCD start on the same
-    // tile and keep streaming the same Q / dO rows through that XCD's L2.
+    // Query tiles are visited from the last one downwards, the group's query heads innermost: under a causal mask
+    // every key block of a document needs the document's last queries, so the workgroups that share an XCD start on
+    // the same tile and walk down in step, streaming the same Q / dO rows through that XCD's L2 once.
     const int total_iters = n_tiles * hpw;
     const int last_q = p.total_q - 1;
     const __bf16* src_base = q_role ? p.q : p.d_o;
@@ -155,9 +159,9 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     const float stat_scale = (tid < BQ) ? 1.4426950408889634f : 1.0f;
     float stat = 0.f;
     auto tile_of = [&](int iter, int& head, int& qt) {
-        const int rep = iter / n_tiles;
+        const int rep = iter % hpw, tile = iter / hpw;
         head = kvh * p.n_rep + hs * hpw + rep;
-        qt = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ;
+        qt = qt0 + (n_tiles - 1 - tile) * BQ;
     };
     auto issue_tile = [&](int iter) {     // Q / dO tile of iteration `iter` -> stage iter & 1
         int head, qt;
@@ -194,9 +198,9 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
         drop_sel = 8u * (uint32_t)(key & 1);
     }
 
-    for (int iter = 0; iter < total_iters; ++iter) {
-        const int buf = iter & 1;
-        const int qs = qt0 + (n_tiles - 1 - iter % n_tiles) * BQ + 32 * sub;
+    auto tile_step = [&](auto buf_c, int iter) {
+        constexpr int buf = decltype(buf_c)::value;
+        const int qs = qt0 + (n_tiles - 1 - iter / hpw) * BQ + 32 * sub;
         if (iter + 1 < total_iters) issue_tile(iter + 1);
 
         if ((qs < wmax) && (qs + 32 > wmin)) {
@@ -230,7 +234,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             bf16x8_t pl[SPLIT ? 2 : 1], dsl[SPLIT ? 2 : 1];   // accuracy mode: low-order terms of P and dS
             uint32_t drop_xb = 0;
             if constexpr (DROP) {
-                const int head_i = kvh * p.n_rep + hs * hpw + iter / n_tiles;
+                const int head_i = kvh * p.n_rep + hs * hpw + iter % hpw;
                 drop_xb = drop_head_base(p.drop_seed, head_i) + drop_xc + (uint32_t)(qs >> 1) * kDropC1;
             }
 #pragma unroll
@@ -281,6 +285,10 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
         if (iter + 1 < total_iters) store_stat(iter + 1);
         wait_vmcnt<0>();                  // the next Q / dO tile has landed
         __syncthreads();
+    };
+    for (int iter = 0; iter < total_iters; iter += 2) {
+        tile_step(std::integral_constant<int, 0>{}, iter);
+        if (iter + 1 < total_iters) tile_step(std::integral_constant<int, 1>{}, iter + 1);
     }
 
     // ---- sum the two wavefronts of each key group (fixed order), then store -------------------------
