@@ -19,6 +19,10 @@
 
 #include <type_traits>
 
+int mi_attn_validate(const mi_attn_args* a, const char* who);
+void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p);
+int mi_compute_units();
+
 namespace {
 
 constexpr int BN = 64;               // keys per tile
@@ -55,10 +59,23 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: role and phase branches stay uniform
     const int lane = tid & 63, l32 = lane & 31, g = lane >> 5;
 
-    // ---- work item ---------------------------------------------------------------------------
+    // ---- work items --------------------------------------------------------------------------
+    // The grid holds at most one workgroup per compute unit (its LDS rings leave room for no second one) and every
+    // workgroup walks through several (head, query block) items: item lists are cut into passes of gridDim.x items,
+    // heaviest first, and a workgroup takes the items at its own index in even passes and at the mirrored index in
+    // odd ones, so that its heavy and light items add up to the same work as everybody else's (the mirror keeps
+    // index mod 8, i.e. the XCD, so an XCD still sees a fixed set of heads).  This saves the few microseconds it takes
+    // to retire a 128 KB workgroup and dispatch the next one onto the compute unit, once per item.
     const int nqb = (p.total_q + BM - 1) / BM;
+    const int n_items = nqb * p.nq;
+    const int G = gridDim.x;
+    for (int pass = 0; pass * G < n_items; ++pass) {
+    int idx = blockIdx.x;
+    if (pass & 1) idx = (G & 7) == 0 ? ((idx & 7) | (((G >> 3) - 1 - (idx >> 3)) << 3)) : G - 1 - idx;
+    const int item = pass * G + idx;
+    if (item >= n_items) continue;        // the same for the whole workgroup
     int head, q_rank;
-    head_and_rank(blockIdx.x, p.nq, head, q_rank);
+    head_and_rank(item, p.nq, head, q_rank);
     const int kvh = head / p.n_rep;
     const int qb = block_for_rank(q_rank, nqb, p.n_docs, p.across_q, true);   // long query blocks first
 
@@ -425,13 +442,17 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
             p.lse[(int64_t)head * p.total_q + tq] = lse;
         }
     }
+    __syncthreads();                      // the LDS rings and range_lds are free for the next item
+    }   // items
 }
 
 template <int D, int NW, int ROT, bool DROP, bool SPLIT = false> int launch(const AttnParams& p, hipStream_t st) {
     constexpr int BM = 32 * NW;
     const int64_t nqb = ((int64_t)p.total_q + BM - 1) / BM;
-    const int64_t grid = nqb * p.nq;
-    if (grid > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_fwd: grid too large");
+    const int64_t items = nqb * p.nq;
+    if (items > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "attn_fwd: too many work items");
+    const int cus = mi_compute_units();
+    const int64_t grid = items < cus ? items : cus;
     attn_fwd_kernel<D, NW, ROT, DROP, SPLIT><<<dim3((unsigned)grid), dim3(64 * NW), 0, st>>>(p);
     return mi_check_launch("attn_fwd");
 }
@@ -469,9 +490,6 @@ template <int D> int launch_d(const AttnParams& p, int rot, bool q_only, int nw,
 }
 
 }  // namespace
-
-int mi_attn_validate(const mi_attn_args* a, const char* who);
-void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p);
 
 extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     int rc = mi_attn_validate(a, "attn_fwd");
