@@ -39,8 +39,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_delta_kernel(const AttnPara
         const uint4 a = *reinterpret_cast<const uint4*>(p.o + t * p.o_st + (int64_t)h * p.o_sh + 8 * c);
         const uint4 b = *reinterpret_cast<const uint4*>(p.d_o + t * p.o_st + (int64_t)h * p.o_sh + 8 * c);
         float fa[8], fb[8];
-        Elem<__bf16>::unpack(a, fa);
-        Elem<__bf16>::unpack(b, fb);
+        Elem<elem_t>::unpack(a, fa);
+        Elem<elem_t>::unpack(b, fb);
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc += fa[i] * fb[i];
     }
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     {
         DmaPlan<D, IPW> plan;
         plan.init(lw * IPW, lane, q_role ? p.k_st : p.v_st);
-        const __bf16* base = q_role ? p.k + (int64_t)kvh * p.k_sh : p.v + (int64_t)kvh * p.v_sh;
+        const elem_t* base = q_role ? p.k + (int64_t)kvh * p.k_sh : p.v + (int64_t)kvh * p.v_sh;
         const int64_t st = q_role ? p.k_st : p.v_st;
         char* dst = q_role ? k_t : v_t;
 #pragma unroll
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     // the same tile and walk down in step, streaming the same Q / dO rows through that XCD's L2 once.
     const int total_iters = n_tiles * hpw;
     const int last_q = p.total_q - 1;
-    const __bf16* src_base = q_role ? p.q : p.d_o;
+    const elem_t* src_base = q_role ? p.q : p.d_o;
     const int64_t src_head_stride = q_role ? p.q_sh : p.o_sh;
     const int64_t src_tok_stride = q_role ? p.q_st : p.o_st;
     char* dst_tile = q_role ? q_t : do_t;
@@ -212,11 +212,11 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const int ao = a_row ^ (ks << 5), bo = b_row ^ (ks << 5);
-                const bf16x8_t aq = *reinterpret_cast<const bf16x8_t*>(qt_ + ao);
-                const bf16x8_t bk = *reinterpret_cast<const bf16x8_t*>(k_t + bo);
+                const elem8_t aq = *reinterpret_cast<const elem8_t*>(qt_ + ao);
+                const elem8_t bk = *reinterpret_cast<const elem8_t*>(k_t + bo);
                 s_acc = mfma_32x32x16(aq, bk, s_acc);
-                const bf16x8_t ad = *reinterpret_cast<const bf16x8_t*>(dt_ + ao);
-                const bf16x8_t bv = *reinterpret_cast<const bf16x8_t*>(v_t + bo);
+                const elem8_t ad = *reinterpret_cast<const elem8_t*>(dt_ + ao);
+                const elem8_t bv = *reinterpret_cast<const elem8_t*>(v_t + bo);
                 dp_acc = mfma_32x32x16(ad, bv, dp_acc);
             }
             // rows of the accumulators are queries qs + 8a + 4g + c, the column is this lane's key
@@ -230,8 +230,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                     if (rel >= len) s_acc[r] = -INFINITY;
                 }
             }
-            bf16x8_t pf[2], dsf[2];
-            bf16x8_t pl[SPLIT ? 2 : 1], dsl[SPLIT ? 2 : 1];   // accuracy mode: low-order terms of P and dS
+            elem8_t pf[2], dsf[2];
+            elem8_t pl[SPLIT ? 2 : 1], dsl[SPLIT ? 2 : 1];   // accuracy mode: low-order terms of P and dS
             uint32_t drop_xb = 0;
             if constexpr (DROP) {
                 const int head_i = kvh * p.n_rep + hs * hpw + iter % hpw;
@@ -258,11 +258,11 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                     const float dpv = DROP ? (keep[c] ? dp_acc[r] * p.drop_rscale : 0.f) : dp_acc[r];
                     const float ds = pv * (dpv - d4[c]);
                     const float pk = (DROP && !keep[c]) ? 0.f : pv;
-                    pf[a >> 1][4 * (a & 1) + c] = (__bf16)pk;
-                    dsf[a >> 1][4 * (a & 1) + c] = (__bf16)ds;
+                    pf[a >> 1][4 * (a & 1) + c] = (elem_t)pk;
+                    dsf[a >> 1][4 * (a & 1) + c] = (elem_t)ds;
                     if constexpr (SPLIT) {
-                        pl[a >> 1][4 * (a & 1) + c] = (__bf16)(pk - (float)pf[a >> 1][4 * (a & 1) + c]);
-                        dsl[a >> 1][4 * (a & 1) + c] = (__bf16)(ds - (float)dsf[a >> 1][4 * (a & 1) + c]);
+                        pl[a >> 1][4 * (a & 1) + c] = (elem_t)(pk - (float)pf[a >> 1][4 * (a & 1) + c]);
+                        dsl[a >> 1][4 * (a & 1) + c] = (elem_t)(ds - (float)dsf[a >> 1][4 * (a & 1) + c]);
                     }
                 }
             }
@@ -271,8 +271,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
                     const int o0 = (tr_h0 ^ (dt << 6)) + 16 * m * RB, o1 = (tr_h1 ^ (dt << 6)) + 16 * m * RB;
-                    const bf16x8_t adt = tr_pair(dt_ + o0, dt_ + o1);
-                    const bf16x8_t aqt = tr_pair(qt_ + o0, qt_ + o1);
+                    const elem8_t adt = tr_pair(dt_ + o0, dt_ + o1);
+                    const elem8_t aqt = tr_pair(qt_ + o0, qt_ + o1);
                     dv_acc[dt] = mfma_32x32x16(adt, pf[m], dv_acc[dt]);
                     dk_acc[dt] = mfma_32x32x16(aqt, dsf[m], dk_acc[dt]);
                     if constexpr (SPLIT) {
@@ -333,18 +333,18 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
         if constexpr (D == 64 || D == 128) {
             if (p.unrotate != 0) unrotate_acc<D>(dk_acc, p, p.pos_k[key], g);   // k was the rotated tensor
         }
-        __bf16* dkr = p.dk + (int64_t)key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * g;
-        __bf16* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
+        elem_t* dkr = p.dk + (int64_t)key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * g;
+        elem_t* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const uint32_t k0 = pack_bf16x2(dk_acc[dt][4 * a], dk_acc[dt][4 * a + 1]);
-                const uint32_t k1 = pack_bf16x2(dk_acc[dt][4 * a + 2], dk_acc[dt][4 * a + 3]);
+                const uint32_t k0 = pack_elem2(dk_acc[dt][4 * a], dk_acc[dt][4 * a + 1]);
+                const uint32_t k1 = pack_elem2(dk_acc[dt][4 * a + 2], dk_acc[dt][4 * a + 3]);
                 *reinterpret_cast<uint2*>(dkr + 32 * dt + 8 * a) = make_uint2(k0, k1);
                 const float vs = DROP ? p.drop_rscale : 1.0f;   // dV = (P * mask / (1 - p))^T dO
-                const uint32_t v0 = pack_bf16x2(dv_acc[dt][4 * a] * vs, dv_acc[dt][4 * a + 1] * vs);
-                const uint32_t v1 = pack_bf16x2(dv_acc[dt][4 * a + 2] * vs, dv_acc[dt][4 * a + 3] * vs);
+                const uint32_t v0 = pack_elem2(dv_acc[dt][4 * a] * vs, dv_acc[dt][4 * a + 1] * vs);
+                const uint32_t v1 = pack_elem2(dv_acc[dt][4 * a + 2] * vs, dv_acc[dt][4 * a + 3] * vs);
                 *reinterpret_cast<uint2*>(dvr + 32 * dt + 8 * a) = make_uint2(v0, v1);
             }
     }
@@ -401,9 +401,9 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_reduce_kernel(const At
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         *reinterpret_cast<uint2*>(p.dk + key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * c + h * (D / 2)) =
-            make_uint2(pack_bf16x2(k4[h][0], k4[h][1]), pack_bf16x2(k4[h][2], k4[h][3]));
+            make_uint2(pack_elem2(k4[h][0], k4[h][1]), pack_elem2(k4[h][2], k4[h][3]));
         *reinterpret_cast<uint2*>(p.dv + key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * c + h * (D / 2)) =
-            make_uint2(pack_bf16x2(v4[h][0], v4[h][1]), pack_bf16x2(v4[h][2], v4[h][3]));
+            make_uint2(pack_elem2(v4[h][0], v4[h][1]), pack_elem2(v4[h][2], v4[h][3]));
     }
 }
 
@@ -451,14 +451,14 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     if (lane == 0) { range_lds[wave] = wmin; range_lds[8 + wave] = wmax; }
 
     const int tl = tq < p.total_q ? tq : p.total_q - 1;
-    bf16x8_t qf[KS], dof[KS];
+    elem8_t qf[KS], dof[KS];
     {
-        const __bf16* qr = p.q + (int64_t)tl * p.q_st + (int64_t)head * p.q_sh + 8 * g;
-        const __bf16* dr = p.d_o + (int64_t)tl * p.o_st + (int64_t)head * p.o_sh + 8 * g;
+        const elem_t* qr = p.q + (int64_t)tl * p.q_st + (int64_t)head * p.q_sh + 8 * g;
+        const elem_t* dr = p.d_o + (int64_t)tl * p.o_st + (int64_t)head * p.o_sh + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            qf[ks] = *reinterpret_cast<const bf16x8_t*>(qr + 16 * ks);
-            dof[ks] = *reinterpret_cast<const bf16x8_t*>(dr + 16 * ks);
+            qf[ks] = *reinterpret_cast<const elem8_t*>(qr + 16 * ks);
+            dof[ks] = *reinterpret_cast<const elem8_t*>(dr + 16 * ks);
         }
     }
     const float lse_nat = p.lse[(int64_t)head * p.total_q + tl];
@@ -488,7 +488,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     // stage whose readers passed the previous barrier
     const bool k_role = wave < 4;
     const int lw = wave & 3;
-    const __bf16* src_base = k_role ? p.k + (int64_t)kvh * p.k_sh : p.v + (int64_t)kvh * p.v_sh;
+    const elem_t* src_base = k_role ? p.k + (int64_t)kvh * p.k_sh : p.v + (int64_t)kvh * p.v_sh;
     const int64_t src_tok_stride = k_role ? p.k_st : p.v_st;
     char* dst_ring = k_role ? k_t : v_t;
     const int last_k = p.total_k - 1;
@@ -529,9 +529,9 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                 const int ao = a_row ^ (ks << 5);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const bf16x8_t ak = *reinterpret_cast<const bf16x8_t*>(kt_ + ao + 32 * t * RB);
+                    const elem8_t ak = *reinterpret_cast<const elem8_t*>(kt_ + ao + 32 * t * RB);
                     s_acc[t] = mfma_32x32x16(ak, qf[ks], s_acc[t]);
-                    const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(vt_ + ao + 32 * t * RB);
+                    const elem8_t av = *reinterpret_cast<const elem8_t*>(vt_ + ao + 32 * t * RB);
                     dp_acc[t] = mfma_32x32x16(av, dof[ks], dp_acc[t]);
                 }
             }
@@ -550,7 +550,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
                 const int t = m >> 1, r0 = 8 * (m & 1);
-                bf16x8_t dsf, dsl;
+                elem8_t dsf, dsl;
                 if constexpr (DROP) {
                     // dP of a dropped probability is zero, that of a kept one carries the 1 / (1 - p) scale
                     const uint32_t drop_xt = drop_xr + (uint32_t)(kt >> 1) * kDropC2;
@@ -567,13 +567,13 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                 for (int e = 0; e < 8; ++e) {
                     const float pv = fast_exp2(s_acc[t][r0 + e] * c2 - lse2);
                     const float ds = pv * (dp_acc[t][r0 + e] - delta);
-                    dsf[e] = (__bf16)ds;
-                    if constexpr (SPLIT) dsl[e] = (__bf16)(ds - (float)dsf[e]);
+                    dsf[e] = (elem_t)ds;
+                    if constexpr (SPLIT) dsl[e] = (elem_t)(ds - (float)dsf[e]);
                 }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
                     const int o0 = (tr_h0 ^ (dt << 6)) + 16 * m * RB, o1 = (tr_h1 ^ (dt << 6)) + 16 * m * RB;
-                    const bf16x8_t akt = tr_pair(kt_ + o0, kt_ + o1);
+                    const elem8_t akt = tr_pair(kt_ + o0, kt_ + o1);
                     dq_acc[dt] = mfma_32x32x16(akt, dsf, dq_acc[dt]);
                     if constexpr (SPLIT) dq_acc[dt] = mfma_32x32x16(akt, dsl, dq_acc[dt]);
                 }
@@ -593,13 +593,13 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
             // q was the rotated tensor: the gradient of the unrotated one is the row rotated back (rotary.py:117-139)
             if (p.unrotate != 0) unrotate_acc<D>(dq_acc, p, p.pos_q[tq], g);
         }
-        __bf16* dqr = p.dq + (int64_t)tq * p.q_st + (int64_t)head * p.q_sh + 4 * g;
+        elem_t* dqr = p.dq + (int64_t)tq * p.q_st + (int64_t)head * p.q_sh + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const uint32_t w0 = pack_bf16x2(dq_acc[dt][4 * a], dq_acc[dt][4 * a + 1]);
-                const uint32_t w1 = pack_bf16x2(dq_acc[dt][4 * a + 2], dq_acc[dt][4 * a + 3]);
+                const uint32_t w0 = pack_elem2(dq_acc[dt][4 * a], dq_acc[dt][4 * a + 1]);
+                const uint32_t w1 = pack_elem2(dq_acc[dt][4 * a + 2], dq_acc[dt][4 * a + 3]);
                 *reinterpret_cast<uint2*>(dqr + 32 * dt + 8 * a) = make_uint2(w0, w1);
             }
     }
@@ -643,14 +643,15 @@ template <int D> int launch_bwd(const AttnParams& p, int flags, hipStream_t st) 
 
 }  // namespace
 
-int mi_attn_validate(const mi_attn_args* a, const char* who);
-void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p);
-
+#ifndef MI_ELEM_F16
 extern "C" size_t mi_attn_bwd_workspace_bytes(int64_t total_q, int32_t n_q_heads, int32_t head_dim) {
     (void)head_dim;
     if (total_q <= 0 || n_q_heads <= 0) return 0;
     return (size_t)total_q * (size_t)n_q_heads * sizeof(float);
 }
+#else
+extern "C" size_t mi_attn_bwd_workspace_bytes(int64_t total_q, int32_t n_q_heads, int32_t head_dim);
+#endif
 
 namespace {
 // query-head split of the dK/dV launch: enough workgroup groups for the 8 XCDs when there are fewer than 8 KV heads
@@ -663,6 +664,7 @@ int dkdv_head_split(int nq, int nkv) {
 size_t delta_bytes_aligned(int64_t total_q, int nq) { return ((size_t)total_q * (size_t)nq * sizeof(float) + 255) & ~(size_t)255; }
 }  // namespace
 
+#ifndef MI_ELEM_F16
 extern "C" size_t mi_attn_bwd_workspace_bytes_kv(int64_t total_q, int64_t total_k, int32_t n_q_heads, int32_t n_kv_heads,
                                                  int32_t head_dim) {
     if (total_q <= 0 || total_k <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0 || head_dim <= 0)
@@ -671,8 +673,9 @@ extern "C" size_t mi_attn_bwd_workspace_bytes_kv(int64_t total_q, int64_t total_
     if (h == 1) return mi_attn_bwd_workspace_bytes(total_q, n_q_heads, head_dim);
     return delta_bytes_aligned(total_q, n_q_heads) + (size_t)2 * h * (size_t)total_k * n_kv_heads * head_dim * sizeof(float);
 }
+#endif
 
-extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
+int MI_ENTRY(mi_attn_bwd_impl)(const mi_attn_bwd_args* b) {
     if (!b) return mi_fail(MI_E_NULL, "attn_bwd: args is null");
     const mi_attn_args* a = &b->fwd;
     int rc = mi_attn_validate(a, "attn_bwd");
@@ -692,7 +695,7 @@ extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
         return mi_fail(MI_E_WORKSPACE, "attn_bwd: workspace needs %zu bytes (16-byte aligned), got %zu", need, b->workspace_bytes);
     AttnParams p;
     mi_attn_fill_params(a, &p);
-    p.d_o = (const __bf16*)b->d_o; p.dq = (__bf16*)b->dq; p.dk = (__bf16*)b->dk; p.dv = (__bf16*)b->dv;
+    p.d_o = (const elem_t*)b->d_o; p.dq = (elem_t*)b->dq; p.dk = (elem_t*)b->dk; p.dv = (elem_t*)b->dv;
     p.dk_st = b->dk_stride_token; p.dk_sh = b->dk_stride_head;
     p.dv_st = b->dv_stride_token; p.dv_sh = b->dv_stride_head;
     p.delta = (float*)b->workspace;

@@ -13,18 +13,35 @@
 #pragma once
 #include "common.h"
 
+// Element type of q / k / v / o and of every MFMA operand.  Each attention source file is compiled twice: as is for
+// bfloat16 and with MI_ELEM_F16 for float16 (half-precision MFMA, same tilings); the bfloat16 objects export the C
+// entry points and hand float16 calls to the MI_ENTRY(...)-named functions of the float16 objects.
+#ifdef MI_ELEM_F16
+typedef _Float16 elem_t;
+typedef _Float16 elem2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 elem4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 elem8_t __attribute__((ext_vector_type(8)));
+#define MI_ELEM_DTYPE MI_F16
+#else
+typedef __bf16 elem_t;
+typedef bf16x2_t elem2_t;
+typedef bf16x4_t elem4_t;
+typedef bf16x8_t elem8_t;
+#define MI_ELEM_DTYPE MI_BF16
+#endif
+
 struct AttnParams {
-    const __bf16* q; const __bf16* k; const __bf16* v; __bf16* o; float* lse;
+    const elem_t* q; const elem_t* k; const elem_t* v; elem_t* o; float* lse;
     const int32_t* cu_q; const int32_t* cu_k;
     int n_docs; int causal;
     int total_q; int total_k;
     int nq; int nkv; int n_rep;
     int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;
     float scale_log2;   // softmax_scale * log2(e)
-    const __bf16* cos; const __bf16* sin; const int64_t* pos_q; const int64_t* pos_k; int table_rows;
+    const elem_t* cos; const elem_t* sin; const int64_t* pos_q; const int64_t* pos_k; int table_rows;
     const float* cos32; const float* sin32;   // interleaved-pair rotary: fp32 tables [table_rows, head_dim / 2]
     // backward only
-    const __bf16* d_o; __bf16* dq; __bf16* dk; __bf16* dv; float* delta;
+    const elem_t* d_o; elem_t* dq; elem_t* dk; elem_t* dv; float* delta;
     int64_t dk_st, dk_sh, dv_st, dv_sh;
     float scale;        // softmax_scale
     // dropout on the attention probabilities (0 = off): an element is dropped iff its random byte < drop_thr,
@@ -37,7 +54,7 @@ struct AttnParams {
     // each writing fp32 partial sums [hsplit][total_k][nkv][head_dim] that a reduce launch adds up (1 = no split)
     int hsplit; float* dk_part; float* dv_part;
     // forward: optional copy of the rotated q (fused rotary), same strides as q
-    __bf16* q_rot;
+    elem_t* q_rot;
     // backward with rotary: q / k are the rotated tensors; dq / dk leave the kernels rotated back (0 = no rotary,
     // 1 = rotate-half with tables in the I/O dtype, 2 = interleaved pairs with fp32 tables)
     int unrotate;
@@ -66,8 +83,12 @@ __device__ __forceinline__ uint32_t drop_head_base(uint32_t seed, int head) {
 // byte `field` (0..3) of the block hash
 __device__ __forceinline__ uint32_t drop_byte(uint32_t h, uint32_t shift) { return __builtin_amdgcn_ubfe(h, shift, 8); }
 
-__device__ __forceinline__ f32x16_t mfma_32x32x16(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+__device__ __forceinline__ f32x16_t mfma_32x32x16(elem8_t a, elem8_t b, f32x16_t c) {
+#ifdef MI_ELEM_F16
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#else
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#endif
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -134,11 +155,11 @@ __device__ __forceinline__ v4i16_t lds_read_tr16_b64(const void* p) {
 // 16m + 4g + {0..3} (first transpose read) and 16m + 8 + 4g + {0..3} (second).
 typedef short v8i16_t __attribute__((ext_vector_type(8)));
 
-__device__ __forceinline__ bf16x8_t tr_pair(const char* lo_addr, const char* hi_addr) {
+__device__ __forceinline__ elem8_t tr_pair(const char* lo_addr, const char* hi_addr) {
     const v4i16_t lo = lds_read_tr16_b64(lo_addr);
     const v4i16_t hi = lds_read_tr16_b64(hi_addr);
     const v8i16_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8_t, both);
+    return __builtin_bit_cast(elem8_t, both);
 }
 
 // ---- token-major LDS tile filled by direct global -> LDS loads ------------------------------------------
@@ -219,15 +240,15 @@ template <int D, int COUNT> struct DmaPlan {
     }
     // All COUNT instructions of the tile whose first token is tok0, straight-line when the tile is full.
     // tile: wave-uniform LDS address of the stage; base + tok0 * tok_stride must be wave-uniform too.
-    __device__ __forceinline__ void issue(const __bf16* base, int64_t tok_stride, int tok0, int last_tok, char* tile) const {
+    __device__ __forceinline__ void issue(const elem_t* base, int64_t tok_stride, int tok0, int last_tok, char* tile) const {
         char* dst = tile + 1024 * n0;
         if (tok0 + 63 <= last_tok) {
-            const __bf16* tile_base = base + (int64_t)tok0 * tok_stride;
+            const elem_t* tile_base = base + (int64_t)tok0 * tok_stride;
 #pragma unroll
             for (int j = 0; j < COUNT; ++j) issue_one(off[j], tile_base, dst + 1024 * j);
         } else {
             const int first = min(tok0, last_tok);            // the lane offsets below must not be negative
-            const __bf16* tile_base = base + (int64_t)first * tok_stride;
+            const elem_t* tile_base = base + (int64_t)first * tok_stride;
             int l = lane;
             asm volatile("" : "+v"(l));   // opaque: keeps this rarely used arithmetic from being hoisted out of the caller's loop
 #pragma unroll
@@ -281,15 +302,20 @@ __device__ __forceinline__ void st128(void* p, const uint4& x) {
     *reinterpret_cast<u32x4_t*>(p) = v;
 }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    bf16x2_t p;
-    p[0] = (__bf16)lo;
-    p[1] = (__bf16)hi;
+__device__ __forceinline__ uint32_t pack_elem2(float lo, float hi) {
+    elem2_t p;
+    p[0] = (elem_t)lo;
+    p[1] = (elem_t)hi;
     return __builtin_bit_cast(uint32_t, p);
 }
 
-__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+#ifdef MI_ELEM_F16
+__device__ __forceinline__ float elem_lo(uint32_t w) { return (float)__builtin_bit_cast(elem2_t, w)[0]; }
+__device__ __forceinline__ float elem_hi(uint32_t w) { return (float)__builtin_bit_cast(elem2_t, w)[1]; }
+#else
+__device__ __forceinline__ float elem_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float elem_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+#endif
 
 // rotate-half rotary applied to a (first-half, second-half) pair of 8-element vectors; cos/sin hold
 // the table values of the first-half columns (both table halves are equal by construction)
@@ -300,12 +326,12 @@ __device__ __forceinline__ void rotate_pair(uint4& lo, uint4& hi, const uint4& c
     const uint32_t* sw = reinterpret_cast<const uint32_t*>(&s);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float x0a = bf16_lo(l[i]), x0b = bf16_hi(l[i]);
-        const float x1a = bf16_lo(h[i]), x1b = bf16_hi(h[i]);
-        const float ca = bf16_lo(cw[i]), cb = bf16_hi(cw[i]);
-        const float sa = sign * bf16_lo(sw[i]), sb = sign * bf16_hi(sw[i]);
-        l[i] = pack_bf16x2(x0a * ca - x1a * sa, x0b * cb - x1b * sb);
-        h[i] = pack_bf16x2(x1a * ca + x0a * sa, x1b * cb + x0b * sb);
+        const float x0a = elem_lo(l[i]), x0b = elem_hi(l[i]);
+        const float x1a = elem_lo(h[i]), x1b = elem_hi(h[i]);
+        const float ca = elem_lo(cw[i]), cb = elem_hi(cw[i]);
+        const float sa = sign * elem_lo(sw[i]), sb = sign * elem_hi(sw[i]);
+        l[i] = pack_elem2(x0a * ca - x1a * sa, x0b * cb - x1b * sb);
+        h[i] = pack_elem2(x1a * ca + x0a * sa, x1b * cb + x0b * sb);
     }
 }
 
@@ -316,9 +342,9 @@ __device__ __forceinline__ void rotate_interleaved(uint4& v, const uint4& c, con
     const uint32_t* sw = reinterpret_cast<const uint32_t*>(&s);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float x0 = bf16_lo(w[i]), x1 = bf16_hi(w[i]);
+        float x0 = elem_lo(w[i]), x1 = elem_hi(w[i]);
         rotate_complex_pair(x0, x1, __uint_as_float(cw[i]), sign * __uint_as_float(sw[i]));
-        w[i] = pack_bf16x2(x0, x1);
+        w[i] = pack_elem2(x0, x1);
     }
 }
 
@@ -332,16 +358,16 @@ __device__ __forceinline__ void unrotate_acc(f32x16_t (&acc)[D / 32], const Attn
     constexpr int DT = D / 32;
     pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
     if (p.unrotate == 1) {
-        const __bf16* cr = p.cos + pos * D + 4 * g;
-        const __bf16* sr = p.sin + pos * D + 4 * g;
+        const elem_t* cr = p.cos + pos * D + 4 * g;
+        const elem_t* sr = p.sin + pos * D + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT / 2; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 const uint2 cw = *reinterpret_cast<const uint2*>(cr + 32 * dt + 8 * a);
                 const uint2 sw = *reinterpret_cast<const uint2*>(sr + 32 * dt + 8 * a);
-                const float c4[4] = {bf16_lo(cw.x), bf16_hi(cw.x), bf16_lo(cw.y), bf16_hi(cw.y)};
-                const float s4[4] = {bf16_lo(sw.x), bf16_hi(sw.x), bf16_lo(sw.y), bf16_hi(sw.y)};
+                const float c4[4] = {elem_lo(cw.x), elem_hi(cw.x), elem_lo(cw.y), elem_hi(cw.y)};
+                const float s4[4] = {elem_lo(sw.x), elem_hi(sw.x), elem_lo(sw.y), elem_hi(sw.y)};
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const float x0 = acc[dt][4 * a + c], x1 = acc[dt + DT / 2][4 * a + c];
@@ -412,3 +438,71 @@ __device__ __forceinline__ int xcd_remap(int linear, int total) {
     if ((total & 7) != 0) return linear;
     return (linear & 7) * (total >> 3) + (linear >> 3);
 }
+
+// ---- host side: argument checking and parameter block shared by the attention entry points -----------------
+#ifdef MI_ELEM_F16
+#define MI_ENTRY(name) name##_f16
+#else
+#define MI_ENTRY(name) name##_bf16
+#endif
+int mi_compute_units();
+int mi_static_scratch(void** out, size_t* bytes);
+
+static inline int mi_attn_validate(const mi_attn_args* a, const char* who) {
+    if (!a) return mi_fail(MI_E_NULL, "%s: args is null", who);
+    if (!a->q || !a->k || !a->v || !a->cu_seqlens_q) return mi_fail(MI_E_NULL, "%s: q, k, v and cu_seqlens_q are required", who);
+    if (a->dtype != MI_ELEM_DTYPE) return mi_fail(MI_E_DTYPE, "%s: the attention kernels take bf16 or f16 tensors (dtype code %d)", who, a->dtype);
+    if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 96 && a->head_dim != 128)
+        return mi_fail(MI_E_SHAPE, "%s: head_dim %d unsupported (32, 64, 96, 128)", who, a->head_dim);
+    if (a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0)
+        return mi_fail(MI_E_SHAPE, "%s: n_q_heads=%d must be a positive multiple of n_kv_heads=%d", who, a->n_q_heads, a->n_kv_heads);
+    if (a->total_q < 0 || a->total_k < 0 || a->total_q > 0x7fffffffLL || a->total_k > 0x7fffffffLL || a->n_docs < 0)
+        return mi_fail(MI_E_SHAPE, "%s: bad token counts q=%lld k=%lld docs=%d", who, (long long)a->total_q, (long long)a->total_k, a->n_docs);
+    if (a->total_q > 0 && (a->n_docs < 1 || a->total_k < 1))
+        return mi_fail(MI_E_SHAPE, "%s: non-empty query needs at least one document and one key", who);
+    if (!mi_aligned16(a->q) || !mi_aligned16(a->k) || !mi_aligned16(a->v))
+        return mi_fail(MI_E_ALIGN, "%s: q, k, v must be 16-byte aligned", who);
+    if (a->q_stride_token % 8 || a->q_stride_head % 8 || a->k_stride_token % 8 || a->k_stride_head % 8 ||
+        a->v_stride_token % 8 || a->v_stride_head % 8)
+        return mi_fail(MI_E_ALIGN, "%s: strides must be multiples of 8 elements", who);
+    if (!(a->softmax_scale > 0.f)) return mi_fail(MI_E_SHAPE, "%s: softmax_scale must be positive", who);
+    if (a->rotary_cos || a->rotary_sin) {
+        if (!a->rotary_cos || !a->rotary_sin || !a->position_ids_q)
+            return mi_fail(MI_E_NULL, "%s: fused rotary needs cos, sin and the query position ids", who);
+        if (a->head_dim != 64 && a->head_dim != 128) return mi_fail(MI_E_SHAPE, "%s: fused rotary needs head_dim 64 or 128", who);
+        if (a->rotary_table_rows <= 0 || a->rotary_table_rows > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "%s: bad rotary table size", who);
+        if (!mi_aligned16(a->rotary_cos) || !mi_aligned16(a->rotary_sin)) return mi_fail(MI_E_ALIGN, "%s: rotary tables must be 16-byte aligned", who);
+    }
+    if (!(a->dropout_p >= 0.f) || a->dropout_p >= 1.f) return mi_fail(MI_E_SHAPE, "%s: dropout_p must be in [0, 1)", who);
+    return MI_OK;
+}
+
+static inline void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p) {
+    *p = AttnParams{};
+    p->q = (const elem_t*)a->q; p->k = (const elem_t*)a->k; p->v = (const elem_t*)a->v;
+    p->o = (elem_t*)a->o; p->lse = a->lse;
+    p->cu_q = a->cu_seqlens_q; p->cu_k = a->cu_seqlens_k ? a->cu_seqlens_k : a->cu_seqlens_q;
+    p->n_docs = a->n_docs; p->causal = a->causal;
+    p->total_q = (int)a->total_q; p->total_k = (int)a->total_k;
+    p->nq = a->n_q_heads; p->nkv = a->n_kv_heads; p->n_rep = a->n_q_heads / a->n_kv_heads;
+    p->q_st = a->q_stride_token; p->q_sh = a->q_stride_head;
+    p->k_st = a->k_stride_token; p->k_sh = a->k_stride_head;
+    p->v_st = a->v_stride_token; p->v_sh = a->v_stride_head;
+    p->o_st = a->o_stride_token; p->o_sh = a->o_stride_head;
+    p->scale = a->softmax_scale;
+    p->scale_log2 = a->softmax_scale * 1.4426950408889634f;
+    if (a->rotary_interleaved) {
+        p->cos32 = (const float*)a->rotary_cos; p->sin32 = (const float*)a->rotary_sin;
+    } else {
+        p->cos = (const elem_t*)a->rotary_cos; p->sin = (const elem_t*)a->rotary_sin;
+    }
+    p->pos_q = a->position_ids_q; p->pos_k = a->position_ids_k; p->table_rows = (int)a->rotary_table_rows;
+    if (a->dropout_p > 0.f) {
+        int t = (int)(a->dropout_p * 256.0f + 0.5f);
+        t = t < 1 ? 1 : (t > 255 ? 255 : t);
+        p->drop_thr = (uint32_t)t;
+        p->drop_rscale = 256.0f / (float)(256 - t);
+        p->drop_seed = (uint32_t)(a->dropout_seed & 0xffffffffu) ^ (uint32_t)(a->dropout_seed >> 32);
+    }
+}
+

@@ -12,8 +12,6 @@
 // applies rotary to it; the query is rotated while its fragments are loaded.
 #include "attn_common.h"
 
-#include <mutex>
-
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 namespace {
@@ -22,10 +20,10 @@ constexpr int kChunk = 32;           // keys per wavefront and iteration
 constexpr int kMaxSplits = 32;
 
 struct DecodeParams {
-    const __bf16* q; __bf16* kc; __bf16* vc; __bf16* o;
+    const elem_t* q; elem_t* kc; elem_t* vc; elem_t* o;
     const int32_t* ctx_len;
-    const __bf16* k_new; const __bf16* v_new;
-    const __bf16* cos; const __bf16* sin; const int64_t* pos; int table_rows;
+    const elem_t* k_new; const elem_t* v_new;
+    const elem_t* cos; const elem_t* sin; const int64_t* pos; int table_rows;
     const float* cos32; const float* sin32;   // interleaved-pair rotary: fp32 tables [table_rows, D / 2]
     int batch, max_ctx, nq, nkv, n_rep, n_splits;
     int n_hc;      // chunks of up to 16 query heads per KV head (a workgroup serves one chunk)
@@ -36,8 +34,12 @@ struct DecodeParams {
     float* ws_ml;  // [batch][nq][n_splits][2]
 };
 
-__device__ __forceinline__ f32x4v mfma_16x16x32(bf16x8_t a, bf16x8_t b, f32x4v c) {
+__device__ __forceinline__ f32x4v mfma_16x16x32(elem8_t a, elem8_t b, f32x4v c) {
+#ifdef MI_ELEM_F16
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+#else
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+#endif
 }
 
 // ---- in-place append of the new K/V row (optionally rotated) -------------------------------------
@@ -115,10 +117,10 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     const int n_iter = s1 > s0 ? (s1 - s0 + NWV * kChunk - 1) / (NWV * kChunk) : 0;
 
     // Q^T fragments: column = head slot l16 (valid when < n_rep), contraction = features 32*ks + 8*G + i
-    bf16x8_t qf[KS];
+    elem8_t qf[KS];
     {
         const int hs = l16 < n_heads ? l16 : 0;
-        const __bf16* qr = p.q + (int64_t)b * p.q_sb + (int64_t)(head0 + hs) * D + 8 * G;
+        const elem_t* qr = p.q + (int64_t)b * p.q_sb + (int64_t)(head0 + hs) * D + 8 * G;
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qr + 32 * ks);
@@ -144,7 +146,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             if (l16 >= n_heads) raw[ks] = make_uint4(0, 0, 0, 0);
-            qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
+            qf[ks] = __builtin_bit_cast(elem8_t, raw[ks]);
         }
     }
 
@@ -153,8 +155,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     for (int dt = 0; dt < DT; ++dt) o_acc[dt] = f32x4v{0.f, 0.f, 0.f, 0.f};
     float m_i = -INFINITY, l_i = 0.f;
 
-    const __bf16* kbase = p.kc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
-    const __bf16* vbase = p.vc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
+    const elem_t* kbase = p.kc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
+    const elem_t* vbase = p.vc + (int64_t)b * p.c_sb + (int64_t)kvh * p.c_sh;
     char* vt = v_lds[wave];
     // transpose-read base of this lane: keys 4G + (l16 >> 2), features 4 * (l16 & 3) (+ 16 per feature tile, + 16 keys for the second half)
     const char* vt_lane = vt + (4 * G + (l16 >> 2)) * VSTR + 8 * (l16 & 3);
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     // K fragments and V rows of a chunk; two sets so that the loads of chunk i+1 are in flight while
     // chunk i is being processed
     struct ChunkRegs {
-        bf16x8_t kf[2][KS];
+        elem8_t kf[2][KS];
         uint4 vraw[V_PER_LANE][4];
     };
     auto load_chunk = [&](ChunkRegs& c, int it) {
@@ -172,9 +174,9 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int tok = min(key0 + 16 * t + l16, last);
-            const __bf16* kr = kbase + (int64_t)tok * p.c_st + 8 * G;
+            const elem_t* kr = kbase + (int64_t)tok * p.c_st + 8 * G;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) c.kf[t][ks] = __builtin_bit_cast(bf16x8_t, ldg_nt(reinterpret_cast<const uint4*>(kr + 32 * ks)));
+            for (int ks = 0; ks < KS; ++ks) c.kf[t][ks] = __builtin_bit_cast(elem8_t, ldg_nt(reinterpret_cast<const uint4*>(kr + 32 * ks)));
         }
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
         // order, so wavefront-scope fences (compiler ordering only) are enough and the wavefronts of a
         // workgroup never wait for each other inside the loop.
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        bf16x8_t pf;
+        elem8_t pf;
         float alpha = 1.f;
         if (active) {
             f32x4v s_acc[2];
@@ -226,7 +228,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
                 for (int r = 0; r < 4; ++r) {
                     const float e = fast_exp2(s_acc[t][r] * p.scale_log2 - m_new);
                     rs += e;
-                    pf[4 * t + r] = (__bf16)e;   // slot (G, i): key 16*(i/4) + 4*G + (i%4)
+                    pf[4 * t + r] = (elem_t)e;   // slot (G, i): key 16*(i/4) + 4*G + (i%4)
                 }
             l_i = l_i * alpha + rs;
             // key-major copy of the V chunk (rows as loaded); the PV operand is read back transposed
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 // slots 0-3: keys 4G..4G+3, slots 4-7: keys 16+4G..16+4G+3 (the order of pf)
-                const bf16x8_t a = tr_pair(vt_lane + 32 * dt, vt_lane + 16 * VSTR + 32 * dt);
+                const elem8_t a = tr_pair(vt_lane + 32 * dt, vt_lane + 16 * VSTR + 32 * dt);
                 o_acc[dt] = o_acc[dt] * alpha;
                 o_acc[dt] = mfma_16x16x32(a, pf, o_acc[dt]);
             }
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
         }
         const int64_t bh = (int64_t)b * p.nq + head0 + hs;
         if (p.n_splits == 1) {
-            p.o[bh * D + d] = (__bf16)(L > 0.f ? O / L : 0.f);
+            p.o[bh * D + d] = (elem_t)(L > 0.f ? O / L : 0.f);
         } else {
             const int64_t slot = bh * p.n_splits + split;
             p.ws_o[slot * D + d] = O;
@@ -315,7 +317,7 @@ __global__ void decode_merge_kernel(const DecodeParams p) {
         L += f * p.ws_ml[(bh * p.n_splits + s) * 2 + 1];
         O += f * p.ws_o[(bh * p.n_splits + s) * D + d];
     }
-    p.o[bh * D + d] = (__bf16)(L > 0.f ? O / L : 0.f);
+    p.o[bh * D + d] = (elem_t)(L > 0.f ? O / L : 0.f);
 }
 
 // 8-wavefront workgroups (one per compute unit) once there is a (batch, KV head) pair for most of the 256
@@ -364,11 +366,13 @@ template <int D> int launch_decode(const DecodeParams& p, bool append, int rot, 
 
 }  // namespace
 
+#ifndef MI_ELEM_F16
 extern "C" size_t mi_attn_decode_workspace_bytes(int32_t batch, int32_t n_q_heads, int32_t head_dim, int32_t max_ctx) {
     (void)max_ctx;
     if (batch <= 0 || n_q_heads <= 0 || head_dim <= 0) return 0;
     return (size_t)batch * n_q_heads * kMaxSplits * (size_t)(head_dim + 2) * sizeof(float);
 }
+#endif
 
 namespace {
 // Validation and launches shared by the two entry points; `ws` / `ws_bytes` is the scratch for the per-split partial
@@ -376,7 +380,7 @@ namespace {
 int decode_entry(const mi_decode_args* a, void* ws, size_t ws_bytes, bool static_ws) {
     if (!a) return mi_fail(MI_E_NULL, "attn_decode: args is null");
     if (!a->q || !a->k_cache || !a->v_cache || !a->o || !a->ctx_len) return mi_fail(MI_E_NULL, "attn_decode: q, caches, o and ctx_len are required");
-    if (a->dtype != MI_BF16) return mi_fail(MI_E_DTYPE, "attn_decode: only bf16 is supported");
+    if (a->dtype != MI_ELEM_DTYPE) return mi_fail(MI_E_DTYPE, "attn_decode: the decode kernels take bf16 or f16 tensors (dtype code %d)", a->dtype);
     if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 96 && a->head_dim != 128)
         return mi_fail(MI_E_SHAPE, "attn_decode: head_dim %d unsupported (32, 64, 96, 128)", a->head_dim);
     if (a->batch <= 0 || a->max_ctx <= 0 || a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0)
@@ -410,12 +414,12 @@ int decode_entry(const mi_decode_args* a, void* ws, size_t ws_bytes, bool static
     if (!ws || ws_bytes < need || !mi_aligned16(ws))
         return mi_fail(MI_E_WORKSPACE, "attn_decode: workspace needs %zu bytes (16-byte aligned), got %zu", need, ws_bytes);
     DecodeParams p{};
-    p.q = (const __bf16*)a->q; p.kc = (__bf16*)a->k_cache; p.vc = (__bf16*)a->v_cache; p.o = (__bf16*)a->o;
-    p.ctx_len = a->ctx_len; p.k_new = (const __bf16*)a->k_new; p.v_new = (const __bf16*)a->v_new;
+    p.q = (const elem_t*)a->q; p.kc = (elem_t*)a->k_cache; p.vc = (elem_t*)a->v_cache; p.o = (elem_t*)a->o;
+    p.ctx_len = a->ctx_len; p.k_new = (const elem_t*)a->k_new; p.v_new = (const elem_t*)a->v_new;
     if (a->rotary_interleaved) {
         p.cos32 = (const float*)a->rotary_cos; p.sin32 = (const float*)a->rotary_sin;
     } else {
-        p.cos = (const __bf16*)a->rotary_cos; p.sin = (const __bf16*)a->rotary_sin;
+        p.cos = (const elem_t*)a->rotary_cos; p.sin = (const elem_t*)a->rotary_sin;
     }
     p.pos = a->position_ids;
     p.table_rows = (int)a->rotary_table_rows;
@@ -439,47 +443,13 @@ int decode_entry(const mi_decode_args* a, void* ws, size_t ws_bytes, bool static
 }
 }  // namespace
 
-extern "C" int mi_attn_decode(const mi_decode_args* a) {
+int MI_ENTRY(mi_attn_decode_impl)(const mi_decode_args* a, bool static_ws) {
     if (!a) return mi_fail(MI_E_NULL, "attn_decode: args is null");
-    return decode_entry(a, a->workspace, a->workspace_bytes, false);
-}
-
-// ---- entry point that allocates nothing ------------------------------------------------------------------------
-// The per-split partial results live in a file-scope device array instead of a caller workspace.  Every GPU the
-// library's code object is loaded on holds its own copy of the array at its own address, obtained once per device with
-// hipGetSymbolAddress (the array's name is only a host-side handle, not a device address) and kept in g_scratch_ptr.
-constexpr size_t kStaticScratchBytes = 8u << 20;
-static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
-
-namespace {
-constexpr int kMaxDevices = 64;
-void* g_scratch_ptr[kMaxDevices];        // per device; written once, under g_scratch_mutex
-std::mutex g_scratch_mutex;
-
-int static_scratch(void** out) {
-    int dev = -1;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
-        return mi_fail(MI_E_LAUNCH, "attn_decode_static: hipGetDevice failed or device index %d out of range (%s)", dev, hipGetErrorString(e));
-    std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (g_scratch_ptr[dev] == nullptr) {
-        void* ptr = nullptr;
-        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-        if (e != hipSuccess || ptr == nullptr)
-            return mi_fail(MI_E_LAUNCH, "attn_decode_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
-        g_scratch_ptr[dev] = ptr;
-    }
-    *out = g_scratch_ptr[dev];
-    return MI_OK;
-}
-}  // namespace
-
-extern "C" size_t mi_attn_decode_static_scratch_bytes(void) { return kStaticScratchBytes; }
-
-extern "C" int mi_attn_decode_static(const mi_decode_args* a) {
-    if (!a) return mi_fail(MI_E_NULL, "attn_decode_static: args is null");
+    if (!static_ws) return decode_entry(a, a->workspace, a->workspace_bytes, false);
+    // the entry point that allocates nothing: partial results go to the library's static device array
     void* ws = nullptr;
-    const int rc = static_scratch(&ws);
+    size_t bytes = 0;
+    const int rc = mi_static_scratch(&ws, &bytes);
     if (rc != MI_OK) return rc;
-    return decode_entry(a, ws, kStaticScratchBytes, true);
+    return decode_entry(a, ws, bytes, true);
 }

@@ -19,10 +19,6 @@
 
 #include <type_traits>
 
-int mi_attn_validate(const mi_attn_args* a, const char* who);
-void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p);
-int mi_compute_units();
-
 namespace {
 
 constexpr int BN = 64;               // keys per tile
@@ -84,18 +80,18 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     int klo, khi;
     key_range(p, tq, klo, khi);
     int wmin = khi > klo ? klo : 0x7fffffff, wmax = khi > klo ? khi : 0;
-    bf16x8_t qf[KS];
+    elem8_t qf[KS];
     {
         const int tl = tq < p.total_q ? tq : p.total_q - 1;
-        const __bf16* qrow = p.q + (int64_t)tl * p.q_st + (int64_t)head * p.q_sh + 8 * g;
+        const elem_t* qrow = p.q + (int64_t)tl * p.q_st + (int64_t)head * p.q_sh + 8 * g;
         uint4 raw[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const uint4*>(qrow + 16 * ks);
         if constexpr (QROT == 1) {
             int64_t pos = p.pos_q[tl];
             pos = pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
-            const __bf16* cr = p.cos + pos * D + 8 * g;
-            const __bf16* sr = p.sin + pos * D + 8 * g;
+            const elem_t* cr = p.cos + pos * D + 8 * g;
+            const elem_t* sr = p.sin + pos * D + 8 * g;
 #pragma unroll
             for (int ks = 0; ks < KS / 2; ++ks) {
                 const uint4 c = *reinterpret_cast<const uint4*>(cr + 16 * ks);
@@ -112,10 +108,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 rotate_interleaved(raw[ks], ld128(cr + 8 * ks), ld128(sr + 8 * ks), 1.0f);
         }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(bf16x8_t, raw[ks]);
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = __builtin_bit_cast(elem8_t, raw[ks]);
         if constexpr (QROT != 0) {
             if (p.q_rot != nullptr && tq < p.total_q) {
-                __bf16* qo = p.q_rot + (int64_t)tq * p.q_st + (int64_t)head * p.q_sh + 8 * g;
+                elem_t* qo = p.q_rot + (int64_t)tq * p.q_st + (int64_t)head * p.q_sh + 8 * g;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) st128(qo + 16 * ks, raw[ks]);
             }
@@ -159,8 +155,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     constexpr int TAB_VECS = ROT == 2 ? KV_VECS : (ROT == 1 ? KV_VECS / 2 : 1);
     uint4 craw[TAB_VECS], sraw[TAB_VECS];                            // rotary table rows of the K tile
     int64_t kpos[ROT ? KV_VECS / 2 : 1];                             // their positions, fetched a tile ahead
-    const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
-    const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
+    const elem_t* kbase = p.k + (int64_t)kvh * p.k_sh;
+    const elem_t* vbase = p.v + (int64_t)kvh * p.v_sh;
     const int last_k = p.total_k - 1;
 
     auto load_kpos = [&](int kt) {
@@ -179,7 +175,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 const int idx = ltid + 256 * j;
                 const int row = idx / (D / 16), c = idx % (D / 16);
                 const int tok = min(kt + row, last_k);
-                const __bf16* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
+                const elem_t* kr = kbase + (int64_t)tok * p.k_st + 8 * c;
                 kraw[2 * j] = ld128(kr);
                 kraw[2 * j + 1] = ld128(kr + D / 2);
                 int64_t pos = kpos[j];
@@ -275,8 +271,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         drop_sel = 16u * (uint32_t)(tq & 1);
     }
     f32x16_t s_acc[2];
-    bf16x8_t pf[4];
-    bf16x8_t pl[SPLIT ? 4 : 1];           // low-order terms of the probabilities
+    elem8_t pf[4];
+    elem8_t pl[SPLIT ? 4 : 1];           // low-order terms of the probabilities
     bool pending = false;                 // pf holds the probabilities of the previous tile
 
     // One MFMA phase = up to 16 steps of O^T += V^T P^T (previous tile) followed by up to 16 steps of
@@ -288,14 +284,14 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     auto mfma_phase = [&](auto mode, const char* vt, const char* ks) {
         constexpr bool kPV = (decltype(mode)::value & 1) != 0, kS = (decltype(mode)::value & 2) != 0;
         constexpr int first = kPV ? 0 : PV_STEPS, last = kS ? PV_STEPS + S_STEPS : PV_STEPS;
-        bf16x8_t ring[kDepth];
-        auto fetch = [&](int i) -> bf16x8_t {
+        elem8_t ring[kDepth];
+        auto fetch = [&](int i) -> elem8_t {
             if (i < PV_STEPS) {
                 const int m = i / DT, dt = i % DT;
                 return tr_pair(vt + (v_h0 ^ (dt << 6)) + 16 * m * RB, vt + (v_h1 ^ (dt << 6)) + 16 * m * RB);
             }
             const int ksi = (i - PV_STEPS) >> 1, t = (i - PV_STEPS) & 1;
-            return *reinterpret_cast<const bf16x8_t*>(ks + (k_row ^ (ksi << 5)) + 32 * t * RB);
+            return *reinterpret_cast<const elem8_t*>(ks + (k_row ^ (ksi << 5)) + 32 * t * RB);
         };
         if constexpr (kS) {
 #pragma unroll
@@ -308,7 +304,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = first; i < last; ++i) {
-            const bf16x8_t a = ring[(i - first) % kDepth];
+            const elem8_t a = ring[(i - first) % kDepth];
             if (i < PV_STEPS) {
                 const int m = i / DT, dt = i % DT;
                 o_acc[dt] = mfma_32x32x16(a, pf[m], o_acc[dt]);
@@ -392,8 +388,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                 for (int e = 0; e < 8; ++e) {
                     const float ev = fast_exp2(s_acc[t][r0 + e] * c2 - m_use);
                     if (e & 1) rs1 += ev; else rs0 += ev;
-                    pf[m][e] = (__bf16)ev;
-                    if constexpr (SPLIT) pl[m][e] = (__bf16)(ev - (float)pf[m][e]);
+                    pf[m][e] = (elem_t)ev;
+                    if constexpr (SPLIT) pl[m][e] = (elem_t)(ev - (float)pf[m][e]);
                 }
                 if constexpr (DROP) {
                     // the row sum above stays that of the full softmax; only the P that multiplies V is masked
@@ -402,8 +398,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
                     for (int pi = 0; pi < 4; ++pi) {
                         const int a = 2 * (m & 1) + (pi >> 1), j = pi & 1;
                         const uint32_t h = lowbias32(drop_xt + (uint32_t)(16 * t + 4 * a + j) * kDropC2);
-                        if (drop_byte(h, drop_sel) < p.drop_thr) { pf[m][2 * pi] = (__bf16)0.f; if constexpr (SPLIT) pl[m][2 * pi] = (__bf16)0.f; }
-                        if (drop_byte(h, drop_sel + 8) < p.drop_thr) { pf[m][2 * pi + 1] = (__bf16)0.f; if constexpr (SPLIT) pl[m][2 * pi + 1] = (__bf16)0.f; }
+                        if (drop_byte(h, drop_sel) < p.drop_thr) { pf[m][2 * pi] = (elem_t)0.f; if constexpr (SPLIT) pl[m][2 * pi] = (elem_t)0.f; }
+                        if (drop_byte(h, drop_sel + 8) < p.drop_thr) { pf[m][2 * pi + 1] = (elem_t)0.f; if constexpr (SPLIT) pl[m][2 * pi + 1] = (elem_t)0.f; }
                     }
                 }
             }
@@ -428,13 +424,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     const float l_tot = l_i + __shfl_xor(l_i, 32, 64);
     const float inv = (l_tot > 0.f ? 1.0f / l_tot : 0.f) * (DROP ? p.drop_rscale : 1.0f);
     if (tq < p.total_q) {
-        __bf16* orow = p.o + (int64_t)tq * p.o_st + (int64_t)head * p.o_sh + 4 * g;
+        elem_t* orow = p.o + (int64_t)tq * p.o_st + (int64_t)head * p.o_sh + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const uint32_t w0 = pack_bf16x2(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv);
-                const uint32_t w1 = pack_bf16x2(o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
+                const uint32_t w0 = pack_elem2(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv);
+                const uint32_t w1 = pack_elem2(o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
                 *reinterpret_cast<uint2*>(orow + 32 * dt + 8 * a) = make_uint2(w0, w1);
             }
         if (g == 0 && p.lse != nullptr) {
@@ -491,7 +487,7 @@ template <int D> int launch_d(const AttnParams& p, int rot, bool q_only, int nw,
 
 }  // namespace
 
-extern "C" int mi_attn_fwd(const mi_attn_args* a) {
+int MI_ENTRY(mi_attn_fwd_impl)(const mi_attn_args* a) {
     int rc = mi_attn_validate(a, "attn_fwd");
     if (rc != MI_OK) return rc;
     if (!a->o) return mi_fail(MI_E_NULL, "attn_fwd: o is null");
@@ -505,7 +501,7 @@ extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     if (a->q_rot_out) {
         if (!rot) return mi_fail(MI_E_NULL, "attn_fwd: q_rot_out needs the fused rotary");
         if (!mi_aligned16(a->q_rot_out)) return mi_fail(MI_E_ALIGN, "attn_fwd: q_rot_out must be 16-byte aligned");
-        p.q_rot = (__bf16*)a->q_rot_out;
+        p.q_rot = (elem_t*)a->q_rot_out;
     }
     // 256-query workgroups (two groups of wavefronts a phase apart) beat 128-query ones at every size measured,
     // also when they leave most compute units without work (1 x 512 tokens x 32 heads: 22 against 25 us,

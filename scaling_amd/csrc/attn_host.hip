@@ -1,63 +1,69 @@
-// Host-side argument checking shared by the attention entry points.
+// Entry points of the attention kernels: the kernels are compiled once per element type (bf16, f16); the C entry points
+// here pick the build that matches args->dtype.  Also home of the few things that exist once per library.
 #include "attn_common.h"
 
-int mi_attn_validate(const mi_attn_args* a, const char* who) {
-    if (!a) return mi_fail(MI_E_NULL, "%s: args is null", who);
-    if (!a->q || !a->k || !a->v || !a->cu_seqlens_q) return mi_fail(MI_E_NULL, "%s: q, k, v and cu_seqlens_q are required", who);
-    if (a->dtype != MI_BF16) return mi_fail(MI_E_DTYPE, "%s: only bf16 is supported (dtype code %d)", who, a->dtype);
-    if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 96 && a->head_dim != 128)
-        return mi_fail(MI_E_SHAPE, "%s: head_dim %d unsupported (32, 64, 96, 128)", who, a->head_dim);
-    if (a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0)
-        return mi_fail(MI_E_SHAPE, "%s: n_q_heads=%d must be a positive multiple of n_kv_heads=%d", who, a->n_q_heads, a->n_kv_heads);
-    if (a->total_q < 0 || a->total_k < 0 || a->total_q > 0x7fffffffLL || a->total_k > 0x7fffffffLL || a->n_docs < 0)
-        return mi_fail(MI_E_SHAPE, "%s: bad token counts q=%lld k=%lld docs=%d", who, (long long)a->total_q, (long long)a->total_k, a->n_docs);
-    if (a->total_q > 0 && (a->n_docs < 1 || a->total_k < 1))
-        return mi_fail(MI_E_SHAPE, "%s: non-empty query needs at least one document and one key", who);
-    if (!mi_aligned16(a->q) || !mi_aligned16(a->k) || !mi_aligned16(a->v))
-        return mi_fail(MI_E_ALIGN, "%s: q, k, v must be 16-byte aligned", who);
-    if (a->q_stride_token % 8 || a->q_stride_head % 8 || a->k_stride_token % 8 || a->k_stride_head % 8 ||
-        a->v_stride_token % 8 || a->v_stride_head % 8)
-        return mi_fail(MI_E_ALIGN, "%s: strides must be multiples of 8 elements", who);
-    if (!(a->softmax_scale > 0.f)) return mi_fail(MI_E_SHAPE, "%s: softmax_scale must be positive", who);
-    if (a->rotary_cos || a->rotary_sin) {
-        if (!a->rotary_cos || !a->rotary_sin || !a->position_ids_q)
-            return mi_fail(MI_E_NULL, "%s: fused rotary needs cos, sin and the query position ids", who);
-        if (a->head_dim != 64 && a->head_dim != 128) return mi_fail(MI_E_SHAPE, "%s: fused rotary needs head_dim 64 or 128", who);
-        if (a->rotary_table_rows <= 0 || a->rotary_table_rows > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "%s: bad rotary table size", who);
-        if (!mi_aligned16(a->rotary_cos) || !mi_aligned16(a->rotary_sin)) return mi_fail(MI_E_ALIGN, "%s: rotary tables must be 16-byte aligned", who);
+#include <mutex>
+
+int mi_attn_fwd_impl_bf16(const mi_attn_args* a);
+int mi_attn_fwd_impl_f16(const mi_attn_args* a);
+int mi_attn_bwd_impl_bf16(const mi_attn_bwd_args* b);
+int mi_attn_bwd_impl_f16(const mi_attn_bwd_args* b);
+int mi_attn_decode_impl_bf16(const mi_decode_args* a, bool static_ws);
+int mi_attn_decode_impl_f16(const mi_decode_args* a, bool static_ws);
+
+extern "C" int mi_attn_fwd(const mi_attn_args* a) {
+    if (!a) return mi_fail(MI_E_NULL, "attn_fwd: args is null");
+    return a->dtype == MI_F16 ? mi_attn_fwd_impl_f16(a) : mi_attn_fwd_impl_bf16(a);
+}
+
+extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
+    if (!b) return mi_fail(MI_E_NULL, "attn_bwd: args is null");
+    return b->fwd.dtype == MI_F16 ? mi_attn_bwd_impl_f16(b) : mi_attn_bwd_impl_bf16(b);
+}
+
+extern "C" int mi_attn_decode(const mi_decode_args* a) {
+    if (!a) return mi_fail(MI_E_NULL, "attn_decode: args is null");
+    return a->dtype == MI_F16 ? mi_attn_decode_impl_f16(a, false) : mi_attn_decode_impl_bf16(a, false);
+}
+
+extern "C" int mi_attn_decode_static(const mi_decode_args* a) {
+    if (!a) return mi_fail(MI_E_NULL, "attn_decode_static: args is null");
+    return a->dtype == MI_F16 ? mi_attn_decode_impl_f16(a, true) : mi_attn_decode_impl_bf16(a, true);
+}
+
+// ---- scratch of the entry point that allocates nothing -----------------------------------------------------------
+// The per-split partial results of mi_attn_decode_static live in a file-scope device array instead of a caller
+// workspace.  Every GPU the library's code object is loaded on holds its own copy of the array at its own address,
+// obtained once per device with hipGetSymbolAddress (the array's name is only a host-side handle, not a device
+// address) and kept in g_scratch_ptr.
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];        // per device; written once, under g_scratch_mutex
+std::mutex g_scratch_mutex;
+}  // namespace
+
+int mi_static_scratch(void** out, size_t* bytes) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return mi_fail(MI_E_LAUNCH, "attn_decode_static: hipGetDevice failed or device index %d out of range (%s)", dev, hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return mi_fail(MI_E_LAUNCH, "attn_decode_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
     }
-    if (!(a->dropout_p >= 0.f) || a->dropout_p >= 1.f) return mi_fail(MI_E_SHAPE, "%s: dropout_p must be in [0, 1)", who);
+    *out = g_scratch_ptr[dev];
+    *bytes = kStaticScratchBytes;
     return MI_OK;
 }
 
-void mi_attn_fill_params(const mi_attn_args* a, AttnParams* p) {
-    *p = AttnParams{};
-    p->q = (const __bf16*)a->q; p->k = (const __bf16*)a->k; p->v = (const __bf16*)a->v;
-    p->o = (__bf16*)a->o; p->lse = a->lse;
-    p->cu_q = a->cu_seqlens_q; p->cu_k = a->cu_seqlens_k ? a->cu_seqlens_k : a->cu_seqlens_q;
-    p->n_docs = a->n_docs; p->causal = a->causal;
-    p->total_q = (int)a->total_q; p->total_k = (int)a->total_k;
-    p->nq = a->n_q_heads; p->nkv = a->n_kv_heads; p->n_rep = a->n_q_heads / a->n_kv_heads;
-    p->q_st = a->q_stride_token; p->q_sh = a->q_stride_head;
-    p->k_st = a->k_stride_token; p->k_sh = a->k_stride_head;
-    p->v_st = a->v_stride_token; p->v_sh = a->v_stride_head;
-    p->o_st = a->o_stride_token; p->o_sh = a->o_stride_head;
-    p->scale = a->softmax_scale;
-    p->scale_log2 = a->softmax_scale * 1.4426950408889634f;
-    if (a->rotary_interleaved) {
-        p->cos32 = (const float*)a->rotary_cos; p->sin32 = (const float*)a->rotary_sin;
-    } else {
-        p->cos = (const __bf16*)a->rotary_cos; p->sin = (const __bf16*)a->rotary_sin;
-    }
-    p->pos_q = a->position_ids_q; p->pos_k = a->position_ids_k; p->table_rows = (int)a->rotary_table_rows;
-    if (a->dropout_p > 0.f) {
-        int t = (int)(a->dropout_p * 256.0f + 0.5f);
-        t = t < 1 ? 1 : (t > 255 ? 255 : t);
-        p->drop_thr = (uint32_t)t;
-        p->drop_rscale = 256.0f / (float)(256 - t);
-        p->drop_seed = (uint32_t)(a->dropout_seed & 0xffffffffu) ^ (uint32_t)(a->dropout_seed >> 32);
-    }
-}
+extern "C" size_t mi_attn_decode_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
 // Compute units of the current device (256 on an MI355X), asked once per device.
 int mi_compute_units() {

@@ -15,6 +15,7 @@ LIB_NAME = "libmi355_layer.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = ["abi.hip", "rmsnorm.hip", "swiglu.hip", "rotary.hip", "attn_host.hip", "attn_fwd.hip", "attn_bwd.hip",
            "attn_decode.hip", "cross_entropy.hip"]
+F16_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "attn_decode.hip"]
 # packed fp32 VALU instructions stay disabled for every device translation unit; the kernels never
 # produce NaNs on purpose (masked scores are -inf and every inf - inf is guarded), so NaN-preserving
 # canonicalisation of the MFMA results before max / min is switched off
@@ -41,15 +42,19 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     obj_dir = os.path.join(HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
 
-    def compile_one(src):
-        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-        _run([hipcc] + FLAGS + ["-c", src, "-o", obj])
+    def compile_one(job):
+        src, suffix, defines = job
+        obj = os.path.join(obj_dir, src.replace(".hip", suffix + ".o"))
+        _run([hipcc] + FLAGS + defines + ["-c", src, "-o", obj])
         if verbose:
-            print("compiled", src, flush=True)
+            print("compiled", src, " ".join(defines), flush=True)
         return obj
 
+    # the attention kernels exist once per element type: bfloat16 (as is) and float16 (-DMI_ELEM_F16)
+    jobs_list = [(s, "", []) for s in SOURCES] + [(s, "_f16", ["-DMI_ELEM_F16"]) for s in F16_SOURCES]
+    jobs_list.sort(key=lambda j: 0 if j[0] in ("attn_fwd.hip", "attn_bwd.hip") else 1)   # the slow ones first
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
+        objs = list(pool.map(compile_one, jobs_list))
     tmp = LIB_PATH + ".tmp"
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs)
     os.replace(tmp, LIB_PATH)

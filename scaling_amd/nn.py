@@ -329,7 +329,7 @@ class ParallelSelfAttention(torch.nn.Module):
     silent fall-backs: attention-score manipulation, LoRA, local attention windows, u-muP and fp8 are not
     available; attention-probability dropout is applied inside the kernels in training mode (its mask comes
     from a counter-based hash, not from torch's generator stream, and its rate is quantised to 1/256);
-    the dtype must be bfloat16.  The KV cache is pre-allocated (see `KVCache`), supports batches of
+    the dtype must be bfloat16 or float16.  The KV cache is pre-allocated (see `KVCache`), supports batches of
     single-document rows and is filled/extended in place.
     """
 
@@ -359,8 +359,8 @@ class ParallelSelfAttention(torch.nn.Module):
         if num_local_attention_heads > 0 or lora_config is not None or fp8_config is not None or \
                 fp8_config_dense_out is not None or bitfit_bias_name is not None:
             raise NotImplementedError("local attention, LoRA, fp8 and bitfit are outside the hip kernel's scope")
-        if dtype != torch.bfloat16:
-            raise NotImplementedError("the hip attention kernels compute in bfloat16; set precision: bfloat16")
+        if dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError("the hip attention kernels compute in bfloat16 or float16; set precision: bfloat16 (or float16)")
 
         self.hidden_size_per_attention_head = hidden_size // num_attention_heads
         self.num_attention_heads = num_attention_heads

@@ -84,6 +84,46 @@ def test_attention_accuracy_mode_meets_the_stated_tolerance(b, s, nq, nkv, d, ca
             check(f"attn.{tag}.{name}", got, r, ro, literal=precise)
 
 
+@pytest.mark.parametrize("b,s,nq,nkv,d,causal,cuts,rot", [
+    (2, 128, 4, 4, 64, True, (), False),
+    (2, 256, 8, 2, 128, True, (100, 300, 301), False),
+    (1, 384, 6, 3, 96, False, (129,), False),
+    (2, 64, 4, 2, 32, True, (32,), False),
+    (1, 320, 8, 1, 128, True, (100,), True),        # rotary on the training path, split dK/dV launch
+])
+def test_attention_float16_fwd_bwd_parity(b, s, nq, nkv, d, causal, cuts, rot):
+    """precision: float16 (transformer/context/config.py:28-48): the same kernels built on the half-precision MFMA."""
+    print(f"case attn f16 b={b} s={s} nq={nq} nkv={nkv} d={d} causal={causal} cuts={cuts} rotary={rot}", flush=True)
+    q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=b * 100 + s + d, dtype=torch.float16)
+    cu = U.make_cu(b, s, cuts)
+    scale, n_rep = 1.0 / math.sqrt(d), nq // nkv
+    pos = U.position_ids_from_cu(cu, b * s)
+    ids = pos.view(b, s).transpose(0, 1)
+    tabs = oracle.rotary_tables(d, s, 10000, torch.float16) if rot else None
+
+    def reference(dtype):
+        qq, kk, vv = (t.to(dtype).clone().requires_grad_() for t in (q, k, v))
+        q4, k4, v4 = U.to_sbnd(qq, b, s), U.to_sbnd(kk, b, s), U.to_sbnd(vv, b, s)
+        if rot:
+            q4, k4 = oracle.apply_rotary(q4, k4, oracle.RotaryTables(tabs.cos.to(dtype), tabs.sin.to(dtype), d), ids, ids)
+        out = oracle.multi_head_attention(q4, oracle.repeat_kv(k4, n_rep), oracle.repeat_kv(v4, n_rep), cu, causal, scale,
+                                          softmax_in_fp32=True)
+        o = U.from_bn_s_d(out, b, nq)
+        o.backward(do.to(dtype))
+        return o.detach(), qq.grad, kk.grad, vv.grad
+
+    ref, ref_o = reference(torch.float32), reference(torch.float16)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    rotary = (tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV), pos.to(DEV)) if rot else None
+    o = ops.attention(qg, kg, vg, cu.to(DEV), None, causal, scale, rotary=rotary)
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    assert o.dtype == torch.float16 and qg.grad.dtype == torch.float16
+    for name, got, r, ro in (("o", o, ref[0], ref_o[0]), ("dq", qg.grad, ref[1], ref_o[1]),
+                             ("dk", kg.grad, ref[2], ref_o[2]), ("dv", vg.grad, ref[3], ref_o[3])):
+        check(f"attn.f16.{name}", got, r, ro)
+
+
 def test_attention_mask_is_bit_exact_on_reference_known_answers():
     """q = k = 0 makes the softmax uniform over the allowed keys; with one-hot values the output row is
     1/count on exactly the allowed key positions, which exposes the kernel's mask predicate."""

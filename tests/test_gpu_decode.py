@@ -186,3 +186,29 @@ def test_decode_takes_column_slices_of_a_fused_projection():
         assert torch.equal(caches[0][0][b, int(ctx[b]) - 1], k[b]) and torch.equal(caches[0][1][b, int(ctx[b]) - 1], v[b])
     with pytest.raises(AssertionError):
         ops.decode_attention(fused.view(B, nq + 2 * nkv, d)[:, ::2], caches[0][0], caches[0][1], ctx)   # heads not contiguous
+
+
+@pytest.mark.parametrize("B,nq,nkv,d,max_ctx,lens", [(3, 8, 2, 128, 300, [1, 137, 300]), (24, 16, 8, 128, 300, [300, 1, 257, 31] * 6),
+                                                    (2, 4, 4, 64, 128, [128, 5])])
+def test_decode_float16_parity(B, nq, nkv, d, max_ctx, lens):
+    """The decode kernels built on the half-precision MFMA (precision: float16), with the in-place append."""
+    print(f"case decode f16 B={B} nq={nq} nkv={nkv} d={d} lens={lens}", flush=True)
+    g = torch.Generator().manual_seed(B + d)
+    q = torch.randn(B, nq, d, generator=g).half()
+    kc = torch.randn(B, max_ctx, nkv, d, generator=g).half()
+    vc = torch.randn(B, max_ctx, nkv, d, generator=g).half()
+    k_new, v_new = torch.randn(B, nkv, d, generator=g).half(), torch.randn(B, nkv, d, generator=g).half()
+    ctx = torch.tensor(lens, dtype=torch.int32)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    for b in range(B):
+        kc_ref[b, lens[b] - 1] = k_new[b]
+        vc_ref[b, lens[b] - 1] = v_new[b]
+    scale = 1 / math.sqrt(d)
+    ref = _oracle_decode(q, kc_ref, vc_ref, ctx, scale, torch.float32)
+    ref_o = _oracle_decode(q, kc_ref, vc_ref, ctx, scale, torch.float16)
+    kcd, vcd = kc.to(DEV), vc.to(DEV)
+    out = ops.decode_attention(q.to(DEV), kcd, vcd, ctx.to(DEV), k_new.to(DEV), v_new.to(DEV), softmax_scale=scale)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    check("decode.f16.o", out, ref, ref_o)
+    assert torch.equal(kcd.cpu(), kc_ref) and torch.equal(vcd.cpu(), vc_ref)

@@ -56,8 +56,8 @@ def _oracle_layer(cfg, weights, x, cu, pos, dy, dtype):
     spec.rotary_percentage = cfg.rotary_percentage
     w = {k: v.detach().cpu().to(dtype).clone().requires_grad_() for k, v in weights.items()}
     xx = x.to(dtype).clone().requires_grad_()
-    # the module keeps its rotary tables in bf16 (reference behaviour); the oracle uses the same values
-    t = oracle.rotary_tables(spec.rotary_dim, spec.sequence_length, spec.rotary_base, torch.bfloat16)
+    # the module keeps its rotary tables in the activation dtype (reference behaviour); the oracle uses the same values
+    t = oracle.rotary_tables(spec.rotary_dim, spec.sequence_length, spec.rotary_base, cfg.precision.dtype)
     tables = oracle.RotaryTables(t.cos.to(dtype), t.sin.to(dtype), t.dim)
     y = oracle.transformer_layer(spec, w, xx, cu, pos, tables=tables)
     y.backward(dy.to(dtype))
@@ -73,14 +73,16 @@ def _oracle_layer(cfg, weights, x, cu, pos, dy, dtype):
     # the reference's default architecture: LayerNorm + GELU MLP with biases
     ("layernorm_gelu", dict(norm_type="layernorm", mlp_type="default", mlp_factor=4.0, attention_bias=True, mlp_bias=True), 2, 64, (50,)),
     ("key_query_layernorm", dict(norm_type="layernorm", mlp_type="default", mlp_factor=4.0, key_query_norm=True), 1, 64, ()),
+    ("float16_gqa", dict(precision="float16", hidden_size=512, num_attention_heads=4, attention_num_kv_heads=2), 2, 96, (40,)),
 ])
 def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
     print(f"case layer {name}", flush=True)
     cfg = _arch(**kw)
     layer = _seeded_layer(cfg, seed=0)
     g = torch.Generator().manual_seed(1)
-    x = torch.randn(b, s, cfg.hidden_size, generator=g).bfloat16()
-    dy = torch.randn(b, s, cfg.hidden_size, generator=g).bfloat16()
+    act = cfg.precision.dtype            # bfloat16, or float16 for the half-precision case
+    x = torch.randn(b, s, cfg.hidden_size, generator=g).to(act)
+    dy = torch.randn(b, s, cfg.hidden_size, generator=g).to(act)
     cu = torch.tensor(sorted(set(i * s for i in range(b + 1)) | set(cuts)), dtype=torch.int32)
     pos = torch.zeros(b * s, dtype=torch.int64)
     for a_, b_ in zip(cu[:-1].tolist(), cu[1:].tolist()):
@@ -88,7 +90,7 @@ def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
     pos = pos.view(b, s)
     weights = {k: v for k, v in layer.state_dict().items()}
     ref = _oracle_layer(cfg, weights, x, cu, pos, dy, torch.float32)
-    ref_o = _oracle_layer(cfg, weights, x, cu, pos, dy, torch.bfloat16)
+    ref_o = _oracle_layer(cfg, weights, x, cu, pos, dy, act)
 
     xg = x.to(DEV).requires_grad_()
     out = layer(TransformerLayerIO(activations=xg, position_ids=pos.to(DEV), cumulative_seq_lengths=cu.to(DEV)))
@@ -99,7 +101,7 @@ def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
     for k, p in layer.named_parameters():
         # parameter gradients sum over all tokens: compare against the reference's own bf16 error, with 25 % slack
         m = metrics(p.grad, ref[2][k])
-        f = metrics(ref_o[2][k], ref[2][k], torch.bfloat16)
+        f = metrics(ref_o[2][k], ref[2][k], act)
         print(f"[parity] {name}.d{k}: mean_rel={m['mean_rel']:.3e} (reference bf16 order {f['mean_rel']:.3e})", flush=True)
         if k.endswith("self_attention.key.bias"):
             # analytically zero (a constant added to every key shifts all scores of a query alike, and softmax is
