@@ -158,14 +158,11 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     const float* stat_base = (tid < BQ) ? p.lse : p.delta;
     const float stat_scale = (tid < BQ) ? 1.4426950408889634f : 1.0f;
     float stat = 0.f;
-    auto tile_of = [&](int iter, int& head, int& qt) {
-        const int rep = iter % hpw, tile = iter / hpw;
-        head = kvh * p.n_rep + hs * hpw + rep;
-        qt = qt0 + (n_tiles - 1 - tile) * BQ;
-    };
-    auto issue_tile = [&](int iter) {     // Q / dO tile of iteration `iter` -> stage iter & 1
-        int head, qt;
-        tile_of(iter, head, qt);
+    // (query head of the group, query tile) of the current and of the next iteration, stepped without divisions
+    int cur_rep = 0, cur_tile = 0, nxt_rep = 0, nxt_tile = 0;
+    auto issue_tile = [&](int iter) {     // Q / dO tile of iteration `iter` (= the next one) -> stage iter & 1
+        const int head = kvh * p.n_rep + hs * hpw + nxt_rep;
+        const int qt = qt0 + (n_tiles - 1 - nxt_tile) * BQ;
         plan.issue(src_base + (int64_t)head * src_head_stride, src_tok_stride, qt, last_q, dst_tile + (iter & 1) * TILE);
         if (tid < 2 * BQ) {
             const int tok = min(qt + (tid & (BQ - 1)), last_q);
@@ -200,7 +197,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 
     auto tile_step = [&](auto buf_c, int iter) {
         constexpr int buf = decltype(buf_c)::value;
-        const int qs = qt0 + (n_tiles - 1 - iter / hpw) * BQ + 32 * sub;
+        const int qs = qt0 + (n_tiles - 1 - cur_tile) * BQ + 32 * sub;
+        if (++nxt_rep == hpw) { nxt_rep = 0; ++nxt_tile; }
         if (iter + 1 < total_iters) issue_tile(iter + 1);
 
         if ((qs < wmax) && (qs + 32 > wmin)) {
@@ -209,15 +207,30 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             f32x16_t s_acc, dp_acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) { s_acc[r] = 0.f; dp_acc[r] = 0.f; }
+            // 2 KS products whose operands come from LDS through rings of kDepth registers filled kDepth products ahead
+            // (sched_barrier pins that order): left to the compiler, the four reads of a contraction step are issued right
+            // before its two products, which then wait out the LDS latency KS times per tile (measured: 1330 -> 810 cycles
+            // for this stage, -3 % on the kernel)
+            {
+                constexpr int kSteps = 2 * KS, kDepth = 3;
+                elem8_t ra[kDepth], rb[kDepth];
+                auto fetch = [&](int i, elem8_t& a, elem8_t& b) {
+                    const int ks = i >> 1;
+                    const int ao = a_row ^ (ks << 5), bo = b_row ^ (ks << 5);
+                    a = *reinterpret_cast<const elem8_t*>(((i & 1) ? dt_ : qt_) + ao);
+                    b = *reinterpret_cast<const elem8_t*>(((i & 1) ? v_t : k_t) + bo);
+                };
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int ao = a_row ^ (ks << 5), bo = b_row ^ (ks << 5);
-                const elem8_t aq = *reinterpret_cast<const elem8_t*>(qt_ + ao);
-                const elem8_t bk = *reinterpret_cast<const elem8_t*>(k_t + bo);
-                s_acc = mfma_32x32x16(aq, bk, s_acc);
-                const elem8_t ad = *reinterpret_cast<const elem8_t*>(dt_ + ao);
-                const elem8_t bv = *reinterpret_cast<const elem8_t*>(v_t + bo);
-                dp_acc = mfma_32x32x16(ad, bv, dp_acc);
+                for (int i = 0; i < kDepth; ++i) fetch(i, ra[i], rb[i]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < kSteps; ++i) {
+                    const elem8_t a = ra[i % kDepth], b = rb[i % kDepth];
+                    if (i & 1) dp_acc = mfma_32x32x16(a, b, dp_acc);
+                    else s_acc = mfma_32x32x16(a, b, s_acc);
+                    if (i + kDepth < kSteps) fetch(i + kDepth, ra[i % kDepth], rb[i % kDepth]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             // rows of the accumulators are queries qs + 8a + 4g + c, the column is this lane's key
             if (__any((qs < qlo) || (qs + 32 > qhi))) {
@@ -234,7 +247,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             elem8_t pl[SPLIT ? 2 : 1], dsl[SPLIT ? 2 : 1];   // accuracy mode: low-order terms of P and dS
             uint32_t drop_xb = 0;
             if constexpr (DROP) {
-                const int head_i = kvh * p.n_rep + hs * hpw + iter % hpw;
+                const int head_i = kvh * p.n_rep + hs * hpw + cur_rep;
                 drop_xb = drop_head_base(p.drop_seed, head_i) + drop_xc + (uint32_t)(qs >> 1) * kDropC1;
             }
 #pragma unroll
@@ -283,6 +296,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             }
         }
         if (iter + 1 < total_iters) store_stat(iter + 1);
+        cur_rep = nxt_rep;
+        cur_tile = nxt_tile;
         wait_vmcnt<0>();                  // the next Q / dO tile has landed
         __syncthreads();
     };
