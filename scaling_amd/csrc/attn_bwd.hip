@@ -539,15 +539,25 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) { s_acc[t][r] = 0.f; dp_acc[t][r] = 0.f; }
+            // 4 KS products whose A operands come from LDS through a ring of kDepth registers filled kDepth products ahead
+            {
+                constexpr int kSteps = 4 * KS, kDepth = 3;
+                elem8_t ring[kDepth];
+                auto fetch = [&](int i) -> elem8_t {
+                    const int ks = i >> 2, t = (i >> 1) & 1;
+                    return *reinterpret_cast<const elem8_t*>(((i & 1) ? vt_ : kt_) + (a_row ^ (ks << 5)) + 32 * t * RB);
+                };
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int ao = a_row ^ (ks << 5);
+                for (int i = 0; i < kDepth; ++i) ring[i] = fetch(i);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const elem8_t ak = *reinterpret_cast<const elem8_t*>(kt_ + ao + 32 * t * RB);
-                    s_acc[t] = mfma_32x32x16(ak, qf[ks], s_acc[t]);
-                    const elem8_t av = *reinterpret_cast<const elem8_t*>(vt_ + ao + 32 * t * RB);
-                    dp_acc[t] = mfma_32x32x16(av, dof[ks], dp_acc[t]);
+                for (int i = 0; i < kSteps; ++i) {
+                    const int ks = i >> 2, t = (i >> 1) & 1;
+                    const elem8_t a = ring[i % kDepth];
+                    if (i & 1) dp_acc[t] = mfma_32x32x16(a, dof[ks], dp_acc[t]);
+                    else s_acc[t] = mfma_32x32x16(a, qf[ks], s_acc[t]);
+                    if (i + kDepth < kSteps) ring[i % kDepth] = fetch(i + kDepth);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
             if (__any((kt < klo) || (kt + BN > khi))) {
@@ -562,36 +572,53 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                         if (rel >= len) s_acc[t][r] = -INFINITY;
                     }
             }
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                const int t = m >> 1, r0 = 8 * (m & 1);
-                elem8_t dsf, dsl;
+            // dS of accumulator register 8 (m & 1) + e of key sub-tile m >> 1 (m = 16-key chunk, e = 0..7), compile-time indices
+            const uint32_t drop_xt = DROP ? drop_xr + (uint32_t)(kt >> 1) * kDropC2 : 0u;
+            auto ds_element = [&](auto m_c, auto e_c, elem8_t& dsf, elem8_t& dsl) {
+                constexpr int m = decltype(m_c)::value, e = decltype(e_c)::value, t = m >> 1, r = 8 * (m & 1) + e;
+                float dpv = dp_acc[t][r];
                 if constexpr (DROP) {
                     // dP of a dropped probability is zero, that of a kept one carries the 1 / (1 - p) scale
-                    const uint32_t drop_xt = drop_xr + (uint32_t)(kt >> 1) * kDropC2;
-#pragma unroll
-                    for (int pi = 0; pi < 4; ++pi) {
-                        const int a = 2 * (m & 1) + (pi >> 1), j = pi & 1;
-                        const uint32_t h = lowbias32(drop_xt + (uint32_t)(16 * t + 4 * a + j) * kDropC2);
-                        const bool keep0 = drop_byte(h, drop_sel) >= p.drop_thr, keep1 = drop_byte(h, drop_sel + 8) >= p.drop_thr;
-                        dp_acc[t][r0 + 2 * pi] = keep0 ? dp_acc[t][r0 + 2 * pi] * p.drop_rscale : 0.f;
-                        dp_acc[t][r0 + 2 * pi + 1] = keep1 ? dp_acc[t][r0 + 2 * pi + 1] * p.drop_rscale : 0.f;
-                    }
+                    constexpr int pi = e >> 1, a = 2 * (m & 1) + (pi >> 1), j = pi & 1;
+                    const uint32_t h = lowbias32(drop_xt + (uint32_t)(16 * t + 4 * a + j) * kDropC2);
+                    dpv = drop_byte(h, drop_sel + 8 * (e & 1)) >= p.drop_thr ? dpv * p.drop_rscale : 0.f;
                 }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float pv = fast_exp2(s_acc[t][r0 + e] * c2 - lse2);
-                    const float ds = pv * (dp_acc[t][r0 + e] - delta);
-                    dsf[e] = (elem_t)ds;
-                    if constexpr (SPLIT) dsl[e] = (elem_t)(ds - (float)dsf[e]);
-                }
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
+                const float pv = fast_exp2(s_acc[t][r] * c2 - lse2);
+                const float ds = pv * (dpv - delta);
+                dsf[e] = (elem_t)ds;
+                if constexpr (SPLIT) dsl[e] = (elem_t)(ds - (float)dsf[e]);
+            };
+            // dQ^T += K^T dS^T: 4 DT products, chunk by chunk of 16 keys; the transposed K operands come through a ring filled
+            // kDepth products ahead and the dS of chunk m + 1 are computed between the products of chunk m, so neither the LDS
+            // latency nor the softmax arithmetic sits between two products (sched_barrier pins the order)
+            {
+                constexpr int kSteps = 4 * DT, kDepth = 3;
+                elem8_t ring[kDepth];
+                elem8_t d[2], dl[2];
+                auto fetch = [&](int i) -> elem8_t {
+                    const int m = i / DT, dt = i % DT;
                     const int o0 = (tr_h0 ^ (dt << 6)) + 16 * m * RB, o1 = (tr_h1 ^ (dt << 6)) + 16 * m * RB;
-                    const elem8_t akt = tr_pair(kt_ + o0, kt_ + o1);
-                    dq_acc[dt] = mfma_32x32x16(akt, dsf, dq_acc[dt]);
-                    if constexpr (SPLIT) dq_acc[dt] = mfma_32x32x16(akt, dsl, dq_acc[dt]);
-                }
+                    return tr_pair(kt_ + o0, kt_ + o1);
+                };
+#pragma unroll
+                for (int i = 0; i < kDepth; ++i) ring[i] = fetch(i);
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<8>([&](auto e_c) { ds_element(std::integral_constant<int, 0>{}, e_c, d[0], dl[0]); });
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<kSteps>([&](auto i_c) {
+                    constexpr int i = decltype(i_c)::value, m = i / DT, dt = i % DT;
+                    const elem8_t a = ring[i % kDepth];
+                    dq_acc[dt] = mfma_32x32x16(a, d[m & 1], dq_acc[dt]);
+                    if constexpr (SPLIT) dq_acc[dt] = mfma_32x32x16(a, dl[m & 1], dq_acc[dt]);
+                    if constexpr (i + kDepth < kSteps) ring[i % kDepth] = fetch(i + kDepth);
+                    if constexpr (m < 3) {
+                        static_for<8>([&](auto e_c) {
+                            constexpr int e = decltype(e_c)::value;
+                            if constexpr ((e * DT) / 8 == dt) ds_element(std::integral_constant<int, m + 1>{}, e_c, d[(m + 1) & 1], dl[(m + 1) & 1]);
+                        });
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             }
         }
         // tile it+1 must have landed; tile it+2 (just issued) may still be in flight

@@ -13,6 +13,8 @@
 #pragma once
 #include "common.h"
 
+#include <type_traits>
+
 // Element type of q / k / v / o and of every MFMA operand.  Each attention source file is compiled twice: as is for
 // bfloat16 and with MI_ELEM_F16 for float16 (half-precision MFMA, same tilings); the bfloat16 objects export the C
 // entry points and hand float16 calls to the MI_ENTRY(...)-named functions of the float16 objects.
@@ -261,6 +263,15 @@ template <int D, int COUNT> struct DmaPlan {
         }
     }
 };
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index is a constant
+// expression inside the body
+template <int N, int I = 0, class F> __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 // waits until at most n (wave-uniform, run-time) vector memory loads are outstanding; large n waits for less
 // than asked only in the sense of waiting for everything older than the newest 24
