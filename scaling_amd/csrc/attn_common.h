@@ -95,6 +95,27 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16(elem8_t a, elem8_t b, f32x16_t
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// max / sum of a value with that of the lane 32 further on (lane ^ 32), exchanged inside the VALU by v_permlane32_swap
+// (afterwards every lane holds the pair (value of the low lane, value of the high lane)) instead of through the LDS
+// crossbar, whose round trip would sit in the middle of the softmax chain of every tile
+__device__ __forceinline__ float pair_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+// the same over the four lanes l16, l16 + 16, l16 + 32, l16 + 48 (v_permlane16_swap pairs the rows of 16 lanes)
+__device__ __forceinline__ float quad_max(float x) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return pair_max(fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1])));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float quad_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return pair_sum(__uint_as_float(r[0]) + __uint_as_float(r[1]));
+}
+
 // index j with cu[j] <= t < cu[j+1]  (cu has n_docs + 1 non-decreasing entries, cu[0] = 0)
 __device__ __forceinline__ int find_doc(const int32_t* __restrict__ cu, int n_docs, int t) {
     int lo = 0, hi = n_docs;

@@ -216,8 +216,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
                     if (key0 + 16 * t + 4 * G + r >= s1) s_acc[t][r] = -INFINITY;
                     mx = fmaxf(mx, s_acc[t][r]);
                 }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = quad_max(mx);
             const float m_new = fmaxf(m_i, mx * p.scale_log2);   // finite: the chunk holds >= 1 valid key
             alpha = fast_exp2(m_i - m_new);
             m_i = m_new;
@@ -265,8 +264,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void decode_split_kernel(const DecodeP
     }
 
     // ---- merge the four wavefronts, emit the split partial -----------------------------------------
-    l_i += __shfl_xor(l_i, 16, 64);
-    l_i += __shfl_xor(l_i, 32, 64);
+    l_i = quad_sum(l_i);
     __syncthreads();
     if (G == 0) { wm_lds[wave][l16] = m_i; wl_lds[wave][l16] = l_i; }
     if (l16 < n_heads) {

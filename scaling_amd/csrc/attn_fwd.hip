@@ -363,7 +363,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
             float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
 #pragma unroll
             for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s_acc[0][r], s_acc[1][r]));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = pair_max(mx);
             const float m_cand = mx * c2;
             if (__any(m_cand > m_i + kRescaleGap)) {
                 const float m_new = fmaxf(m_i, m_cand);
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     if (grp == 0) __syncthreads();
 
     // ---- epilogue ------------------------------------------------------------------------------
-    const float l_tot = l_i + __shfl_xor(l_i, 32, 64);
+    const float l_tot = pair_sum(l_i);
     const float inv = (l_tot > 0.f ? 1.0f / l_tot : 0.f) * (DROP ? p.drop_rscale : 1.0f);
     if (tq < p.total_q) {
         elem_t* orow = p.o + (int64_t)tq * p.o_st + (int64_t)head * p.o_sh + 4 * g;
