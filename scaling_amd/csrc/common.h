@@ -110,9 +110,27 @@ __device__ __forceinline__ void rotate_complex_pair(float& x0, float& x1, float 
 }
 
 // ---- wavefront reductions (64 lanes) -------------------------------------------------------
+// Sum over aligned groups of WIDTH lanes, every lane receiving the total, without going through the LDS crossbar
+// (six dependent ds_bpermute round trips per 64-lane sum otherwise): DPP lane selects inside a row of 16 lanes
+// (quad permutes, then the mirror images of 8 and of 16 lanes, which pair every partial sum with the one it still
+// lacks), v_permlane16_swap across the rows of a half and v_permlane32_swap across the halves.
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
+}
 template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-    for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, MI_WAVE);
+    static_assert(WIDTH == 1 || WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16 || WIDTH == 32 || WIDTH == 64, "group width");
+    if constexpr (WIDTH >= 2) v += dpp_mov<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+    if constexpr (WIDTH >= 4) v += dpp_mov<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+    if constexpr (WIDTH >= 8) v += dpp_mov<0x141>(v);    // row_half_mirror
+    if constexpr (WIDTH >= 16) v += dpp_mov<0x140>(v);   // row_mirror
+    if constexpr (WIDTH >= 32) {
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
+    if constexpr (WIDTH >= 64) {
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    }
     return v;
 }
 
