@@ -307,40 +307,49 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     }
 
     // ---- sum the two wavefronts of each key group (fixed order), then store -------------------------
-    float* red = reinterpret_cast<float*>(smem) + (size_t)kgp * (16 * DT * 64) + lane;
+    // One exchange: the second wavefront of a pair hands its dK to the first and receives the first's dV, so each of them
+    // sums and stores one of the two tensors (half the LDS traffic and half the stores per wavefront of a one-way sum).
+    constexpr int kAccFloats = 16 * DT * 64;          // one accumulator set of one wavefront
+    static_assert(2 * 4 * kAccFloats * 4 <= SMEM_BYTES, "the exchange reuses the tile stages");
+    float* red_k = reinterpret_cast<float*>(smem) + (size_t)kgp * kAccFloats + lane;
+    float* red_v = reinterpret_cast<float*>(smem) + (size_t)(4 + kgp) * kAccFloats + lane;
+    {
+        const f32x16_t* mine = sub == 1 ? dk_acc : dv_acc;
+        float* out = sub == 1 ? red_k : red_v;
 #pragma unroll
-    for (int which = 0; which < 2; ++which) {
-        f32x16_t* acc = which == 0 ? dk_acc : dv_acc;
-        if (sub == 1) {
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) red[(dt * 16 + r) * 64] = acc[dt][r];
-        }
-        __syncthreads();
-        if (sub == 0) {
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[dt][r] += red[(dt * 16 + r) * 64];
-        }
-        __syncthreads();
+            for (int r = 0; r < 16; ++r) out[(dt * 16 + r) * 64] = mine[dt][r];
     }
+    __syncthreads();
+    if (sub == 0) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dk_acc[dt][r] += red_k[(dt * 16 + r) * 64];
+    } else {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dv_acc[dt][r] = red_v[(dt * 16 + r) * 64] + dv_acc[dt][r];
+    }
+    if (key >= p.total_k) return;
 
-    if (sub == 0 && key < p.total_k && p.hsplit > 1) {
+    if (p.hsplit > 1) {
         const int64_t prow = (((int64_t)hs * p.total_k + key) * p.nkv + kvh) * D + 4 * g;
-        const float vs = DROP ? p.drop_rscale : 1.0f;
+        const float sc = sub == 0 ? p.scale : (DROP ? p.drop_rscale : 1.0f);
+        const f32x16_t* acc = sub == 0 ? dk_acc : dv_acc;
+        float* part = sub == 0 ? p.dk_part : p.dv_part;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                f32x4_t k4, v4;
+                f32x4_t x4;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) { k4[c] = dk_acc[dt][4 * a + c] * p.scale; v4[c] = dv_acc[dt][4 * a + c] * vs; }
-                *reinterpret_cast<f32x4_t*>(p.dk_part + prow + 32 * dt + 8 * a) = k4;
-                *reinterpret_cast<f32x4_t*>(p.dv_part + prow + 32 * dt + 8 * a) = v4;
+                for (int c = 0; c < 4; ++c) x4[c] = acc[dt][4 * a + c] * sc;
+                *reinterpret_cast<f32x4_t*>(part + prow + 32 * dt + 8 * a) = x4;
             }
-    } else if (sub == 0 && key < p.total_k) {
+    } else if (sub == 0) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -349,7 +358,6 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             if (p.unrotate != 0) unrotate_acc<D>(dk_acc, p, p.pos_k[key], g);   // k was the rotated tensor
         }
         elem_t* dkr = p.dk + (int64_t)key * p.dk_st + (int64_t)kvh * p.dk_sh + 4 * g;
-        elem_t* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -357,7 +365,14 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
                 const uint32_t k0 = pack_elem2(dk_acc[dt][4 * a], dk_acc[dt][4 * a + 1]);
                 const uint32_t k1 = pack_elem2(dk_acc[dt][4 * a + 2], dk_acc[dt][4 * a + 3]);
                 *reinterpret_cast<uint2*>(dkr + 32 * dt + 8 * a) = make_uint2(k0, k1);
-                const float vs = DROP ? p.drop_rscale : 1.0f;   // dV = (P * mask / (1 - p))^T dO
+            }
+    } else {
+        const float vs = DROP ? p.drop_rscale : 1.0f;   // dV = (P * mask / (1 - p))^T dO
+        elem_t* dvr = p.dv + (int64_t)key * p.dv_st + (int64_t)kvh * p.dv_sh + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
                 const uint32_t v0 = pack_elem2(dv_acc[dt][4 * a] * vs, dv_acc[dt][4 * a + 1] * vs);
                 const uint32_t v1 = pack_elem2(dv_acc[dt][4 * a + 2] * vs, dv_acc[dt][4 * a + 3] * vs);
                 *reinterpret_cast<uint2*>(dvr + 32 * dt + 8 * a) = make_uint2(v0, v1);
