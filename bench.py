@@ -65,25 +65,42 @@ def causal_pairs(cu):
     return sum((b - a) * (b - a + 1) // 2 for a, b in zip(cu[:-1], cu[1:]))
 
 
-def time_gpu(fn, steps, warmup):
-    """Average milliseconds per call, measured with events on the current stream."""
+def time_gpu(fn, steps, warmup, stats=None):
+    """Average milliseconds per call over exactly `steps` calls bracketed by events on the current stream (the figure
+    `value` / `ms_per_step` are built from).  With a dict in `stats` every call is also bracketed by its own pair of
+    events and the median, minimum and maximum of the per-call times are stored there."""
     import torch
     for _ in range(warmup):
         fn()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)] if stats is not None else None
     torch.cuda.synchronize()
     start.record()
-    for _ in range(steps):
+    for i in range(steps):
+        if marks is not None:
+            marks[i].record()
         fn()
+    if marks is not None:
+        marks[steps].record()
     stop.record()
     torch.cuda.synchronize()
+    if marks is not None:
+        per_call = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+        stats.update(median=per_call[len(per_call) // 2], min=per_call[0], max=per_call[-1])
     return start.elapsed_time(stop) / steps
+
+
+def time_gpu_median(fn, steps, warmup):
+    """Median milliseconds per call (each call bracketed by its own events on the current stream)."""
+    st = {}
+    time_gpu(fn, max(steps, 20), warmup, st)
+    return st["median"]
 
 
 def time_gpu_graph(fn, steps, warmup):
     """Average milliseconds per call with the calls replayed from one HIP graph, so that a launch that takes the
     host longer than the kernel takes the GPU (the 20-30 us bandwidth kernels) is still timed on the GPU side.
-    Best of three replays; falls back to eager timing if the calls cannot be captured."""
+    Median of five replays; falls back to eager timing if the calls cannot be captured."""
     import torch
     try:
         side = torch.cuda.Stream()
@@ -97,17 +114,17 @@ def time_gpu_graph(fn, steps, warmup):
         with torch.cuda.graph(graph):
             for _ in range(steps):
                 fn()
-        best = float("inf")
-        for _ in range(3):
+        times = []
+        for _ in range(5):
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             start.record()
             graph.replay()
             stop.record()
             torch.cuda.synchronize()
-            best = min(best, start.elapsed_time(stop) / steps)
+            times.append(start.elapsed_time(stop) / steps)
         del graph
-        return best
+        return sorted(times)[len(times) // 2]
     except Exception as exc:  # noqa: BLE001 - any capture problem: measure eagerly instead
         print(f"[bench] graph timing unavailable ({type(exc).__name__}: {exc}); timing eagerly", file=sys.stderr)
         torch.cuda.synchronize()
@@ -226,13 +243,23 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
         fwd()
         bwd()
 
+    def step_precise():
+        o2, lse2 = ops.attention_forward(q, k, v, cu, None, True, scale, precise=True)
+        ops.attention_backward(do, q, k, v, o2, lse2, cu, None, True, scale, buffers=bufs, precise=True)
+
     res = {"pairs_per_head": pairs}
-    res["ms_step"] = time_gpu(step, steps, warmup)
+    res["ms_step"] = time_gpu(step, steps, warmup)              # mean over exactly `steps` steps: the contract's figure
+    st = {}
+    time_gpu(step, max(steps, 20), 1, st)                       # the same again with every step bracketed on its own
+    res["ms_step_median"], res["ms_step_min"], res["ms_step_max"] = st["median"], st["min"], st["max"]
     res["ms_step_graph"] = time_gpu_graph(step, steps, warmup)
-    res["ms_fwd"] = time_gpu(fwd, steps, warmup)
-    res["ms_bwd_delta"] = time_gpu(lambda: bwd(16), steps, 1)
-    res["ms_bwd_dkdv"] = time_gpu(lambda: bwd(32), steps, 1)
-    res["ms_bwd_dq"] = time_gpu(lambda: bwd(64), steps, 1)
+    res["ms_fwd"] = time_gpu_median(fwd, steps, warmup)
+    res["ms_bwd_delta"] = time_gpu_median(lambda: bwd(16), steps, 1)
+    res["ms_bwd_dkdv"] = time_gpu_median(lambda: bwd(32), steps, 1)
+    res["ms_bwd_dq"] = time_gpu_median(lambda: bwd(64), steps, 1)
+    # accuracy mode (MI_ATTN_SPLIT_P): the mode whose outputs and gradients meet max-abs 2e-2 / mean-rel 1e-3 literally
+    res["ms_step_precise"] = time_gpu(step_precise, steps, warmup)
+    step()                                                      # leave the default mode's results in the buffers
     if rot is not None:
         res["ms_fwd_fused_rotary"] = time_gpu(fwd_rot, steps, warmup)
         # training step with the rotary embedding as ops.attention runs it: k rotated by one stand-alone launch, q
@@ -251,6 +278,8 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
     res["tflops_fwd"] = 4 * flops_unit / (res["ms_fwd"] * 1e-3) / 1e12
     res["tflops_step"] = 14 * flops_unit / (res["ms_step"] * 1e-3) / 1e12
     res["tflops_step_graph"] = 14 * flops_unit / (res["ms_step_graph"] * 1e-3) / 1e12
+    res["tflops_step_precise"] = 14 * flops_unit / (res["ms_step_precise"] * 1e-3) / 1e12
+    res["precise_over_default_time"] = res["ms_step_precise"] / res["ms_step"]
     res["frac_of_bf16_peak_step"] = res["tflops_step"] / PEAK_BF16_TFLOPS
     return res
 
@@ -513,13 +542,71 @@ def cpu_baseline(seconds_budget=25.0):
             t.grad = None
 
     med1, n1 = median_time(step_c1, seconds_budget / 3, min_runs=5, max_runs=200)
+
+    # config 5 (decode): the oracle's batch-1 cached decode step (the reference's cache is batch-1, attention.py:855-857)
+    # at the config-5 layer shape on a reduced layer count, extrapolated linearly in the layers.  The caches are filled
+    # with random post-rotary K / V for a context of 4096 tokens instead of running the prefill (a decode step's cost
+    # depends on the shapes only); torch.cat grows them by one token per step as the reference does.
+    n_layers_cpu, ctx5, hid5, inter5, vocab5 = 2, 4096, 4096, 14336, 128256
+    spec5 = oracle.LayerSpec(hidden_size=hid5, num_attention_heads=32, num_kv_heads=8, qkv_in_one=False, norm_type="rms",
+                             mlp_type="swiglu", layernorm_epsilon=1e-5, rotary_base=500000, sequence_length=ctx5 + 64,
+                             causal=True, softmax_in_fp32=True, dtype=torch.bfloat16)
+    g5 = torch.Generator().manual_seed(0)
+
+    def w5(*shape):
+        return (torch.randn(shape, generator=g5) * 0.02).bfloat16()
+
+    layers5 = []
+    for _ in range(n_layers_cpu):
+        layers5.append({"self_attention.query.weight": w5(hid5, hid5), "self_attention.key.weight": w5(1024, hid5),
+                        "self_attention.value.weight": w5(1024, hid5), "self_attention.dense.weight": w5(hid5, hid5),
+                        "mlp.dense_in.weight": w5(inter5, hid5), "mlp.siglu_weight.weight": w5(inter5, hid5),
+                        "mlp.dense_out.weight": w5(hid5, inter5),
+                        "input_layernorm.weight": torch.ones(hid5, dtype=torch.bfloat16),
+                        "post_attention_layernorm.weight": torch.ones(hid5, dtype=torch.bfloat16)})
+    final5 = {"norm.weight": torch.ones(hid5, dtype=torch.bfloat16)}
+    head5 = w5(vocab5, hid5)
+    tables5 = spec5.tables()
+    cu5 = torch.tensor([0, 1], dtype=torch.int32)
+
+    def fresh_caches():
+        return [{0: (torch.randn(ctx5, 1, 8, 128, generator=g5).bfloat16(), torch.randn(ctx5, 1, 8, 128, generator=g5).bfloat16())}
+                for _ in range(n_layers_cpu)]
+
+    caches5 = fresh_caches()
+    x5 = torch.randn(1, 1, hid5, generator=g5).bfloat16()
+    step_no = [0]
+
+    @torch.no_grad()
+    def decode_layers():
+        pos = torch.tensor([[ctx5 + step_no[0] % 32]])
+        step_no[0] += 1
+        h = x5
+        for w, cache in zip(layers5, caches5):
+            h = oracle.transformer_layer(spec5, w, h, cu5, pos, tables=tables5, use_cache=True, reset_cache=False, cache=cache)
+        return h
+
+    @torch.no_grad()
+    def decode_head():
+        return torch.nn.functional.linear(oracle.final_norm(spec5, final5, x5), head5).argmax()
+
+    med_layers, n_l = median_time(decode_layers, seconds_budget / 6, min_runs=3, max_runs=30)
+    med_head, n_h = median_time(decode_head, seconds_budget / 6, min_runs=3, max_runs=30)
+    step32 = 32 * med_layers / n_layers_cpu + med_head
+    del layers5, head5, caches5
     return {"value": flops / med / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "cpu_model": model, "logical_cpus": logical, "physical_cores": physical,
             "sample": f"oracle (reference op order, bf16 + fp32 softmax) attention fwd+bwd, b1 s{s} {nq}q/{nkv}kv d{d} causal, "
                       f"median of {n_runs} runs = {med * 1e3:.1f} ms; config 1 (one layer fwd+bwd, fp32, hidden 256, 4 heads x 64, "
                       f"SwiGLU 688, batch 2 x seq 128) at full size: median of {n1} runs = {med1 * 1e3:.2f} ms "
                       f"({256 / med1:.0f} tokens/s)",
-            "config1_layer_ms": med1 * 1e3, "config1_tokens_per_s": 256 / med1}
+            "config1_layer_ms": med1 * 1e3, "config1_tokens_per_s": 256 / med1,
+            "config5_decode": {"tok_per_s_extrapolated": 1.0 / step32, "ms_per_step_32_layers_extrapolated": step32 * 1e3,
+                               "ms_per_layer_measured": med_layers / n_layers_cpu * 1e3, "ms_final_norm_lm_head_argmax": med_head * 1e3,
+                               "how": f"EXTRAPOLATED: oracle cached decode step, batch 1 (the reference's cache takes one sequence), context "
+                                      f"{ctx5}, bf16, measured on {n_layers_cpu} layers (median of {n_l} steps) and scaled linearly to 32 "
+                                      f"layers, plus final norm + LM head + argmax (median of {n_h}); one token per step, so a batch of "
+                                      f"32 prompts would be served one after the other at this rate"}}
 
 
 def main():
@@ -588,8 +675,14 @@ def main():
         "value": main_res["tflops_step"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": main_res["ms_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "attention core fwd+bwd, GQA 32q/8kv, head_dim 128, batch 1 x seq 8192, causal, bf16, fp32 softmax",
-                   "pairs_per_head": main_res["pairs_per_head"], "flop_formula": "14*d*n_q*P"},
+        "config": {"workload": "attention core fwd+bwd, GQA 32q/8kv, head_dim 128, batch 1 x seq 8192, causal, bf16, fp32 softmax; "
+                               "default mode: P rounded to bf16 before P V as the reference does (attention.py:211)",
+                   "pairs_per_head": main_res["pairs_per_head"], "flop_formula": "14*d*n_q*P",
+                   "accuracy_mode": {"what": "MI_ATTN_SPLIT_P (P and dS as two bf16 terms): meets max-abs 2e-2 / mean-rel 1e-3 "
+                                             "literally without rotary; the default mode meets them through the documented "
+                                             "second clauses of tests/parity.py",
+                                     "ms_per_step": main_res["ms_step_precise"], "value": main_res["tflops_step_precise"],
+                                     "time_over_default": main_res["precise_over_default_time"]}},
         "frac_of_bf16_peak": main_res["tflops_step"] / PEAK_BF16_TFLOPS,
         "roofline": roofline,
     }

@@ -34,11 +34,23 @@ _CHECKED: Dict[str, tuple] = {}
 def _checked_once(kind: str, t: torch.Tensor, extra: tuple, compute: Callable[[], bool]) -> bool:
     """Result of a device-side validation of tensor `t` that needs a host read-back: computed once per tensor and
     kind, so the layers of one forward share it.  The tensor is identified by address, layout and version counter,
-    and the last validated one is kept alive here, so its memory cannot be handed to another tensor meanwhile."""
-    key = (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t._version, t.device, extra)
+    and the last validated one is kept alive here, so its memory cannot be handed to another tensor meanwhile.
+
+    Limits: tensors created under torch.inference_mode() carry no version counter and are validated on every
+    call; writes through this package's raw-pointer kernels (ops.*) do not bump the counter, so a tensor that is
+    overwritten in place that way keeps its cached answer; while the current stream is being captured into a graph
+    a read-back is impossible, so a tensor that is not the one validated last is passed as valid (the kernels
+    clamp out-of-range position ids instead of faulting): validate once before the capture."""
+    try:
+        version = t._version
+    except RuntimeError:                   # inference tensors do not track a version counter
+        version = None
+    key = (t.data_ptr(), tuple(t.shape), tuple(t.stride()), version, t.device, extra)
     hit = _CHECKED.get(kind)
-    if hit is not None and hit[0] == key:
+    if version is not None and hit is not None and hit[0] == key:
         return hit[1]
+    if t.is_cuda and torch.cuda.is_current_stream_capturing():
+        return True
     ok = compute()
     _CHECKED[kind] = (key, ok, t)
     return ok
@@ -467,9 +479,10 @@ class ParallelSelfAttention(torch.nn.Module):
         return t if ok else t.contiguous()
 
     def _rows_are_single_documents(self, cu: torch.Tensor, b: int, s: int) -> bool:
-        """True when every batch row is one document.  A decode step (s == 1) needs the shape only: b + 1 strictly
-        increasing offsets that end at b are 0..b.  A prefill compares on the device and reads the answer back once
-        per cumulative-lengths tensor (all layers of a forward receive the same one), not once per layer."""
+        """True when every batch row is one document.  A decode step (s == 1) needs the shape only: cumulative lengths
+        as transformer/data/utils.py:40-74 builds them contain every multiple of s, and b + 1 of them on b tokens can
+        only be 0..b (a caller that breaks that contract is not detected here).  A prefill compares on the device and
+        reads the answer back once per cumulative-lengths tensor (all layers of a forward receive the same one)."""
         if cu.numel() != b + 1:
             return False
         if s == 1:

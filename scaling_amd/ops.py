@@ -610,7 +610,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
     order whatever its value.
     precise selects the accuracy mode of forward and backward: P and dS enter their products as two bf16 terms, which
     brings outputs and gradients within max-abs 2e-2 / mean-relative 1e-3 of the fp32 reference (the default mode
-    rounds P once to bf16 as the reference does); about 1.4 x the time; no dropout.
+    rounds P once to bf16 as the reference does); bench.py times both modes (`accuracy_mode.time_over_default`); no
+    dropout.  Exception: with `rotary` the rotated q and k are rounded once to the I/O dtype before the score product
+    in either mode, which leaves a mean-relative error of about 2e-3 against the fp32 reference (0.5 - 0.75 x what the
+    reference's own bf16 path shows there).
     """
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[2])

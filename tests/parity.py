@@ -18,16 +18,26 @@ measured rather than by what the reference's own bf16 path would tolerate:
     carries their rounding, so the ulp is taken at max(|ref|, rms of the element's row over the last dimension).
   * relative: any path that rounds probabilities to bf16 before P*V (the reference does, attention.py:211)
     sits near mean_rel 1.3e-3 against the rounded fp32 truth.  mean_rel also passes at
-    <= FLOOR_FRAC x the error of the reference's own bf16 operation order (the oracle run on bf16 tensors)
-    against the same target (clause "floor").  The kernels measure 0.35 - 0.73 x that floor (largest for a handful
-    of keys per row), so the clause fails on a regression that brings them level with the reference's bf16 path.
+    <= FLOOR_FRAC[kind] x the error of the reference's own bf16 operation order (the oracle run on bf16 tensors)
+    against the same target (clause "floor").  The bound depends on the class of tensor (`kind=`), each set at
+    least 10 % above the largest ratio measured for that class and well under 1, so the clause fails on a
+    regression that brings a kernel level with the reference's bf16 path:
+        "o"       attention outputs                      measured 0.42 - 0.45   bound 0.55
+        "grad"    dq / dk / dv                           measured 0.35 - 0.67   bound 0.75
+        "rotary"  outputs / gradients behind the fused   measured 0.47 - 0.74   bound 0.85
+                  rotary (q and k are rounded once more after the rotation, on both sides of the comparison)
+        "decode"  decode attention (largest for a        measured 0.41 - 0.73   bound 0.82
+                  handful of keys per row)
+    A check that names no kind is held to the "grad" bound.
 `literal=True` holds the relative gate to its stated form and the absolute one to max(2e-2, ONE ulp of the element's
 own value) (every tensor of the split-precision attention mode: a bf16 result that agrees with the rounded fp32
 reference to the last bit everywhere but on a rounding boundary cannot do better where |y| >= 4);
 `literal_rel=True` only the relative one (the elementwise kernels).
 `module_level=True` is for outputs of whole modules (layer, decoder stack): activations are rounded to bf16 between
 the sub-modules exactly where the reference rounds them and the projections run on the library GEMM, so the module
-can at best equal the reference's own bf16 path: both gates then pass at <= MODULE_FLOOR_FRAC x that path's error.
+can at best equal the reference's own bf16 path: both gates then pass at <= MODULE_FLOOR_FRAC x that path's error
+(measured 0.66 - 1.00; the 2 % allow for the summation order of the library GEMM, which differs between the GPU
+and the CPU run of the same operation order).
 
 Every check is recorded in RESULTS with the clause it passed by; tests/conftest.py prints the summary.
 """
@@ -37,8 +47,8 @@ import torch
 MAX_ABS_TOL = 2e-2
 MEAN_REL_TOL = 1e-3
 MAX_ULP_TOL = 2.0
-FLOOR_FRAC = 0.75
-MODULE_FLOOR_FRAC = 1.05
+FLOOR_FRAC = {"o": 0.55, "grad": 0.75, "rotary": 0.85, "decode": 0.82, None: 0.75}
+MODULE_FLOOR_FRAC = 1.02
 
 RESULTS = []   # dicts: name, max_abs, mean_rel, max_ulp, clause_abs, clause_rel, floor_mean_rel
 
@@ -75,13 +85,16 @@ def metrics(got: torch.Tensor, ref_fp32: torch.Tensor, dtype: torch.dtype = None
 
 def check(name: str, got: torch.Tensor, ref_fp32: torch.Tensor, ref_order: torch.Tensor = None,
           max_abs_tol: float = MAX_ABS_TOL, mean_rel_tol: float = MEAN_REL_TOL, verbose: bool = True,
-          literal: bool = False, literal_rel: bool = False, floor_frac: float = FLOOR_FRAC, module_level: bool = False) -> dict:
+          literal: bool = False, literal_rel: bool = False, floor_frac: float = None, module_level: bool = False,
+          kind: str = None) -> dict:
     """Asserts the gates described in the module docstring; returns the metrics with the clauses that passed.
 
     literal: both gates in their stated form only.  literal_rel: only the relative gate is held to its stated form
     (tensors whose values reach |y| >= 4, where one ulp is already over the absolute gate)."""
     m = metrics(got, ref_fp32, max_abs_tol=max_abs_tol)
     floor = metrics(ref_order, ref_fp32, got.dtype) if ref_order is not None else None
+    if floor_frac is None:
+        floor_frac = FLOOR_FRAC[kind]
     if module_level:
         assert floor is not None, "module-level checks need the reference-order run"
         floor_frac = MODULE_FLOOR_FRAC
@@ -101,7 +114,9 @@ def check(name: str, got: torch.Tensor, ref_fp32: torch.Tensor, ref_order: torch
         clause_rel = None
     m["clause_abs"], m["clause_rel"] = clause_abs, clause_rel
     m["floor_mean_rel"] = floor["mean_rel"] if floor is not None else None
-    RESULTS.append({"name": name, **{k: m[k] for k in ("max_abs", "mean_rel", "max_ulp", "clause_abs", "clause_rel", "floor_mean_rel")}})
+    m["floor_max_abs"] = floor["max_abs"] if floor is not None else None
+    RESULTS.append({"name": name, "module_level": module_level,
+                    **{k: m[k] for k in ("max_abs", "mean_rel", "max_ulp", "clause_abs", "clause_rel", "floor_mean_rel", "floor_max_abs")}})
     if verbose:
         line = (f"[parity] {name}: max_abs={m['max_abs']:.3e} mean_rel={m['mean_rel']:.3e} max_ulp={m['max_ulp']:.2f}"
                 f" -> abs:{clause_abs} rel:{clause_rel}")
@@ -133,4 +148,9 @@ def summary_lines():
                 worst[key] = (ratio, r["mean_rel"], r["floor_mean_rel"])
     for key, (ratio, mr, fl) in sorted(worst.items(), key=lambda kv: -kv[1][0])[:40]:
         lines.append(f"  floor clause: {key}: mean_rel {mr:.3e} = {ratio:.2f} x floor {fl:.3e}")
+    # whole-module outputs whose ABSOLUTE gate passed by the floor clause stay visible too
+    for r in RESULTS:
+        if r["clause_abs"] == "floor" and r["floor_max_abs"]:
+            lines.append(f"  module abs by floor clause: {r['name']}: max_abs {r['max_abs']:.3e} = "
+                         f"{r['max_abs'] / r['floor_max_abs']:.2f} x floor {r['floor_max_abs']:.3e}")
     return lines

@@ -49,10 +49,10 @@ def test_attention_fwd_bwd_parity(b, s, nq, nkv, d, causal, cuts):
     o = ops.attention(qg, kg, vg, cu.to(DEV), None, causal, scale)
     o.backward(do.to(DEV))
     torch.cuda.synchronize()
-    check("attn.o", o, ref[0], ref_o[0])
-    check("attn.dq", qg.grad, ref[1], ref_o[1])
-    check("attn.dk", kg.grad, ref[2], ref_o[2])
-    check("attn.dv", vg.grad, ref[3], ref_o[3])
+    check("attn.o", o, ref[0], ref_o[0], kind="o")
+    check("attn.dq", qg.grad, ref[1], ref_o[1], kind="grad")
+    check("attn.dk", kg.grad, ref[2], ref_o[2], kind="grad")
+    check("attn.dv", vg.grad, ref[3], ref_o[3], kind="grad")
 
 
 @pytest.mark.parametrize("b,s,nq,nkv,d,causal,cuts", [
@@ -81,7 +81,7 @@ def test_attention_accuracy_mode_meets_the_stated_tolerance(b, s, nq, nkv, d, ca
         tag = "precise" if precise else "default"
         for name, got, r, ro in (("o", o, ref[0], ref_o[0]), ("dq", qg.grad, ref[1], ref_o[1]),
                                  ("dk", kg.grad, ref[2], ref_o[2]), ("dv", vg.grad, ref[3], ref_o[3])):
-            check(f"attn.{tag}.{name}", got, r, ro, literal=precise)
+            check(f"attn.{tag}.{name}", got, r, ro, literal=precise, kind="o" if name == "o" else "grad")
 
 
 @pytest.mark.parametrize("b,s,nq,nkv,d,causal,cuts,rot", [
@@ -121,7 +121,7 @@ def test_attention_float16_fwd_bwd_parity(b, s, nq, nkv, d, causal, cuts, rot):
     assert o.dtype == torch.float16 and qg.grad.dtype == torch.float16
     for name, got, r, ro in (("o", o, ref[0], ref_o[0]), ("dq", qg.grad, ref[1], ref_o[1]),
                              ("dk", kg.grad, ref[2], ref_o[2]), ("dv", vg.grad, ref[3], ref_o[3])):
-        check(f"attn.f16.{name}", got, r, ro)
+        check(f"attn.f16.{name}", got, r, ro, kind="o" if name == "o" else "grad")
 
 
 def test_attention_mask_is_bit_exact_on_reference_known_answers():
@@ -181,8 +181,8 @@ def test_attention_fused_rotary_matches_separate_rotary():
     k2 = ops.rotary_embedding(kd, cos, sin, posd)
     sep, _ = ops.attention_forward(q2, k2, vd, cud, None, True, None)
     torch.cuda.synchronize()
-    check("attn.fused_rotary", fused, ref, ref_o)
-    check("attn.separate_rotary", sep, ref, ref_o)
+    check("attn.fused_rotary", fused, ref, ref_o, kind="rotary")
+    check("attn.separate_rotary", sep, ref, ref_o, kind="rotary")
     # same rounding points (rotate in fp32, round once to bf16); only fma contraction may differ
     diff = (fused.float() - sep.float()).abs()
     assert float(diff.max()) <= 2e-2 and float((diff > 0).float().mean()) < 0.02
@@ -245,7 +245,7 @@ def test_attention_with_rotary_fwd_bwd_parity(kind, b, s, nq, nkv, d, cuts, p_dr
     torch.cuda.synchronize()
     for name, got, r, ro in (("o", o, ref[0], ref_o[0]), ("dq", qg.grad, ref[1], ref_o[1]),
                              ("dk", kg.grad, ref[2], ref_o[2]), ("dv", vg.grad, ref[3], ref_o[3])):
-        check(f"attn.rotary[{kind}].{name}", got, r, ro)
+        check(f"attn.rotary[{kind}].{name}", got, r, ro, kind="rotary")
     # without autograd the same kernels run (minus the copy of the rotated q): same output bits
     with torch.no_grad():
         o2 = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale, rotary=(*dev_tabs, posd, posd), dropout_p=p_drop, dropout_seed=seed)
@@ -304,10 +304,10 @@ def test_attention_with_separate_key_lengths(causal, nq, nkv, d):
     o = ops.attention(qg, kg, vg, cu_q.to(DEV), cu_k.to(DEV), causal, scale)
     o.backward(do.to(DEV))
     torch.cuda.synchronize()
-    check("cross.o", o, ref[0], ref_o[0])
-    check("cross.dq", qg.grad, ref[1], ref_o[1])
-    check("cross.dk", kg.grad, ref[2], ref_o[2])
-    check("cross.dv", vg.grad, ref[3], ref_o[3])
+    check("cross.o", o, ref[0], ref_o[0], kind="o")
+    check("cross.dq", qg.grad, ref[1], ref_o[1], kind="grad")
+    check("cross.dk", kg.grad, ref[2], ref_o[2], kind="grad")
+    check("cross.dv", vg.grad, ref[3], ref_o[3], kind="grad")
     if causal:   # document 5: 10 queries, 4 keys -> queries 0..5 have no key
         a = int(cu_q[5])
         assert torch.count_nonzero(o[a:a + 6]) == 0 and torch.count_nonzero(qg.grad[a:a + 6]) == 0
@@ -357,7 +357,7 @@ def test_attention_fused_interleaved_rotary_matches_separate_rotary(d, flags):
     k2 = ops.rotary_embedding_complex(kd, real, imag, posd)
     sep, lse_s = ops.attention_forward(q2, k2, vd, cud, None, True, None, flags=flags)
     torch.cuda.synchronize()
-    check("attn.fused_interleaved_rotary", fused, ref, ref_o)
+    check("attn.fused_interleaved_rotary", fused, ref, ref_o, kind="rotary")
     assert torch.equal(fused, sep) and torch.equal(lse_f, lse_s)
     # tables of the wrong shape or type are refused before the launch
     with pytest.raises(AssertionError):
@@ -401,7 +401,7 @@ def test_attention_strided_views_of_fused_qkv():
     ref_o = U.oracle_attention(qkv[..., :d], qkv[..., d:2 * d], qkv[..., 2 * d:], cu, b, s, True, 1 / math.sqrt(d), torch.bfloat16)
     qd = qkv.to(DEV)
     o, _ = ops.attention_forward(qd[..., :d], qd[..., d:2 * d], qd[..., 2 * d:], cu.to(DEV))
-    check("attn.o(strided)", o, ref, ref_o)
+    check("attn.o(strided)", o, ref, ref_o, kind="o")
 
 
 def test_attention_rejects_unsupported_input():
@@ -437,7 +437,7 @@ def test_attention_forward_tilings_agree_with_oracle(flags, rot):
     rotary = (tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV), pos.to(DEV)) if rot else None
     o, _ = ops.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), None, True, scale, rotary=rotary, flags=flags)
     torch.cuda.synchronize()
-    check(f"attn.o(flags={flags},rot={rot})", o, ref, ref_o)
+    check(f"attn.o(flags={flags},rot={rot})", o, ref, ref_o, kind="rotary" if rot else "o")
 
 
 def test_attention_medium_multi_tile_backward():
@@ -452,10 +452,10 @@ def test_attention_medium_multi_tile_backward():
     o = ops.attention(qg, kg, vg, cu.to(DEV), None, True, scale)
     o.backward(do.to(DEV))
     torch.cuda.synchronize()
-    check("attn1k.o", o, ref[0], ref_o[0])
-    check("attn1k.dq", qg.grad, ref[1], ref_o[1])
-    check("attn1k.dk", kg.grad, ref[2], ref_o[2])
-    check("attn1k.dv", vg.grad, ref[3], ref_o[3])
+    check("attn1k.o", o, ref[0], ref_o[0], kind="o")
+    check("attn1k.dq", qg.grad, ref[1], ref_o[1], kind="grad")
+    check("attn1k.dk", kg.grad, ref[2], ref_o[2], kind="grad")
+    check("attn1k.dv", vg.grad, ref[3], ref_o[3], kind="grad")
 
 
 @pytest.mark.parametrize("name,b,s,nq,nkv,docs", [("config2", 4, 2048, 32, 32, False), ("config3", 1, 8192, 32, 8, True)])
@@ -483,7 +483,7 @@ def test_attention_full_size_properties(name, b, s, nq, nkv, docs):
         kvh = head // (nq // nkv)
         ref = U.rows_reference(q, k, v, lo_hi, rows, head, kvh, scale)
         ref_o = U.rows_reference(q, k, v, lo_hi, rows, head, kvh, scale, reference_bf16_order=True)
-        check(f"{name}.rows.head{head}", o[rows, head], ref, ref_o)
+        check(f"{name}.rows.head{head}", o[rows, head], ref, ref_o, kind="o")
     ones = torch.ones_like(vd)
     o1, _ = ops.attention_forward(qd, kd, ones, cud, None, True, scale)
     assert float((o1.float() - 1).abs().max()) <= 2 ** -7
@@ -516,7 +516,7 @@ def test_attention_dropout_matches_oracle_with_the_same_mask(b, s, nq, nkv, d, c
     torch.cuda.synchronize()
     for name, got, r, ro in (("o", o, ref[0], ref_o[0]), ("dq", qg.grad, ref[1], ref_o[1]),
                              ("dk", kg.grad, ref[2], ref_o[2]), ("dv", vg.grad, ref[3], ref_o[3])):
-        check(f"attn.dropout.{name}", got, r, ro)
+        check(f"attn.dropout.{name}", got, r, ro, kind="o" if name == "o" else "grad")
     # the mask really dropped something, the same seed reproduces the result, another seed does not
     plain = ops.attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), None, causal, scale)
     assert not torch.equal(plain, o.detach())

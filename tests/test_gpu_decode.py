@@ -59,7 +59,7 @@ def test_decode_parity(B, nq, nkv, d, max_ctx, lens, n_splits):
     ref_o = _oracle_decode(q, kc, vc, ctx, scale, torch.bfloat16)
     out = ops.decode_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), ctx.to(DEV), softmax_scale=scale, n_splits=n_splits)
     torch.cuda.synchronize()
-    check("decode.o", out, ref, ref_o)
+    check("decode.o", out, ref, ref_o, kind="decode")
 
 
 def test_decode_append_and_fused_rotary():
@@ -89,7 +89,7 @@ def test_decode_append_and_fused_rotary():
     out = ops.decode_attention(q.to(DEV), kcd, vcd, ctx.to(DEV), k_new.to(DEV), v_new.to(DEV),
                                rotary=(tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV)), softmax_scale=scale)
     torch.cuda.synchronize()
-    check("decode.o(append+rotary)", out, ref, ref_o)
+    check("decode.o(append+rotary)", out, ref, ref_o, kind="decode")
     # the cache was updated in place: only the appended rows changed, and they hold the rotated key
     for b in range(B):
         kd = (kcd[b, lens[b] - 1].float().cpu() - kr[b].float()).abs()
@@ -137,7 +137,7 @@ def test_decode_append_and_fused_interleaved_rotary(B, nq, nkv, d):
     k2 = ops.rotary_embedding_complex(knd, real, imag, posd)
     sep = ops.decode_attention(q2, kc2, vc2, ctxd, k2, vnd, softmax_scale=scale)
     torch.cuda.synchronize()
-    check("decode.o(append+interleaved rotary)", fused, ref, ref_o)
+    check("decode.o(append+interleaved rotary)", fused, ref, ref_o, kind="decode")
     assert torch.equal(fused, sep) and torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
     for b in range(B):
         kd = (kc1[b, lens[b] - 1].float().cpu() - kr[b].float()).abs()
@@ -210,5 +210,5 @@ def test_decode_float16_parity(B, nq, nkv, d, max_ctx, lens):
     out = ops.decode_attention(q.to(DEV), kcd, vcd, ctx.to(DEV), k_new.to(DEV), v_new.to(DEV), softmax_scale=scale)
     torch.cuda.synchronize()
     assert out.dtype == torch.float16
-    check("decode.f16.o", out, ref, ref_o)
+    check("decode.f16.o", out, ref, ref_o, kind="decode")
     assert torch.equal(kcd.cpu(), kc_ref) and torch.equal(vcd.cpu(), vc_ref)

@@ -74,10 +74,10 @@ def test_attention_fwd_bwd_full_size_against_oracle_slices(name, b, s, nq, nkv, 
         ref_o = _slice_reference(q, k, v, do, cu, b, s, heads, kvh, scale, torch.bfloat16, rot_ref)
         lit = precise and not rotary
         tag = f"{name}.precise" if precise else name
-        check(f"{tag}.o[kv{kvh}]", o[:, heads], ref[0], ref_o[0], literal=lit)
-        check(f"{tag}.dq[kv{kvh}]", qg.grad[:, heads], ref[1], ref_o[1], literal=lit)
-        check(f"{tag}.dk[kv{kvh}]", kg.grad[:, kvh], ref[2], ref_o[2], literal=lit)
-        check(f"{tag}.dv[kv{kvh}]", vg.grad[:, kvh], ref[3], ref_o[3], literal=lit)
+        check(f"{tag}.o[kv{kvh}]", o[:, heads], ref[0], ref_o[0], literal=lit, kind="rotary" if rotary else "o")
+        check(f"{tag}.dq[kv{kvh}]", qg.grad[:, heads], ref[1], ref_o[1], literal=lit, kind="rotary" if rotary else "grad")
+        check(f"{tag}.dk[kv{kvh}]", kg.grad[:, kvh], ref[2], ref_o[2], literal=lit, kind="rotary" if rotary else "grad")
+        check(f"{tag}.dv[kv{kvh}]", vg.grad[:, kvh], ref[3], ref_o[3], literal=lit, kind="rotary" if rotary else "grad")
 
 
 @pytest.mark.timeout(600)
@@ -107,7 +107,7 @@ def test_decode_attention_config5_shape():
         return torch.stack(outs)
 
     rows = list(range(B))
-    check("decode.config5.o", out[rows], ref_for(rows, torch.float32), ref_for(rows, torch.bfloat16))
+    check("decode.config5.o", out[rows], ref_for(rows, torch.float32), ref_for(rows, torch.bfloat16), kind="decode")
 
 
 @pytest.mark.timeout(900)

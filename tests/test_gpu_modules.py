@@ -222,9 +222,79 @@ def test_batched_cached_decode_equals_single_sequences(tmp_path):
 
 
 def test_index_construction_on_device_is_bit_exact():
-    ids = torch.tensor([[1, 2, 3, 0, 1, 2], [1, 2, 3, 4, 5, 6], [1, 2, 3, 4, 5, 0]], device=DEV)
-    assert D.get_cumulative_seq_lengths(ids).tolist() == [0, 4, 6, 12, 18]
-    assert D.get_position_ids(ids).tolist() == [[0, 1, 2, 3, 0, 1], [0, 1, 2, 3, 4, 5], [0, 1, 2, 3, 4, 5]]
+    """Every integer helper of transformer/data/utils.py:4-108 and attention.py:72-73 on device tensors, against the
+    known answers the reference's own tests hold and against the oracle on random token ids."""
+    from tests.golden import known_answers as KA
+    ids = torch.tensor(KA.TOKEN_IDS, device=DEV)
+    cu = D.get_cumulative_seq_lengths(ids)
+    assert cu.is_cuda and cu.dtype == torch.int32 and cu.tolist() == KA.CU_WITH_RESET
+    assert D.get_cumulative_seq_lengths(ids, reset_attention_mask=False).tolist() == KA.CU_WITHOUT_RESET
+    pos = D.get_position_ids(ids)
+    assert pos.is_cuda and pos.dtype == torch.int64 and pos.tolist() == KA.POSITION_IDS_WITH_RESET
+    assert D.get_position_ids(ids, reset_position_ids=False).tolist() == KA.POSITION_IDS_WITHOUT_RESET
+    # padding of the cumulative lengths to a fixed length and back (data/utils.py:4-37)
+    padded = D.add_cumulative_seq_lengths_padding(torch.tensor(KA.PADDING_INPUT, dtype=torch.int32, device=DEV), KA.PADDING_PAD_TO)
+    assert padded.is_cuda and padded.dtype == torch.int32 and padded.tolist() == KA.PADDING_EXPECTED
+    stripped = D.remove_cumulative_seq_lengths_padding(padded)
+    assert stripped.is_cuda and stripped.dtype == torch.int32 and stripped.tolist() == KA.PADDING_INPUT
+    b, s = ids.shape
+    roundtrip = D.remove_cumulative_seq_lengths_padding(D.add_cumulative_seq_lengths_padding(cu, b * (s + 1)))
+    assert torch.equal(roundtrip, cu)
+    # longest document (attention.py:72-73)
+    assert D.get_max_seq_length(torch.tensor(KA.MASK_CU_SEQLENS, dtype=torch.int32, device=DEV)) == KA.MASK_MAX_SEQ_LENGTH
+    assert D.get_max_seq_length(cu) == 6
+    g = torch.Generator().manual_seed(3)
+    for _ in range(10):
+        bb, ss = int(torch.randint(1, 6, (1,), generator=g)), int(torch.randint(1, 70, (1,), generator=g))
+        host = torch.randint(0, 4, (bb, ss), generator=g)
+        for reset in (True, False):
+            got, want = D.get_cumulative_seq_lengths(host.to(DEV), reset), oracle.get_cumulative_seq_lengths(host, reset)
+            assert got.dtype == want.dtype and torch.equal(got.cpu(), want)
+            assert D.get_max_seq_length(got) == oracle.get_max_seq_length(want)
+            pad_to = bb * (ss + 1)
+            pg = D.add_cumulative_seq_lengths_padding(got, pad_to)
+            assert torch.equal(pg.cpu(), oracle.add_cumulative_seq_lengths_padding(want, pad_to))
+            assert torch.equal(D.remove_cumulative_seq_lengths_padding(pg).cpu(), want)
+            got, want = D.get_position_ids(host.to(DEV), reset), oracle.get_position_ids(host, reset)
+            assert got.dtype == want.dtype and torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("case", ["gqa_documents", "mha_bidirectional", "decode_step", "cross_length"])
+def test_scaled_dot_product_attention_reference_layout(case):
+    """ScaledDotProductAttention.forward in the reference's own layout (attention.py:280-395: query [s_q, b, n, d],
+    key / value [s_k, b, n_kv, d] -> [(b n), s_q, d]) against oracle.multi_head_attention, including the branch for
+    key.shape[0] != s_q.  The reference's dense mask is [b, 1, s_q, s_q] (attention.py:166-168), which only
+    broadcasts over s_k keys when s_q == 1 (a cached decode step, nothing masked); for s_q > 1 the kernels align the
+    causal diagonal to the end of the keys and the oracle receives that mask explicitly."""
+    from scaling_amd.nn import ScaledDotProductAttention
+    from tests import attn_utils as U
+    print("case sdpa.forward", case, flush=True)
+    s_q, s_k, b, n, nkv, d, causal, cuts = {
+        "gqa_documents": (96, 96, 2, 4, 2, 64, True, (40, 96 + 17)),
+        "mha_bidirectional": (80, 80, 3, 2, 2, 128, False, (33,)),
+        "decode_step": (1, 37, 3, 4, 1, 64, True, ()),
+        "cross_length": (24, 88, 2, 4, 2, 64, True, ()),
+    }[case]
+    g = torch.Generator().manual_seed(11)
+    query = torch.randn(s_q, b, n, d, generator=g).bfloat16()
+    key = torch.randn(s_k, b, nkv, d, generator=g).bfloat16()
+    value = torch.randn(s_k, b, nkv, d, generator=g).bfloat16()
+    cu = U.make_cu(b, s_q, cuts)
+    cfg = C.MaskedSoftmaxConfig(kernel="hip", softmax_in_fp32=True, scale=1.5)
+    sdpa = ScaledDotProductAttention(head_dim=d, dropout_p=0.0, masked_softmax_config=cfg, causal=causal).eval()
+    out = sdpa(query.to(DEV), key.to(DEV), value.to(DEV), cu.to(DEV))
+    assert out.shape == (b * n, s_q, d) and out.dtype == torch.bfloat16
+    mask = None
+    if s_k != s_q and s_q > 1:
+        allowed = torch.ones(s_q, s_k, dtype=torch.bool).tril(diagonal=s_k - s_q)
+        mask = (~allowed).view(1, 1, s_q, s_k).expand(b, 1, s_q, s_k)
+
+    def ref(dtype):
+        return oracle.multi_head_attention(query.to(dtype), oracle.repeat_kv(key.to(dtype), n // nkv),
+                                           oracle.repeat_kv(value.to(dtype), n // nkv), cu, causal, 1 / d ** 0.5,
+                                           softmax_in_fp32=True, softmax_scale=1.5, mask=mask)
+
+    check(f"sdpa.forward[{case}]", out, ref(torch.float32), ref(torch.bfloat16), kind="decode" if s_q == 1 else "o")
 
 
 @pytest.mark.parametrize("max_tokens", [1, 2, 3, 9])

@@ -184,3 +184,32 @@ def test_unsupported_options_raise():
     with pytest.raises(NotImplementedError):
         TransformerLayer(_arch(umup={"enable": True}), 0, device=CPU)
     assert RMSNorm(16, CPU).weight.tolist() == [1.0] * 16
+
+
+def test_checked_once_handles_inference_tensors_and_caches_by_version():
+    """The validation cache keys on the version counter; tensors made under torch.inference_mode() have none and
+    must be validated on every call instead of raising."""
+    from scaling_amd import nn as N
+    calls = []
+
+    def compute():
+        calls.append(1)
+        return True
+
+    t = torch.arange(4)
+    assert N._checked_once("test_kind", t, (1,), compute) and N._checked_once("test_kind", t, (1,), compute)
+    assert len(calls) == 1                      # second call is a cache hit
+    t.add_(1)                                   # in-place write bumps the version: validated again
+    assert N._checked_once("test_kind", t, (1,), compute) and len(calls) == 2
+    with torch.inference_mode():
+        u = torch.arange(4)
+        assert N._checked_once("test_kind", u, (1,), compute) and N._checked_once("test_kind", u, (1,), compute)
+    assert len(calls) == 4                      # no version counter: no caching, no exception
+    att = ParallelSelfAttention(256, 4, C.MaskedSoftmaxConfig(kernel="hip"), dtype=torch.bfloat16, device=CPU,
+                                rotary_config=C.RotaryConfig(dimensions=64, max_seq_length=16))
+    with torch.inference_mode():
+        att._check_positions(torch.arange(16))
+        with pytest.raises(IndexError):
+            att._check_positions(torch.arange(17))
+        assert att._rows_are_single_documents(torch.tensor([0, 8, 16], dtype=torch.int32), 2, 8)
+        assert not att._rows_are_single_documents(torch.tensor([0, 5, 16], dtype=torch.int32), 2, 8)
