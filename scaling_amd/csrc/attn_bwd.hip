@@ -449,7 +449,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     constexpr int BN = 64;
     constexpr int KS = D / 16;
     constexpr int DT = D / 32;
-    constexpr int NS = 3;                 // LDS stages per operand
+    constexpr int NS = 4;                 // LDS stages per operand
     using Tile = LdsTile<D>;
     constexpr int RB = Tile::RB;
     constexpr int TILE = Tile::kBytes;
@@ -529,7 +529,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     };
     issue_tile(0);
     issue_tile(1);
-    if (n_tiles > 1) wait_vmcnt<IPW>(); else wait_vmcnt<0>();
+    issue_tile(2);
+    if (n_tiles > 2) wait_vmcnt<2 * IPW>(); else if (n_tiles > 1) wait_vmcnt<IPW>(); else wait_vmcnt<0>();
     __syncthreads();
 
     const float c2 = p.scale_log2;
@@ -544,7 +545,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     }
     for (int it = 0; it < n_tiles; ++it) {
         const int kt = kt0 + it * BN;
-        issue_tile(it + 2);
+        issue_tile(it + 3);
 
         if ((kt < wmax) && (kt + BN > wmin)) {
             const char* kt_ = k_t + (it % NS) * TILE;
@@ -636,8 +637,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
                 });
             }
         }
-        // tile it+1 must have landed; tile it+2 (just issued) may still be in flight
-        if (it + 2 < n_tiles) wait_vmcnt<IPW>(); else wait_vmcnt<0>();
+        // tile it+1 must have landed; tiles it+2 and it+3 (just issued) may still be in flight
+        if (it + 3 < n_tiles) wait_vmcnt<2 * IPW>(); else if (it + 2 < n_tiles) wait_vmcnt<IPW>(); else wait_vmcnt<0>();
         __syncthreads();
     }
 
