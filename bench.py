@@ -316,6 +316,21 @@ def bandwidth_cases(steps, warmup):
     both("layernorm_bwd", 3 * N * H * 2, lambda k: (lambda: ops.layer_norm_backward(xs[k], w, dys[k], 1e-5, True, stats[k])),
          lambda: ops.layer_norm_backward(x, w, dy, 1e-5, True, ln_stats))
     del xs, dys, stats
+    # the same kernels on 8 x the rows (one launch streams 1.1 - 1.6 GB): the launch's ramp and tail and the dweight
+    # reduction launch weigh an eighth as much, so this is the steady-state rate of the same code
+    N8 = 8 * N
+    x8 = torch.randn(N8, H, generator=g).bfloat16().to(dev)
+    dy8 = torch.randn(N8, H, generator=g).bfloat16().to(dev)
+    st8 = ops.layer_norm_forward(x8, w, bias, 1e-5, save_stats=True)[1]
+    for name, nbytes, call in (
+            ("rmsnorm_fwd", 2 * N8 * H * 2, lambda: ops.rms_norm_forward(x8, w, 1e-5)),
+            ("rmsnorm_bwd", 3 * N8 * H * 2, lambda: ops.rms_norm_backward(x8, w, dy8, 1e-5)),
+            ("layernorm_fwd", 2 * N8 * H * 2, lambda: ops.layer_norm_forward(x8, w, bias, 1e-5)),
+            ("layernorm_bwd", 3 * N8 * H * 2, lambda: ops.layer_norm_backward(x8, w, dy8, 1e-5, True, st8))):
+        ms8 = time_gpu_graph(call, max(5, steps // 2), 2)
+        out[name]["ms_8x_rows"] = ms8
+        out[name]["GBs_8x_rows"] = nbytes / ms8 / 1e6
+    del x8, dy8, st8
     a = torch.randn(N, I, generator=g).bfloat16().to(dev)
     gate = torch.randn(N, I, generator=g).bfloat16().to(dev)
     dout = torch.randn(N, I, generator=g).bfloat16().to(dev)
@@ -344,7 +359,12 @@ def bandwidth_cases(steps, warmup):
     pos = torch.arange(N, dtype=torch.int64, device=dev) % 4096
     both("rotary", 2 * N * (nq + nkv) * d * 2 + 8 * N, lambda k: (lambda: ops.rotary_embedding(qks[k], cos, sin, pos)),
          lambda: ops.rotary_embedding(qks[0], cos, sin, pos))
-    del qks
+    qk8 = torch.randn(8 * N, nq + nkv, d, generator=g).bfloat16().to(dev)
+    pos8 = torch.arange(8 * N, dtype=torch.int64, device=dev) % 4096
+    ms8 = time_gpu_graph(lambda: ops.rotary_embedding(qk8, cos, sin, pos8), max(5, steps // 2), 2)
+    out["rotary"]["ms_8x_rows"] = ms8
+    out["rotary"]["GBs_8x_rows"] = (2 * 8 * N * (nq + nkv) * d * 2 + 8 * 8 * N) / ms8 / 1e6
+    del qks, qk8, pos8
     B, ctx, max_ctx = 32, 4096, 4352
     # head-major storage viewed as [batch, token, kv head, d]: the layout scaling_amd.nn.KVCache allocates
     kc = torch.randn(B, nkv, max_ctx, d, generator=g).bfloat16().to(dev).transpose(1, 2)
@@ -363,7 +383,66 @@ def bandwidth_cases(steps, warmup):
     del src, dst
     for v_ in out.values():
         v_["frac_of_hbm_peak"] = v_["GBs"] / PEAK_HBM_GBS
+        if "GBs_8x_rows" in v_:
+            v_["frac_of_hbm_peak_8x_rows"] = v_["GBs_8x_rows"] / PEAK_HBM_GBS
     return out
+
+
+def profile_kernels(repeats=3):
+    """Each HBM-bound kernel a few times, eagerly, at the sizes bandwidth_cases() times them at, plus a plain 1 GiB device
+    copy: the run that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes are taken over (the copy gives the scale of the
+    counters).  Returns the algorithmic bytes per launch by kernel family."""
+    import torch
+    from scaling_amd import ops
+    dev = "cuda"
+    g = torch.Generator().manual_seed(1)
+    N, H, I = 8192, 4096, 14336
+    w = torch.ones(H, dtype=torch.bfloat16, device=dev)
+    bias = torch.zeros(H, dtype=torch.bfloat16, device=dev)
+    x = torch.randn(N, H, generator=g).bfloat16().to(dev)
+    dy = torch.randn(N, H, generator=g).bfloat16().to(dev)
+    _, stats = ops.layer_norm_forward(x, w, bias, 1e-5, save_stats=True)
+    a = torch.randn(N, I, generator=g).bfloat16().to(dev)
+    gate = torch.randn(N, I, generator=g).bfloat16().to(dev)
+    dout = torch.randn(N, I, generator=g).bfloat16().to(dev)
+    rows, vocab = 4096, 128256
+    logits = (torch.randn(rows, vocab, generator=torch.Generator(device=dev).manual_seed(2), device=dev) * 2).bfloat16()
+    targets = torch.randint(0, vocab, (rows,), device=dev)
+    row_scale = torch.full((rows,), 1.0 / rows, device=dev)
+    dlogits = torch.empty_like(logits)
+    nq, nkv, d = 32, 8, 128
+    qk = torch.randn(N, nq + nkv, d, generator=g).bfloat16().to(dev)
+    cos, sin = _rotary_tables(d, 8192, 500000, dev)
+    pos = torch.arange(N, dtype=torch.int64, device=dev) % 4096
+    B, ctx, max_ctx = 32, 4096, 4352
+    kc = torch.randn(B, nkv, max_ctx, d, generator=g).bfloat16().to(dev).transpose(1, 2)
+    vc = torch.randn(B, nkv, max_ctx, d, generator=g).bfloat16().to(dev).transpose(1, 2)
+    q1 = torch.randn(B, nq, d, generator=g).bfloat16().to(dev)
+    ctx_len = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    wsd = ops.decode_workspace(B, nq, d, max_ctx, dev)
+    od = torch.empty_like(q1)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    calls = [
+        ("rmsnorm_fwd", 2 * N * H * 2, lambda: ops.rms_norm_forward(x, w, 1e-5)),
+        ("rmsnorm_bwd", 3 * N * H * 2, lambda: ops.rms_norm_backward(x, w, dy, 1e-5)),
+        ("layernorm_fwd", 2 * N * H * 2, lambda: ops.layer_norm_forward(x, w, bias, 1e-5)),
+        ("layernorm_bwd", 3 * N * H * 2, lambda: ops.layer_norm_backward(x, w, dy, 1e-5, True, stats)),
+        ("swiglu_fwd", 3 * N * I * 2, lambda: ops.swiglu_forward(a, gate)),
+        ("swiglu_bwd", 5 * N * I * 2, lambda: ops.swiglu_backward(a, gate, dout)),
+        ("gelu_fwd", 2 * N * I * 2, lambda: ops.gelu_forward(a)),
+        ("gelu_bwd", 3 * N * I * 2, lambda: ops.gelu_backward(a, dout)),
+        ("cross_entropy_fwd", rows * vocab * 2, lambda: ops.cross_entropy_forward(logits, targets)),
+        ("cross_entropy_fwd_bwd", 2 * rows * vocab * 2, lambda: ops.cross_entropy_forward(logits, targets, row_scale, dlogits)),
+        ("rotary", 2 * N * (nq + nkv) * d * 2 + 8 * N, lambda: ops.rotary_embedding(qk, cos, sin, pos)),
+        ("decode_attention", 2 * B * ctx * nkv * d * 2, lambda: ops.decode_attention(q1, kc, vc, ctx_len, workspace=wsd, out=od)),
+        ("device_copy_1GiB", 2 * (1 << 30), lambda: dst.copy_(src)),
+    ]
+    for _, _, call in calls:
+        for _ in range(repeats):
+            call()
+            torch.cuda.synchronize()
+    return {name: nbytes for name, nbytes, _ in calls}
 
 
 def layer_case(steps, warmup):
@@ -620,6 +699,10 @@ def main():
     ap.add_argument("--decode-only", action="store_true",
                     help="only run the config-5 decode workload (for a kernel trace of the decode step)")
     ap.add_argument("--decode-layers", type=int, default=32, help="layers of the config-5 model")
+    ap.add_argument("--bandwidth-only", action="store_true",
+                    help="only run the HBM-bound kernels (norms, SwiGLU, GELU, cross entropy, rotary, decode attention)")
+    ap.add_argument("--profile-kernels", action="store_true",
+                    help="only launch every HBM-bound kernel three times (the run the FETCH_SIZE / WRITE_SIZE counter passes are taken over)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 1 GiB device copy (reference point for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -639,6 +722,14 @@ def main():
         ms = time_gpu(lambda: dst.copy_(src), args.steps, args.warmup)
         print(json.dumps({"calibration": "device copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "ms": ms,
                           "GBs": 2 * (1 << 30) / ms / 1e6}))
+        return
+
+    if args.profile_kernels:
+        print(json.dumps({"algorithmic_bytes_per_launch": profile_kernels()}))
+        return
+
+    if args.bandwidth_only:
+        print(json.dumps({"bandwidth_kernels": bandwidth_cases(args.steps, args.warmup)}))
         return
 
     if args.decode_only:
