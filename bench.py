@@ -284,6 +284,35 @@ def attention_case(b, s, nq, nkv, d, cu_list, steps, warmup, seed=0, rotary=Fals
     return res
 
 
+def attention_float32_case(steps, warmup):
+    """The float32 attention core (the reference's default precision; exact-fp32 kernels on the fp32 matrix pipe) at GQA
+    32 / 8 heads of 128, one causal sequence of 4096 tokens: forward + backward time and the fraction of the fp32 MFMA peak."""
+    import torch
+    from scaling_amd import ops
+    dev = "cuda"
+    g = torch.Generator().manual_seed(5)
+    T, nq, nkv, d = 4096, 32, 8, 128
+    q = torch.randn(T, nq, d, generator=g).to(dev)
+    k = torch.randn(T, nkv, d, generator=g).to(dev)
+    v = torch.randn(T, nkv, d, generator=g).to(dev)
+    do = torch.randn(T, nq, d, generator=g).to(dev)
+    cu = torch.tensor([0, T], dtype=torch.int32, device=dev)
+    scale = 1.0 / math.sqrt(d)
+    o, lse = ops.attention_forward(q, k, v, cu, None, True, scale)
+    bufs = None
+
+    def step():
+        o2, lse2 = ops.attention_forward(q, k, v, cu, None, True, scale)
+        ops.attention_backward(do, q, k, v, o2, lse2, cu, None, True, scale, buffers=bufs)
+
+    ms = time_gpu(step, max(3, steps // 4), 1)
+    ms_fwd = time_gpu(lambda: ops.attention_forward(q, k, v, cu, None, True, scale), max(3, steps // 4), 1)
+    flops = 14 * d * nq * (T * (T + 1) // 2)
+    return {"ms_step": ms, "ms_fwd": ms_fwd, "tflops_step": flops / (ms * 1e-3) / 1e12,
+            "frac_of_fp32_mfma_peak": flops / (ms * 1e-3) / 1e12 / 157.3,
+            "note": "float32 q / k / v / o, fp32 probabilities; completeness path, one wavefront per 32 x 32 tile"}
+
+
 def bandwidth_cases(steps, warmup):
     """RMSNorm / SwiGLU / rotary at the config-4 sizes and decode attention at the config-5 layer shape."""
     import torch
@@ -757,6 +786,7 @@ def main():
         cu3 = random_docs_cu(8192, 256, 2048, seed=0).tolist()
         extra["config3_gqa_packed_rotary_s8192"] = attention_case(1, 8192, 32, 8, 128, cu3, args.steps, args.warmup, seed=3, rotary=True)
         extra["config3_gqa_packed_rotary_s8192"]["n_docs"] = len(cu3) - 1
+        extra["attention_float32_gqa32x8_d128_s4096"] = attention_float32_case(args.steps, args.warmup)
         extra.update(bandwidth_cases(args.steps, args.warmup))
         extra["config4_layer_fwd_bwd_b2_s4096_h4096"] = layer_case(max(5, args.steps // 2), 3)
         extra["config5_decode_8b_b32_ctx4096"] = decode_case(args.decode_steps, layers=args.decode_layers)

@@ -184,7 +184,10 @@ int mi_rotary_complex(const void* x, void* out, const float* cos, const float* s
  * one of core/nn/rotary.py:59-90 instead: pairs (2i, 2i+1), fp32 tables [rotary_table_rows,
  * head_dim / 2] (real and imaginary part of freqs_cis), fp32 arithmetic, one rounding -- the same
  * bits as mi_rotary_complex followed by the plain call.  Fused rotary needs head_dim in {64, 128}.
- * Supported: dtype MI_BF16 or MI_F16 (the same kernels built on the bf16 / f16 MFMA), head_dim in {32, 64, 96, 128}.
+ * Supported: dtype MI_BF16 or MI_F16 (the same kernels built on the bf16 / f16 MFMA), head_dim in {32, 64, 96, 128};
+ * dtype MI_F32 (the reference's default `precision`, transformer/context/config.py:346): separate kernels on the
+ * fp32 MFMA with fp32 probabilities throughout (probs.to(value.dtype) is the identity there), same masks, layouts,
+ * lse and workspace contract, strides multiples of 4 elements, no dropout, no fused rotary, flags ignored.
  * Algorithmic work: 4 * head_dim * n_q_heads * P flop forward, 10 * head_dim * n_q_heads * P backward,
  * P = number of allowed (query, key) pairs per head.
  * ------------------------------------------------------------------------------------------ */

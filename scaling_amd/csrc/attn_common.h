@@ -480,10 +480,11 @@ __device__ __forceinline__ int xcd_remap(int linear, int total) {
 int mi_compute_units();
 int mi_static_scratch(void** out, size_t* bytes);
 
-static inline int mi_attn_validate(const mi_attn_args* a, const char* who) {
+// want_dtype / vec: the element type this build of the kernels takes and its elements per 128-bit access
+static inline int mi_attn_validate(const mi_attn_args* a, const char* who, int want_dtype = MI_ELEM_DTYPE, int vec = 8) {
     if (!a) return mi_fail(MI_E_NULL, "%s: args is null", who);
     if (!a->q || !a->k || !a->v || !a->cu_seqlens_q) return mi_fail(MI_E_NULL, "%s: q, k, v and cu_seqlens_q are required", who);
-    if (a->dtype != MI_ELEM_DTYPE) return mi_fail(MI_E_DTYPE, "%s: the attention kernels take bf16 or f16 tensors (dtype code %d)", who, a->dtype);
+    if (a->dtype != want_dtype) return mi_fail(MI_E_DTYPE, "%s: dtype code %d does not match the kernels of this entry point (%d)", who, a->dtype, want_dtype);
     if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 96 && a->head_dim != 128)
         return mi_fail(MI_E_SHAPE, "%s: head_dim %d unsupported (32, 64, 96, 128)", who, a->head_dim);
     if (a->n_q_heads <= 0 || a->n_kv_heads <= 0 || a->n_q_heads % a->n_kv_heads != 0)
@@ -494,9 +495,9 @@ static inline int mi_attn_validate(const mi_attn_args* a, const char* who) {
         return mi_fail(MI_E_SHAPE, "%s: non-empty query needs at least one document and one key", who);
     if (!mi_aligned16(a->q) || !mi_aligned16(a->k) || !mi_aligned16(a->v))
         return mi_fail(MI_E_ALIGN, "%s: q, k, v must be 16-byte aligned", who);
-    if (a->q_stride_token % 8 || a->q_stride_head % 8 || a->k_stride_token % 8 || a->k_stride_head % 8 ||
-        a->v_stride_token % 8 || a->v_stride_head % 8)
-        return mi_fail(MI_E_ALIGN, "%s: strides must be multiples of 8 elements", who);
+    if (a->q_stride_token % vec || a->q_stride_head % vec || a->k_stride_token % vec || a->k_stride_head % vec ||
+        a->v_stride_token % vec || a->v_stride_head % vec)
+        return mi_fail(MI_E_ALIGN, "%s: strides must be multiples of %d elements", who, vec);
     if (!(a->softmax_scale > 0.f)) return mi_fail(MI_E_SHAPE, "%s: softmax_scale must be positive", who);
     if (a->rotary_cos || a->rotary_sin) {
         if (!a->rotary_cos || !a->rotary_sin || !a->position_ids_q)

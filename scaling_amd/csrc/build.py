@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libmi355_layer.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 SOURCES = ["abi.hip", "rmsnorm.hip", "swiglu.hip", "rotary.hip", "attn_host.hip", "attn_fwd.hip", "attn_bwd.hip",
-           "attn_decode.hip", "cross_entropy.hip"]
+           "attn_decode.hip", "attn_f32.hip", "cross_entropy.hip"]
 F16_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "attn_decode.hip"]
 # packed fp32 VALU instructions stay disabled for every device translation unit; the kernels never
 # produce NaNs on purpose (masked scores are -inf and every inf - inf is guarded), so NaN-preserving

@@ -341,7 +341,8 @@ class ParallelSelfAttention(torch.nn.Module):
     silent fall-backs: attention-score manipulation, LoRA, local attention windows, u-muP and fp8 are not
     available; attention-probability dropout is applied inside the kernels in training mode (its mask comes
     from a counter-based hash, not from torch's generator stream, and its rate is quantised to 1/256);
-    the dtype must be bfloat16 or float16.  The KV cache is pre-allocated (see `KVCache`), supports batches of
+    float32 (the reference's default precision) runs separate exact-fp32 kernels without dropout, fused rotary or
+    KV cache.  The KV cache is pre-allocated (see `KVCache`), supports batches of
     single-document rows and is filled/extended in place.
     """
 
@@ -371,8 +372,10 @@ class ParallelSelfAttention(torch.nn.Module):
         if num_local_attention_heads > 0 or lora_config is not None or fp8_config is not None or \
                 fp8_config_dense_out is not None or bitfit_bias_name is not None:
             raise NotImplementedError("local attention, LoRA, fp8 and bitfit are outside the hip kernel's scope")
-        if dtype not in (torch.bfloat16, torch.float16):
-            raise NotImplementedError("the hip attention kernels compute in bfloat16 or float16; set precision: bfloat16 (or float16)")
+        if dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise NotImplementedError("the hip attention kernels take bfloat16, float16 or float32 tensors")
+        if dtype == torch.float32 and self.dropout_attention_probs > 0.0:
+            raise NotImplementedError("attention-probability dropout needs precision bfloat16 or float16 with the hip kernel")
 
         self.hidden_size_per_attention_head = hidden_size // num_attention_heads
         self.num_attention_heads = num_attention_heads
@@ -412,7 +415,8 @@ class ParallelSelfAttention(torch.nn.Module):
             self.rotary_embedding = RotaryEmbeddingComplex(config=rotary_config, device=self._device)
         # rotary can be applied inside the attention kernels (on the Q/K load), either pairing
         # when it covers the whole head
-        self._fusable_rotary = self.rotary_embedding is not None and \
+        # (16-bit tensors only: float32 runs the stand-alone rotary kernel in front of the fp32 attention core)
+        self._fusable_rotary = self.rotary_embedding is not None and dtype != torch.float32 and \
             rotary_config.dimensions == self.hidden_size_per_attention_head and self.hidden_size_per_attention_head in (64, 128)
 
         self.key_query_norm = key_query_norm
@@ -519,6 +523,8 @@ class ParallelSelfAttention(torch.nn.Module):
         if use_cache:
             if not self.causal:
                 raise ValueError("KV caching is only supported for causal attention.")
+            if self.dtype == torch.float32:
+                raise NotImplementedError("the KV-cache decode kernels take bfloat16 or float16 tensors")
             assert self._rows_are_single_documents(cu, b, s), "sequence packing is not supported with cache"
             if not reset_cache:
                 return self.dense(self._decode_step(q, k, v, pos, b, s, cache_index).view(b, s, nq * d))

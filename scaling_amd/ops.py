@@ -595,7 +595,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
               cu_seqlens_k: Optional[torch.Tensor] = None, causal: bool = True,
               softmax_scale: Optional[float] = None, dropout_p: float = 0.0,
               dropout_seed: Optional[int] = None, rotary=None, deterministic: bool = False, precise: bool = False) -> torch.Tensor:
-    """Differentiable attention core on q [tokens, n_q, d], k/v [tokens_k, n_kv, d] (bf16).
+    """Differentiable attention core on q [tokens, n_q, d], k/v [tokens_k, n_kv, d] (bfloat16, float16 or float32;
+    float32 tensors run separate kernels on the fp32 matrix pipe with exact fp32 probabilities, without dropout).
 
     Tokens are the flattened (batch seq) axis; cu_seqlens are int32 offsets on it.  Returns
     o [tokens, n_q, d].  dropout_p > 0 drops attention probabilities (attention.py:204-207) with a mask that
@@ -620,6 +621,12 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: t
     if dropout_p > 0.0 and dropout_seed is None:
         dropout_seed = next_dropout_seed(q.device)
     cos = sin = pos_q = pos_k = None
+    if rotary is not None and q.dtype == torch.float32:
+        # float32 tensors: the rotation runs as the stand-alone (differentiable) kernel in front of the fp32 attention core
+        cos, sin, pos_q, pos_k = rotary
+        rot = rotary_embedding_complex if cos.shape[1] * 2 == q.shape[2] else rotary_embedding
+        q, k = rot(q, cos, sin, pos_q), rot(k, cos, sin, pos_k)
+        rotary = cos = sin = pos_q = pos_k = None
     if rotary is not None:
         cos, sin, pos_q, pos_k = rotary
         _fused_rotary_kind(cos, sin, q.shape[2], q.dtype)

@@ -68,8 +68,24 @@ def test_null_and_shape_errors_are_status_codes(lib):
     assert lib.mi_attn_fwd(ctypes.byref(a)) == -1
     a.q = a.k = a.v = a.o = base
     a.cu_seqlens_q = base
-    a.dtype = _lib.MI_F32
-    assert lib.mi_attn_fwd(ctypes.byref(a)) == -2                                                   # dtype
+    a.dtype = 7
+    assert lib.mi_attn_fwd(ctypes.byref(a)) == -2                                                   # unknown dtype code
+    a.dtype = _lib.MI_F32                                                                           # float32: its own kernels
+    a.head_dim, a.n_q_heads, a.n_kv_heads = 64, 2, 2
+    a.rotary_cos = a.rotary_sin = a.position_ids_q = base
+    a.total_q = a.total_k = 4
+    a.n_docs = 1
+    a.q_stride_token = a.k_stride_token = a.v_stride_token = a.o_stride_token = 128
+    a.q_stride_head = a.k_stride_head = a.v_stride_head = a.o_stride_head = 64
+    a.softmax_scale = 0.125
+    a.rotary_table_rows = 4
+    assert lib.mi_attn_fwd(ctypes.byref(a)) == -2 and b"rotary" in lib.mi_last_error()              # no fused rotary in fp32
+    a.rotary_cos = a.rotary_sin = a.position_ids_q = None
+    a.q_stride_head = 62
+    assert lib.mi_attn_fwd(ctypes.byref(a)) == -4                                                   # fp32 strides: multiples of 4
+    a = _lib.MiAttnArgs()
+    a.q = a.k = a.v = a.o = base
+    a.cu_seqlens_q = base
     a.dtype = _lib.MI_BF16
     a.head_dim = 80
     assert lib.mi_attn_fwd(ctypes.byref(a)) == -3

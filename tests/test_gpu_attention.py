@@ -549,3 +549,68 @@ def test_attention_dropout_statistics_and_generator_seed():
     torch.manual_seed(7)
     a2 = ops.attention(q, k, v, cu, None, False, 1.0, dropout_p=p)
     assert torch.equal(a, a2) and not torch.equal(a, b2)
+
+
+# ---- float32 tensors (the reference's default precision) ---------------------------------------------------------------
+@pytest.mark.parametrize("b,s,nq,nkv,d,causal,cuts", [
+    (2, 128, 4, 4, 64, True, ()),                 # config 1 attention shape, in config 1's own dtype
+    (2, 64, 4, 2, 32, False, (32,)),              # GQA, bidirectional, documents
+    (1, 200, 2, 1, 64, True, (3, 77, 78, 150)),   # ragged: not a multiple of the 32-token tiles, tiny documents
+    (2, 96, 8, 2, 128, True, (100,)),
+    (1, 160, 6, 3, 96, True, (33,)),
+    (3, 1, 2, 2, 64, True, ()),                   # one token per sequence
+])
+def test_attention_float32_fwd_bwd_parity(b, s, nq, nkv, d, causal, cuts):
+    """fp32 q / k / v through the fp32 kernels against the oracle in fp32: the stated gates, with no second clause, and
+    far inside them (the arithmetic is fp32 on both sides; what differs is the summation order)."""
+    print(f"case attn f32 b={b} s={s} nq={nq} nkv={nkv} d={d} causal={causal} cuts={cuts}", flush=True)
+    q, k, v, do = U.make_qkv(b, s, nq, nkv, d, seed=7 + s + d, dtype=torch.float32)
+    cu = U.make_cu(b, s, cuts)
+    scale = 1.0 / math.sqrt(d)
+    ref = U.oracle_attention(q, k, v, cu, b, s, causal, scale, torch.float32, do)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o = ops.attention(qg, kg, vg, cu.to(DEV), None, causal, scale)
+    assert o.dtype == torch.float32
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    for name, got, r in (("o", o, ref[0]), ("dq", qg.grad, ref[1]), ("dk", kg.grad, ref[2]), ("dv", vg.grad, ref[3])):
+        m = check(f"attn.f32.{name}", got, r, literal=True, max_abs_tol=1e-4, mean_rel_tol=1e-5)
+        assert m["clause_abs"] == "literal" and m["clause_rel"] == "literal"
+    # bit-reproducible, and GQA equals explicitly repeated heads
+    o2, lse2 = ops.attention_forward(qg.detach(), kg.detach(), vg.detach(), cu.to(DEV), None, causal, scale)
+    assert torch.equal(o2, o.detach())
+    if nq != nkv:
+        rep = nq // nkv
+        o3, _ = ops.attention_forward(qg.detach(), kg.detach().repeat_interleave(rep, 1).contiguous(),
+                                      vg.detach().repeat_interleave(rep, 1).contiguous(), cu.to(DEV), None, causal, scale)
+        assert torch.equal(o3, o2)
+
+
+def test_attention_float32_cross_length_and_rotary():
+    """fp32: keys longer than queries (causal diagonal aligned to the end of the keys), and the rotary embedding applied
+    by the stand-alone kernel in front of the fp32 core when ops.attention is handed fp32 tables."""
+    b, s_q, s_k, nq, nkv, d = 2, 24, 88, 4, 2, 64
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(b * s_q, nq, d, generator=g)
+    k = torch.randn(b * s_k, nkv, d, generator=g)
+    v = torch.randn(b * s_k, nkv, d, generator=g)
+    cu_q = torch.arange(0, b * s_q + 1, s_q, dtype=torch.int32)
+    cu_k = torch.arange(0, b * s_k + 1, s_k, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    o = ops.attention(q.to(DEV), k.to(DEV), v.to(DEV), cu_q.to(DEV), cu_k.to(DEV), True, scale)
+    allowed = torch.ones(s_q, s_k, dtype=torch.bool).tril(diagonal=s_k - s_q)
+    mask = (~allowed).view(1, 1, s_q, s_k).expand(b, 1, s_q, s_k)
+    ref = oracle.multi_head_attention(U.to_sbnd(q, b, s_q), oracle.repeat_kv(U.to_sbnd(k, b, s_k), nq // nkv),
+                                      oracle.repeat_kv(U.to_sbnd(v, b, s_k), nq // nkv), cu_q, True, scale, mask=mask)
+    check("attn.f32.cross.o", o, U.from_bn_s_d(ref, b, nq), literal=True, max_abs_tol=1e-4, mean_rel_tol=1e-5)
+    # rotary through ops.attention on fp32 tensors
+    s = 96
+    q, k, v, do = U.make_qkv(1, s, 4, 2, d, seed=9, dtype=torch.float32)
+    cu = U.make_cu(1, s, (40,))
+    pos = U.position_ids_from_cu(cu, s)
+    tabs = oracle.rotary_tables(d, s, 10000, torch.float32)
+    qr, kr = oracle.apply_rotary(U.to_sbnd(q, 1, s), U.to_sbnd(k, 1, s), tabs, pos.view(s, 1), pos.view(s, 1))
+    ref = U.oracle_attention(qr.permute(1, 0, 2, 3).reshape(s, 4, d), kr.permute(1, 0, 2, 3).reshape(s, 2, d), v, cu, 1, s, True, scale)
+    o = ops.attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), None, True, scale,
+                      rotary=(tabs.cos.to(DEV), tabs.sin.to(DEV), pos.to(DEV), pos.to(DEV)))
+    check("attn.f32.rotary.o", o, ref, literal=True, max_abs_tol=1e-4, mean_rel_tol=1e-5)

@@ -111,6 +111,73 @@ def test_transformer_layer_fwd_bwd_parity(name, kw, b, s, cuts):
         assert m["finite"] and m["mean_rel"] <= max(1e-3, PARAM_GRAD_FLOOR_FRAC * f["mean_rel"]), (k, m, f)
 
 
+def test_config1_layer_float32_through_the_hip_path():
+    """Config 1 as BASELINE states it (hidden 256, 4 heads x 64, SwiGLU 688, RMSNorm, rotary base 10000, causal, batch
+    2 x seq 128, float32): forward + backward of the drop-in layer on the GPU (fp32 attention, norm, SwiGLU and rotary
+    kernels; the projections on the library GEMM in full fp32) against the oracle layer in fp32, the stated gates with no
+    second clause."""
+    print("case layer config 1 float32", flush=True)
+    allow = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        cfg = _arch(precision="float32")
+        layer = _seeded_layer(cfg, seed=0)
+        assert layer.self_attention.query.weight.dtype == torch.float32
+        g = torch.Generator().manual_seed(1)
+        b, s = 2, 128
+        x = torch.randn(b, s, cfg.hidden_size, generator=g)
+        dy = torch.randn(b, s, cfg.hidden_size, generator=g)
+        cu = torch.tensor([0, s, 2 * s], dtype=torch.int32)
+        pos = torch.arange(s).repeat(b, 1)
+        weights = {k: v for k, v in layer.state_dict().items()}
+        ref = _oracle_layer(cfg, weights, x, cu, pos, dy, torch.float32)
+        xg = x.to(DEV).requires_grad_()
+        out = layer(TransformerLayerIO(activations=xg, position_ids=pos.to(DEV), cumulative_seq_lengths=cu.to(DEV)))
+        assert out.activations.dtype == torch.float32
+        out.activations.backward(dy.to(DEV))
+        torch.cuda.synchronize()
+        check("config1.f32.y", out.activations, ref[0], literal=True, max_abs_tol=1e-4, mean_rel_tol=1e-5)
+        check("config1.f32.dx", xg.grad, ref[1], literal=True, max_abs_tol=1e-4, mean_rel_tol=1e-5)
+        for k, p in layer.named_parameters():
+            m = metrics(p.grad, ref[2][k])
+            assert m["finite"] and m["mean_rel"] <= 1e-4, (k, m)
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = allow
+
+
+def test_attention_block_reproduces_the_reference_golden(golden_dir):
+    """`hidden_states_attention` of the reference's own fixture (tests/transformer/files/backward_compatibility_checkpoint,
+    gate 3e-3 in tests/transformer/test_backwards_compatibility.py:175; float32, hidden 16, 2 heads of 8, fused qkv,
+    rotary, causal, 4 tokens) through the GPU kernels: LayerNorm, rotary and the fp32 attention core.  The kernels take
+    head_dim >= 32, so the 8 features of a head are padded with zeros (which change neither scores nor outputs) and the
+    score scale 1 / sqrt(8) is passed explicitly."""
+    import os
+    from scaling_amd import ops
+    d = os.path.join(golden_dir, "backward_compatibility")
+    gt = torch.load(os.path.join(d, "ground_truth.pt"), weights_only=True)
+    sd = torch.load(os.path.join(d, "state_dict.pt"), weights_only=True)
+    gt = {k: (v.detach() if torch.is_tensor(v) else v) for k, v in gt.items()}
+    P = "transformer.layer0."
+    h0 = gt["hidden_states_embedding"].to(DEV)                                   # [1, 4, 16]
+    ln1 = ops.layer_norm(h0, sd[P + "input_layernorm.weight"].to(DEV), sd[P + "input_layernorm.bias"].to(DEV), 1e-5)
+    nh, hd, s = 2, 8, 4
+    qkv = torch.nn.functional.linear(ln1, sd[P + "attention.query_key_value.weight"].to(DEV),
+                                     sd[P + "attention.query_key_value.bias"].to(DEV)).view(s, nh, 3 * hd)
+    q, k, v = qkv[..., :hd], qkv[..., hd:2 * hd], qkv[..., 2 * hd:]                # per head: q then k then v
+    tabs = oracle.rotary_tables(hd, s, 10000, torch.float32)
+    pos = torch.arange(s, device=DEV)
+    q = ops.rotary_embedding(q.contiguous(), tabs.cos.to(DEV), tabs.sin.to(DEV), pos)
+    k = ops.rotary_embedding(k.contiguous(), tabs.cos.to(DEV), tabs.sin.to(DEV), pos)
+    pad = lambda t: torch.nn.functional.pad(t, (0, 32 - hd)).contiguous()           # noqa: E731
+    cu = torch.tensor([0, s], dtype=torch.int32, device=DEV)
+    ctx = ops.attention(pad(q), pad(k), pad(v.contiguous()), cu, None, True, 1.0 / hd ** 0.5)[..., :hd]
+    att = h0 + torch.nn.functional.linear(ctx.reshape(1, s, nh * hd), sd[P + "attention.dense.weight"].to(DEV),
+                                          sd[P + "attention.dense.bias"].to(DEV))
+    err = float((att.cpu() - gt["hidden_states_attention"]).abs().max())
+    print(f"[parity] golden hidden_states_attention: max_abs={err:.3e} (reference gate 3e-3)", flush=True)
+    assert err < 1e-4
+
+
 def test_layer_full_size_properties():
     """Config 4 (hidden 4096, 32 query / 8 KV heads x 128, SwiGLU 14336, batch 2 x sequence 4096), where the oracle
     is out of reach: the step is bit-reproducible, finite, and its backward is linear in the upstream gradient

@@ -159,8 +159,14 @@ def test_unsupported_options_raise():
         ParallelSelfAttention(256, 4, C.MaskedSoftmaxConfig(kernel="torch"), dtype=torch.bfloat16, device=CPU)
     assert ParallelSelfAttention(256, 4, hip, dropout_attention_probs=0.1, dtype=torch.bfloat16, device=CPU,
                                  rotary_config=C.RotaryConfig(dimensions=64)).dropout_attention_probs == 0.1
-    with pytest.raises(NotImplementedError, match="bfloat16"):
-        ParallelSelfAttention(256, 4, hip, dtype=torch.float32, device=CPU)
+    # float32 (the reference's default precision) is accepted: exact-fp32 kernels, stand-alone rotary, no dropout
+    f32 = ParallelSelfAttention(256, 4, hip, dtype=torch.float32, device=CPU, rotary_config=C.RotaryConfig(dimensions=64))
+    assert f32.dtype == torch.float32 and not f32._fusable_rotary and f32.query_key_value.weight.dtype == torch.float32
+    with pytest.raises(NotImplementedError, match="dropout"):
+        ParallelSelfAttention(256, 4, hip, dropout_attention_probs=0.1, dtype=torch.float32, device=CPU,
+                              rotary_config=C.RotaryConfig(dimensions=64))
+    with pytest.raises(NotImplementedError, match="float32"):
+        ParallelSelfAttention(256, 4, hip, dtype=torch.float64, device=CPU, rotary_config=C.RotaryConfig(dimensions=64))
     cplx = ParallelSelfAttention(256, 4, hip, dtype=torch.bfloat16, device=CPU, rotary_config=C.RotaryConfig(dimensions=64, max_seq_length=16),
                                  relative_position_embedding_type=C.RelativePositionEmbeddingType.ROTARY_COMPLEX)
     assert cplx.rotary_embedding.freqs_cis_real.shape == (16, 32) and cplx._fusable_rotary
