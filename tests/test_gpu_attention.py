@@ -409,9 +409,18 @@ def test_attention_rejects_unsupported_input():
     cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
     with pytest.raises(RuntimeError, match="head_dim"):
         ops.attention_forward(q, q, q, cu)
+    # float32 runs its own kernels, which take neither dropout nor the fused rotary
     qf = torch.zeros(8, 2, 64, dtype=torch.float32, device=DEV)
-    with pytest.raises(RuntimeError, match="bf16"):
-        ops.attention_forward(qf, qf, qf, cu)
+    with pytest.raises(RuntimeError, match="dropout"):
+        ops.attention_forward(qf, qf, qf, cu, dropout=(0.1, 3))
+    with pytest.raises(RuntimeError, match="rotary"):
+        a = ops._fill_attn_args(qf, qf, qf, torch.empty_like(qf), torch.empty(2, 8, device=DEV), cu, None, True, 0.125)
+        a.rotary_cos = a.rotary_sin = a.position_ids_q = qf.data_ptr()
+        a.rotary_table_rows = 8
+        ops.check(ops._lib.load().mi_attn_fwd(ops.ctypes.byref(a)), "mi_attn_fwd")
+    qd = torch.zeros(8, 2, 64, dtype=torch.float64, device=DEV)
+    with pytest.raises((RuntimeError, TypeError)):
+        ops.attention_forward(qd, qd, qd, cu)
 
 
 @pytest.mark.parametrize("flags", [1, 2])
