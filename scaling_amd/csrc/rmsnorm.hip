@@ -348,7 +348,9 @@ __global__ __launch_bounds__(kRmsWideBlock) void rmsnorm_bwd_wide_kernel(const T
     for (int i = threadIdx.x; i < hidden; i += kRmsWideBlock) out[i] = dw_lds[i];
 }
 
-// dw[col] = sum_p partial[p][col]; 16 columns x 16 row groups per block, fixed summation order.
+// dw[col] = sum_p partial[p][col]; 32 columns x 8 row groups per block (a row group reads 128 contiguous bytes of a
+// partial row: with 16 columns the 64-byte pieces cost twice their size in fetched sectors), fixed summation order.
+constexpr int kDwCols = 32, kDwGroups = kBlock / kDwCols;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, T* __restrict__ dw,
                                                                     int n_partial, int hidden, T* __restrict__ dw2 = nullptr) {
@@ -357,26 +359,26 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* 
         partial += (int64_t)n_partial * hidden;
         dw = dw2;
     }
-    __shared__ float lds[16][17];
-    const int cl = threadIdx.x % 16, pg = threadIdx.x / 16;
-    const int col = blockIdx.x * 16 + cl;
+    __shared__ float lds[kDwGroups][kDwCols + 1];
+    const int cl = threadIdx.x % kDwCols, pg = threadIdx.x / kDwCols;
+    const int col = blockIdx.x * kDwCols + cl;
     float s = 0.f;
     if (col < hidden) {
         // the launch is latency bound (a few MB, one short dependent chain per thread): 16 loads are requested
-        // before the first is used, so 256 partial rows cost one memory round trip instead of four
+        // before the first is used, so 256 partial rows cost two memory round trips
         constexpr int K = 16;
         float acc[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) acc[k] = 0.f;
         int p = pg;
-        for (; p + 16 * (K - 1) < n_partial; p += 16 * K) {
+        for (; p + kDwGroups * (K - 1) < n_partial; p += kDwGroups * K) {
             float v[K];
 #pragma unroll
-            for (int k = 0; k < K; ++k) v[k] = partial[(int64_t)(p + 16 * k) * hidden + col];
+            for (int k = 0; k < K; ++k) v[k] = partial[(int64_t)(p + kDwGroups * k) * hidden + col];
 #pragma unroll
             for (int k = 0; k < K; ++k) acc[k] += v[k];
         }
-        for (; p < n_partial; p += 16) acc[0] += partial[(int64_t)p * hidden + col];
+        for (; p < n_partial; p += kDwGroups) acc[0] += partial[(int64_t)p * hidden + col];
 #pragma unroll
         for (int w = K / 2; w > 0; w >>= 1)          // fixed pairwise order
 #pragma unroll
@@ -388,7 +390,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* 
     if (pg == 0 && col < hidden) {
         float t = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) t += lds[i][cl];
+        for (int i = 0; i < kDwGroups; ++i) t += lds[i][cl];
         Elem<T>::store1(dw + col, t);
     }
 }
@@ -490,7 +492,7 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
 #undef RMS_WIDE
         int rcw = mi_check_launch("rmsnorm_bwd_wide");
         if (rcw != MI_OK) return rcw;
-        rmsnorm_dw_reduce_kernel<T><<<dim3((unsigned)((hidden + 15) / 16)), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw,
+        rmsnorm_dw_reduce_kernel<T><<<dim3((unsigned)((hidden + kDwCols - 1) / kDwCols)), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw,
                                                                                                    blocks, (int)hidden);
         return mi_check_launch("rmsnorm_dw_reduce");
     }
@@ -503,7 +505,7 @@ int launch_bwd(const void* x, const void* w, const void* dy, void* dx, void* dw,
     if (!launched) return mi_fail(MI_E_SHAPE, "rmsnorm: no kernel for hidden=%lld", (long long)hidden);
     int rc = mi_check_launch("rmsnorm_bwd");
     if (rc != MI_OK) return rc;
-    rmsnorm_dw_reduce_kernel<T><<<dim3((unsigned)((hidden + 15) / 16)), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw,
+    rmsnorm_dw_reduce_kernel<T><<<dim3((unsigned)((hidden + kDwCols - 1) / kDwCols)), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw,
                                                                                                blocks, (int)hidden);
     return mi_check_launch("rmsnorm_dw_reduce");
 }
@@ -1030,7 +1032,7 @@ int launch_ln_bwd(const void* x, const void* w, const void* dy, const float* mea
     if (!launched) return mi_fail(MI_E_SHAPE, "layernorm: no kernel for hidden=%lld", (long long)hidden);
     int rc = mi_check_launch("layernorm_bwd");
     if (rc != MI_OK) return rc;
-    const unsigned rgrid = (unsigned)((hidden + 15) / 16);
+    const unsigned rgrid = (unsigned)((hidden + kDwCols - 1) / kDwCols);
     rmsnorm_dw_reduce_kernel<T><<<dim3(rgrid, db != nullptr ? 2 : 1), dim3(kBlock), 0, st>>>((const float*)ws, (T*)dw, blocks,
                                                                                              (int)hidden, (T*)db);
     return mi_check_launch("layernorm_dw_reduce");
