@@ -56,6 +56,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_delta_kernel(const AttnPara
 // (32 of the 64 queries staged per iteration), so the pair (w, w + 4) accumulates the same dK / dV
 // rows and is summed once at the end.  The first four wavefronts stage Q, the last four dO; the staged
 // tiles are double buffered (one barrier per iteration).
+// __launch_bounds__(512, 2): the second argument is wavefronts per SIMD, i.e. the two that one 512-thread workgroup
+// brings; the kernel takes 250 - 254 of the 256 registers each of them can have (no AGPRs, no scratch).
 template <int D, bool DROP, bool SPLIT>
 __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
     constexpr int BNK = 128;              // keys per workgroup
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     constexpr int TILE = Tile::kBytes;    // one 64-token tile
     constexpr int IPW = Tile::kInstrs / 4;   // direct-load instructions per loader wavefront and 64-token tile
     constexpr int STAGE_BYTES = 4 * TILE + 4 * TILE;  // K, V (two tiles each) + Q, dO (two stages each)
-    constexpr int RED_BYTES = 4 * 16 * DT * 64 * 4;   // one accumulator set of four wavefronts
+    constexpr int RED_BYTES = 8 * 16 * DT * 64 * 4;   // the pair exchange: one accumulator set (dK or dV) of each of the 8 wavefronts
     constexpr int SMEM_BYTES = STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES;
 
     __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
