@@ -76,6 +76,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     __shared__ __attribute__((aligned(16))) float lse_lds[2][BQ];
     __shared__ __attribute__((aligned(16))) float delta_lds[2][BQ];
     __shared__ int range_lds[16];
+    __shared__ int lpt_lds[2 * kLptMax];  // work estimates and hand-out order of the key blocks (packed documents)
     // The streamed tiles come first: with the stage index a compile-time constant (the tile loop is unrolled by two)
     // their LDS addresses are a per-lane register plus an immediate offset, which reaches 64 KB.
     char* q_t = smem;                     // [2 stages]
@@ -103,7 +104,11 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
         kb_rank = blockIdx.x / n_groups;
         group = blockIdx.x - kb_rank * n_groups;
     }
-    const int kb = block_for_rank(kb_rank, nkb, p.n_docs, p.across_k, false);   // key blocks with the most queries first
+    int kb = block_for_rank(kb_rank, nkb, p.n_docs, p.across_k, false);   // key blocks with the most queries first
+    if (p.lpt_k) {                        // documents of different lengths: by the work each key block really has
+        lpt_order<true>(p, nkb, BNK, lpt_lds, lpt_lds + kLptMax);
+        kb = lpt_lds[kLptMax + kb_rank];
+    }
     const int hpw = p.n_rep / p.hsplit;   // query heads of this workgroup: hs * hpw .. + hpw of the group
     const int kvh = group / p.hsplit;
     const int hs = group - kvh * p.hsplit;
@@ -460,6 +465,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     __shared__ __attribute__((aligned(1024))) char k_t[NS * TILE];   // row operand and transposed operand
     __shared__ __attribute__((aligned(1024))) char v_t[NS * TILE];   // row operand
     __shared__ int range_lds[16];
+    __shared__ int lpt_lds[2 * kLptMax];  // work estimates and hand-out order of the query blocks (packed documents)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -469,7 +475,11 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     int head, q_rank;
     head_and_rank(blockIdx.x, p.nq, head, q_rank);
     const int kvh = head / p.n_rep;
-    const int qb = block_for_rank(q_rank, nqb, p.n_docs, p.across_q, true);
+    int qb = block_for_rank(q_rank, nqb, p.n_docs, p.across_q, true);
+    if (p.lpt_q) {                        // documents of different lengths: by the work each query block really has
+        lpt_order<false>(p, nqb, BM, lpt_lds, lpt_lds + kLptMax);
+        qb = lpt_lds[kLptMax + q_rank];
+    }
     const int tq = qb * BM + wave * 32 + l32;
 
     int klo, khi;
@@ -771,8 +781,14 @@ int MI_ENTRY(mi_attn_bwd_impl)(const mi_attn_bwd_args* b) {
             p.dv_part = (float*)((char*)b->workspace + base + part);
         }
     }
-    if (p.n_rep == 1) p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 256);                   // dQ: 256-query blocks
-    if (((a->total_k + 127) / 128) * p.nkv * p.hsplit <= 1024) p.across_k = mi_blocks_per_doc(a->total_k, a->n_docs, 128);   // dK/dV: 128-key blocks
+    if (p.n_rep == 1) {                                                                             // dQ: 256-query blocks
+        p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 256);
+        p.lpt_q = mi_use_lpt(a->total_q, a->n_docs, 256, p.across_q);
+    }
+    if (((a->total_k + 127) / 128) * p.nkv * p.hsplit <= 1024) {                                    // dK/dV: 128-key blocks
+        p.across_k = mi_blocks_per_doc(a->total_k, a->n_docs, 128);
+        p.lpt_k = mi_use_lpt(a->total_k, a->n_docs, 128, p.across_k);
+    }
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
         case 32: return launch_bwd<32>(p, a->flags, st);

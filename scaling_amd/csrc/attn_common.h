@@ -52,6 +52,10 @@ struct AttnParams {
     // blocks per document on the query / key axis when the workgroups are to be handed out across documents
     // (see block_for_rank), 0 for the order along the flattened axis; set by the host entry points
     int across_q, across_k;
+    // documents of different lengths: hand the blocks out longest-processing-time first, by the order that every
+    // workgroup derives from the cumulative lengths itself (see lpt_order); set by the host entry points where the
+    // hand-out across documents pays (same conditions as across_q / across_k) and the batch does not look equal-length
+    int lpt_q, lpt_k;
     // dK/dV with fewer than 8 KV heads: the query heads of a group are split over hsplit workgroups per key block,
     // each writing fp32 partial sums [hsplit][total_k][nkv][head_dim] that a reduce launch adds up (1 = no split)
     int hsplit; float* dk_part; float* dv_part;
@@ -451,6 +455,46 @@ __device__ __forceinline__ int block_for_rank(int rank, int n_blocks, int n_docs
         return doc * per_doc + (late_first ? per_doc - 1 - pos : pos);
     }
     return late_first ? n_blocks - 1 - rank : rank;
+}
+
+// Longest-processing-time-first order of the blocks of a token axis whose documents differ in length: perm_lds[r] =
+// block that is handed out r-th.  A block's work is estimated as the extent of the union of the allowed ranges of its
+// first and its last token (exact for causal and bidirectional documents whose q and k lengths agree); ties go to the
+// lower block index, so the result is a permutation whatever the estimate.  Every workgroup computes the same table
+// from the cumulative lengths (two interval lookups per block, then a rank by counting: n_blocks <= kLptMax keeps
+// that under a microsecond), so no extra launch, workspace or host read-back is involved.  All threads of the
+// workgroup must call; ends with a barrier.
+constexpr int kLptMax = 128;
+template <bool KEY_BLOCKS>
+__device__ __forceinline__ void lpt_order(const AttnParams& p, int n_blocks, int block, int* w_lds, int* perm_lds) {
+    for (int b = threadIdx.x; b < n_blocks; b += blockDim.x) {
+        const int t0 = b * block, t1 = min(t0 + block, KEY_BLOCKS ? p.total_k : p.total_q) - 1;
+        int lo0, hi0, lo1, hi1;
+        if constexpr (KEY_BLOCKS) { query_range(p, t0, lo0, hi0); query_range(p, t1, lo1, hi1); }
+        else { key_range(p, t0, lo0, hi0); key_range(p, t1, lo1, hi1); }
+        int lo = 0x7fffffff, hi = 0;
+        if (hi0 > lo0) { lo = min(lo, lo0); hi = max(hi, hi0); }
+        if (hi1 > lo1) { lo = min(lo, lo1); hi = max(hi, hi1); }
+        w_lds[b] = hi > lo ? hi - lo : 0;
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < n_blocks; b += blockDim.x) {
+        const int wb = w_lds[b];
+        int r = 0;
+        for (int j = 0; j < n_blocks; ++j) {
+            const int wj = w_lds[j];
+            r += (wj > wb || (wj == wb && j < b)) ? 1 : 0;
+        }
+        perm_lds[r] = b;
+    }
+    __syncthreads();
+}
+
+// Host side: whether lpt_order applies (several documents that do not look equal-length, few enough blocks)
+static inline int mi_use_lpt(int64_t total_tokens, int n_docs, int block, int across) {
+    if (n_docs <= 1 || across != 0) return 0;
+    const int64_t n_blocks = (total_tokens + block - 1) / block;
+    return n_blocks > 1 && n_blocks <= kLptMax ? 1 : 0;
 }
 
 // Host side of the above: blocks per document if the batch looks like n_docs documents of one length that is a

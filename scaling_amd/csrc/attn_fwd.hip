@@ -50,6 +50,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     __shared__ __attribute__((aligned(1024))) char k_lds[NS * TILE];
     __shared__ __attribute__((aligned(1024))) char v_lds[NS * TILE];
     __shared__ int range_lds[2 * NW];
+    __shared__ int lpt_lds[2 * kLptMax];  // work estimates and hand-out order of the query blocks (packed documents)
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: role and phase branches stay uniform
@@ -65,6 +66,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     const int nqb = (p.total_q + BM - 1) / BM;
     const int n_items = nqb * p.nq;
     const int G = gridDim.x;
+    if (p.lpt_q) lpt_order<false>(p, nqb, BM, lpt_lds, lpt_lds + kLptMax);   // documents of different lengths, once per workgroup
     for (int pass = 0; pass * G < n_items; ++pass) {
     int idx = blockIdx.x;
     if (pass & 1) idx = (G & 7) == 0 ? ((idx & 7) | (((G >> 3) - 1 - (idx >> 3)) << 3)) : G - 1 - idx;
@@ -73,7 +75,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     int head, q_rank;
     head_and_rank(item, p.nq, head, q_rank);
     const int kvh = head / p.n_rep;
-    const int qb = block_for_rank(q_rank, nqb, p.n_docs, p.across_q, true);   // long query blocks first
+    const int qb = p.lpt_q ? lpt_lds[kLptMax + q_rank]                        // long query blocks first: by their real work,
+                           : block_for_rank(q_rank, nqb, p.n_docs, p.across_q, true);   // or by position
 
     // ---- per-lane query, mask interval, Q fragment ---------------------------------------------
     const int tq = qb * BM + wave * 32 + l32;
@@ -511,7 +514,10 @@ int MI_ENTRY(mi_attn_fwd_impl)(const mi_attn_args* a) {
     if (a->flags & MI_ATTN_QG2) nw = 8;
     const bool split = (a->flags & MI_ATTN_SPLIT_P) != 0;
     if (split) nw = 8;
-    if (p.n_rep == 1) p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 32 * nw);
+    if (p.n_rep == 1) {
+        p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 32 * nw);
+        p.lpt_q = mi_use_lpt(a->total_q, a->n_docs, 32 * nw, p.across_q);
+    }
     hipStream_t st = (hipStream_t)a->stream;
     switch (a->head_dim) {
         case 32: return launch_d<32>(p, rot, q_only, nw, split, st);

@@ -33,6 +33,11 @@ CASES = [
     (2, 256, 8, 1, 128, True, (100, 300)),     # multi-query attention, 8-way split
     (1, 384, 8, 2, 64, False, (129,)),         # 4-way split, bidirectional
     (1, 320, 12, 4, 96, True, ()),             # group of 3: no split possible, the unsplit kernel
+    # documents of different lengths over several blocks: blocks are handed out longest-processing-time first, in an
+    # order every workgroup derives from the cumulative lengths (key blocks in dK/dV; query blocks too when n_q = n_kv)
+    (1, 1300, 4, 4, 64, True, (100, 450, 451, 1000)),
+    (1, 1300, 8, 2, 128, True, (300, 1100)),
+    (1, 1100, 4, 4, 64, False, (64, 700)),
 ]
 
 
