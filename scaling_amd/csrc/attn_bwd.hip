@@ -781,9 +781,10 @@ int MI_ENTRY(mi_attn_bwd_impl)(const mi_attn_bwd_args* b) {
             p.dv_part = (float*)((char*)b->workspace + base + part);
         }
     }
-    if (p.n_rep == 1) {                                                                             // dQ: 256-query blocks
-        p.across_q = mi_blocks_per_doc(a->total_q, a->n_docs, 256);
-        p.lpt_q = mi_use_lpt(a->total_q, a->n_docs, 256, p.across_q);
+    {                                                                                               // dQ: 256-query blocks
+        const int per_doc = mi_blocks_per_doc(a->total_q, a->n_docs, 256);
+        if (p.n_rep == 1) p.across_q = per_doc;
+        p.lpt_q = mi_use_lpt(a->total_q, a->n_docs, 256, per_doc);      // documents of different lengths, any head grouping
     }
     if (((a->total_k + 127) / 128) * p.nkv * p.hsplit <= 1024) {                                    // dK/dV: 128-key blocks
         p.across_k = mi_blocks_per_doc(a->total_k, a->n_docs, 128);
