@@ -11,6 +11,8 @@
 //                     scalar accesses, the row is re-read for each of three passes
 #include "common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int kCeBlock = 1024;
@@ -93,32 +95,86 @@ __device__ __forceinline__ void row_outputs(const CeArgs& a, int64_t row, const 
     (void)target;
 }
 
-template <typename T, int NV>
+// One logit as raw bits (16-bit types zero-extended): a single load instruction with no arithmetic behind it, so
+// that nothing waits for the load where it is issued; bits_to_float converts where the value is used.
+template <typename T> __device__ __forceinline__ uint32_t load1_bits(const T* p) {
+    if constexpr (sizeof(T) == 2) return *reinterpret_cast<const uint16_t*>(p);
+    else return *reinterpret_cast<const uint32_t*>(p);
+}
+template <typename T> __device__ __forceinline__ float bits_to_float(uint32_t b) {
+    if constexpr (std::is_same<T, __bf16>::value) return __uint_as_float(b << 16);
+    else if constexpr (std::is_same<T, _Float16>::value) return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+    else return __uint_as_float(b);
+}
+
+// NL > 0: the first NL vectors per thread of the next row are fetched into LDS by direct global -> LDS loads.  They
+// need no register, so they are in flight during the second pass and the reduction of the current row, when the
+// registers still hold that row and nothing else could be requested; only the remaining NV - NL vectors per thread
+// are requested when the gradient pass frees their registers.
+template <typename T, int NV, int NL>
 __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_rows) {
     constexpr int V = Elem<T>::kVec;
+    static_assert(NL >= 0 && NL <= NV && NL * kCeBlock * 16 <= 152 * 1024, "staging area within the LDS");
     // reduction slots, double-buffered by row parity so that one barrier per row is enough
     __shared__ float lds_m[2][kCeWaves], lds_s[2][kCeWaves];
     __shared__ int lds_i[2][kCeWaves];
+    __shared__ __attribute__((aligned(1024))) u32x4_t stage[NL > 0 ? NL : 1][kCeBlock];
     const int vecs = a.vocab / V;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const bool lane0 = (threadIdx.x & 63) == 0;
+    // LDS byte address of this wavefront's 64 slots of staged vector 0
+    const uint32_t stage_base = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)&stage[0][0]) + (uint32_t)wave * 1024u;
 
-    // A workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ...  The vectors of the next row are requested
-    // as soon as the gradient pass over the current row has consumed the register they land in, so the read of
-    // row r + 1 (and the write of row r) overlap the arithmetic of row r.  Registers past the end of the row are
-    // never loaded and stay at -inf, which every pass treats as "no element" (max ignores it, exp gives 0).
+    // A workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ...  The vectors of the next row that are not
+    // staged are requested as soon as the gradient pass over the current row has consumed the register they land
+    // in, so the read of row r + 1 (and the write of row r) overlap the arithmetic of row r.  Registers past the end
+    // of the row are never loaded and stay at -inf, which every pass treats as "no element" (max ignores it, exp
+    // gives 0).  Staged vectors are whole: the launch asks for vecs >= NL * kCeBlock.
     uint4 raw[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) raw[j] = neg_inf_vec<T>();
     auto row_ptr = [&](int64_t r) { return reinterpret_cast<const T*>(a.logits) + r * a.logits_stride; };
+    auto in_row = [&](int j) { return j < NL || j * kCeBlock + (int)threadIdx.x < vecs; };
     auto load_vec = [&](int64_t r, int j) {
-        const int v = j * kCeBlock + threadIdx.x;
-        if (v < vecs) raw[j] = ldg_nt(reinterpret_cast<const uint4*>(row_ptr(r)) + v);
+        if (in_row(j)) raw[j] = ldg_nt(reinterpret_cast<const uint4*>(row_ptr(r)) + j * kCeBlock + threadIdx.x);
     };
-    auto load_target = [&](int64_t r, int64_t& target, bool& ignored, float& x_target) {
-        target = a.targets[r];
-        ignored = target < 0 || target >= a.vocab;
-        x_target = ignored ? 0.f : Elem<T>::load1(row_ptr(r) + target);   // read before an in-place gradient overwrites it
+    // Direct load of vector j of row r into this thread's staging slot.  A wavefront writes and later reads only its
+    // own 64 slots of a vector, so its own wait for the loads is all the ordering the staging needs.  The compiler
+    // does not count these loads.  Vector memory operations complete in order, so a wait it places for one of its
+    // own loads still covers that load; it waits for the direct loads as well when they are older, which is why
+    // they are issued where no tracked load is consumed before the explicit wait.  The barrier of the reduction
+    // must not wait for them either, hence the hand-written one.
+    auto stage_vec = [&](int64_t r, int j) {
+        const uint32_t dst = stage_base + (uint32_t)j * (kCeBlock * 16u);
+        const uint4* src = reinterpret_cast<const uint4*>(row_ptr(r)) + j * kCeBlock;
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt"
+                     :: "v"((uint32_t)threadIdx.x * 16u), "s"(src), "s"(dst) : "memory", "m0");
+    };
+    auto take_staged = [&](int j) {
+        const u32x4_t x = stage[j][threadIdx.x];
+        raw[j] = make_uint4(x[0], x[1], x[2], x[3]);
+    };
+    auto block_barrier = [&]() {
+        if constexpr (NL > 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else __syncthreads();
+    };
+    // Target and target logit of the next row are requested at the start of the gradient pass, where nothing else is
+    // in flight, the target a row before its logit (whose address it gives): waiting for either at the top of a row
+    // would wait for every older load, i.e. for the whole row in flight.  The index passes through a register the
+    // compiler knows nothing about, or it would move the (uniform) target into scalar registers right behind the
+    // load, which waits on the spot; to_scalar does that a row later.
+    int lane_zero = 0;
+    asm volatile("" : "+v"(lane_zero));
+    auto load_target = [&](int64_t r) { return a.targets[r + lane_zero]; };
+    auto to_scalar = [](int64_t t) {
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)t);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)t >> 32));
+        return (int64_t)(((uint64_t)hi << 32) | lo);
+    };
+    auto is_ignored = [&](int64_t t) { return t < 0 || t >= a.vocab; };
+    auto load_x_bits = [&](int64_t r, int64_t t) {      // read before an in-place gradient overwrites it
+        return is_ignored(t) ? 0u : load1_bits<T>(row_ptr(r) + t);
     };
     auto emit_argmax = [&](int64_t r, int par) {      // thread 0, after a barrier that follows the slot writes
         if (a.argmax == nullptr) return;
@@ -130,29 +186,41 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
 
     int64_t row = blockIdx.x;
     if (row >= n_rows) return;
-    int64_t target, target_next = 0;
-    bool ignored, ignored_next = true;
-    float x_target, x_target_next = 0.f;
 #pragma unroll
     for (int j = 0; j < NV; ++j) load_vec(row, j);
-    load_target(row, target, ignored, x_target);
+    int64_t target = to_scalar(load_target(row));
+    int64_t target_pending = -1;              // of the next row, in flight until the gradient pass
+    if (row + gridDim.x < n_rows) target_pending = load_target(row + gridDim.x);
+    uint32_t x_bits = load_x_bits(row, target), x_bits_next = 0;
 
     int par = 0;
     int64_t prev_row = -1;
     for (; row < n_rows; row += gridDim.x, par ^= 1) {
         const int64_t next = row + gridDim.x;
         const bool has_next = next < n_rows;
-        if (has_next) load_target(next, target_next, ignored_next, x_target_next);
-        // pass 1: this thread's maximum
+        // pass 1: this thread's maximum.  The vectors that came from memory first; once they are here nothing the
+        // compiler tracks is in flight, and the staged part of the next row is requested.
         float mt = -INFINITY;
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
+        auto max_vec = [&](int j) {
             float f[V];
             forget(raw[j]);
             Elem<T>::unpack(raw[j], f);
 #pragma unroll
             for (int i = 0; i < V; ++i) mt = fmaxf(mt, f[i]);
             if (j & 1) __builtin_amdgcn_sched_barrier(0);    // two vectors at a time: unpacking further ahead only costs registers
+        };
+#pragma unroll
+        for (int j = NL; j < NV; ++j) max_vec(j);
+        if constexpr (NL > 0) {
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the slots have been read before they are refilled
+            if (has_next) {
+#pragma unroll
+                for (int j = 0; j < NL; ++j) stage_vec(next, j);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NL; ++j) max_vec(j);
         }
         // pass 2: this thread's sum of exponentials relative to its own maximum
         const float mt2 = (mt == -INFINITY ? 0.f : mt) * kLog2e;
@@ -176,7 +244,7 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
         float ws = (mt == -INFINITY) ? 0.f : (s0 + s1) * __builtin_amdgcn_exp2f((mt - wm) * kLog2e);
         ws = group_sum<64>(ws);
         if (lane0) { lds_m[par][wave] = wm; lds_s[par][wave] = ws; }
-        __syncthreads();
+        block_barrier();
         if (threadIdx.x == 0 && prev_row >= 0) emit_argmax(prev_row, par ^ 1);   // slots of the previous row are complete
         float mx = lds_m[par][0];
 #pragma unroll
@@ -187,39 +255,52 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
             const float m_w = lds_m[par][w];
             sum += (m_w == -INFINITY) ? 0.f : lds_s[par][w] * __builtin_amdgcn_exp2f((m_w - mx) * kLog2e);
         }
-        // first position of the maximum: only the few threads that hold it look, and they re-read their vectors
-        // from memory (cache-hot, not yet overwritten) instead of walking the register copy a fourth time
+        // first position of the maximum: only the wavefronts with a thread that holds it look, walking their register
+        // copy once more (a few hundred instructions for one wavefront; re-reading the vectors from memory instead
+        // put a chain of dependent loads, each behind everything else in flight, on the critical path of the row)
         int arg = 0x7fffffff;
-        if (mt == mx) {
-            const uint4* xr = reinterpret_cast<const uint4*>(row_ptr(row));
-#pragma unroll 1
-            for (int v = threadIdx.x; v < vecs && arg == 0x7fffffff; v += kCeBlock) {
+        if (__any(mt == mx)) {
+#pragma unroll
+            for (int j = NV - 1; j >= 0; --j) {
                 float f[V];
-                Elem<T>::unpack(xr[v], f);
+                forget(raw[j]);
+                Elem<T>::unpack(raw[j], f);
+                const int e0 = (j * kCeBlock + (int)threadIdx.x) * V;
 #pragma unroll
                 for (int i = V - 1; i >= 0; --i)
-                    if (f[i] == mx) arg = v * V + i;
+                    if (f[i] == mx) arg = e0 + i;
+                if (j & 1) __builtin_amdgcn_sched_barrier(0);
             }
         }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) arg = min(arg, __shfl_xor(arg, off, MI_WAVE));
         if (lane0) lds_i[par][wave] = arg;
 
+        // ---- gradient pass.  Everything requested so far is waited for here: the staged part of the next row, the
+        // target of the next row and the target logit of this one.
+        if constexpr (NL > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        const int64_t target_next = to_scalar(target_pending);
+        if (has_next) x_bits_next = load_x_bits(next, target_next);
+        if (next + gridDim.x < n_rows) target_pending = load_target(next + gridDim.x);
+
+        const bool ignored = is_ignored(target);
+        asm volatile("" : "+v"(x_bits));
+        const float x_target = bits_to_float<T>(x_bits);
         const float lse = mx + __builtin_amdgcn_logf(sum) * kLn2;
         const float scale = ignored ? 0.f : (a.row_scale != nullptr ? a.row_scale[row] : 1.0f);
         if (threadIdx.x == 0) {
             if (a.losses != nullptr) a.losses[row] = ignored ? 0.f : lse - x_target;
             if (a.lse != nullptr) a.lse[row] = lse;
         }
-        // pass 3: gradient; the thread that stores the vector holding the target patches that element right
-        // after (two stores of one thread to one address keep their order)
+        // the thread that stores the vector holding the target patches that element right after (two stores of one
+        // thread to one address keep their order)
         T* dx = reinterpret_cast<T*>(a.dlogits) + row * a.dlogits_stride;
         const float l2 = lse * kLog2e;
         const int v_target = ignored ? -1 : (int)(target / V);
-#pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            const int v = j * kCeBlock + threadIdx.x;
-            if (v < vecs) {
+        auto grad_vec = [&](int j) {
+            if (in_row(j)) {
+                const int v = j * kCeBlock + threadIdx.x;
                 float f[V];
                 forget(raw[j]);
                 Elem<T>::unpack(raw[j], f);
@@ -229,15 +310,24 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
                 if (v == v_target)
                     Elem<T>::store1(dx + target, (__builtin_amdgcn_exp2f(x_target * kLog2e - l2) - 1.0f) * scale);
             }
+        };
+#pragma unroll
+        for (int j = NL; j < NV; ++j) {
+            grad_vec(j);
             if (has_next) load_vec(next, j);
+            if (j & 1) __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            grad_vec(j);
+            if (has_next) take_staged(j);
             if (j & 1) __builtin_amdgcn_sched_barrier(0);
         }
         prev_row = row;
         target = target_next;
-        ignored = ignored_next;
-        x_target = x_target_next;
+        x_bits = x_bits_next;
     }
-    __syncthreads();
+    block_barrier();
     if (threadIdx.x == 0) emit_argmax(prev_row, par ^ 1);
 }
 
@@ -468,11 +558,12 @@ int launch_ce(const CeArgs& a, int64_t n_rows, hipStream_t st) {
         // one resident workgroup per compute unit, each walking its share of the rows
         const dim3 pgrid((unsigned)(n_rows < kCeResident ? n_rows : kCeResident));
         const int nr = (int)n_rows;
-        if (nv <= 1) ce_row_kernel<T, 1><<<pgrid, block, 0, st>>>(a, nr);
-        else if (nv <= 2) ce_row_kernel<T, 2><<<pgrid, block, 0, st>>>(a, nr);
-        else if (nv <= 4) ce_row_kernel<T, 4><<<pgrid, block, 0, st>>>(a, nr);
-        else if (nv <= 8) ce_row_kernel<T, 8><<<pgrid, block, 0, st>>>(a, nr);
-        else ce_row_kernel<T, 16><<<pgrid, block, 0, st>>>(a, nr);
+        if (nv <= 1) ce_row_kernel<T, 1, 0><<<pgrid, block, 0, st>>>(a, nr);
+        else if (nv <= 2) ce_row_kernel<T, 2, 0><<<pgrid, block, 0, st>>>(a, nr);
+        else if (nv <= 4) ce_row_kernel<T, 4, 0><<<pgrid, block, 0, st>>>(a, nr);
+        else if (nv <= 8) ce_row_kernel<T, 8, 0><<<pgrid, block, 0, st>>>(a, nr);
+        else if (vecs >= 9 * kCeBlock) ce_row_kernel<T, 16, 9><<<pgrid, block, 0, st>>>(a, nr);
+        else ce_row_kernel<T, 16, 0><<<pgrid, block, 0, st>>>(a, nr);
     } else if (same_phase && a.lse != nullptr && n_rows <= 65535) {
         // rows too long for the register-resident kernel, not a whole number of vectors or not 16-byte aligned:
         // streaming forward, then an elementwise gradient launch

@@ -36,8 +36,10 @@ def _oracle(logits, targets, row_scale):
 
 
 # vocab sizes: one 128-bit vector per thread and less, several vectors per thread (register-resident row), the
-# config-5 vocabulary, sizes that are not a multiple of the vector width and rows beyond the register path
-@pytest.mark.parametrize("rows,vocab", [(7, 128), (33, 1000), (4, 8192), (12, 32000), (6, 128256), (5, 50257), (3, 262144), (2, 3)])
+# config-5 vocabulary, sizes that are not a multiple of the vector width and rows beyond the register path; more rows
+# than compute units, so that a workgroup walks several rows (the next row staged through LDS at the large vocabularies)
+@pytest.mark.parametrize("rows,vocab", [(7, 128), (33, 1000), (4, 8192), (12, 32000), (6, 128256), (5, 50257), (3, 262144), (2, 3),
+                                        (600, 4096), (530, 50000), (777, 128256)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_cross_entropy_parity(rows, vocab, dtype):
     print(f"case cross_entropy rows={rows} vocab={vocab} dtype={dtype}", flush=True)
