@@ -1,6 +1,8 @@
 // Shared device/host helpers for the gfx950 kernels of libmi355_layer.so.
 #pragma once
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
@@ -132,6 +134,35 @@ template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
         v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
     }
     return v;
+}
+
+// The same lane pairing for any associative, commutative operation on 32-bit values (maximum, integer minimum, ...).
+template <int WIDTH, class Op> __device__ __forceinline__ uint32_t group_reduce_bits(uint32_t v, Op op) {
+    static_assert(WIDTH == 1 || WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16 || WIDTH == 32 || WIDTH == 64, "group width");
+    auto dpp = [](uint32_t x, auto ctrl) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, 0xf, 0xf, true);
+    };
+    if constexpr (WIDTH >= 2) v = op(v, dpp(v, std::integral_constant<int, 0xB1>{}));
+    if constexpr (WIDTH >= 4) v = op(v, dpp(v, std::integral_constant<int, 0x4E>{}));
+    if constexpr (WIDTH >= 8) v = op(v, dpp(v, std::integral_constant<int, 0x141>{}));
+    if constexpr (WIDTH >= 16) v = op(v, dpp(v, std::integral_constant<int, 0x140>{}));
+    if constexpr (WIDTH >= 32) {
+        const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+        v = op(r[0], r[1]);
+    }
+    if constexpr (WIDTH >= 64) {
+        const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+        v = op(r[0], r[1]);
+    }
+    return v;
+}
+template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
+    return __uint_as_float(group_reduce_bits<WIDTH>(__float_as_uint(v), [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
+    }));
+}
+template <int WIDTH> __device__ __forceinline__ int group_min(int v) {
+    return (int)group_reduce_bits<WIDTH>((uint32_t)v, [](uint32_t a, uint32_t b) { return (uint32_t)min((int)a, (int)b); });
 }
 
 #define MI_DISPATCH_DTYPE(dtype, ...)                                       \

@@ -238,23 +238,17 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
             if (j & 1) __builtin_amdgcn_sched_barrier(0);
         }
         // merge (maximum, sum) pairs: wavefront, then block
-        float wm = mt;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) wm = fmaxf(wm, __shfl_xor(wm, off, MI_WAVE));
+        const float wm = group_max<64>(mt);
         float ws = (mt == -INFINITY) ? 0.f : (s0 + s1) * __builtin_amdgcn_exp2f((mt - wm) * kLog2e);
         ws = group_sum<64>(ws);
         if (lane0) { lds_m[par][wave] = wm; lds_s[par][wave] = ws; }
         block_barrier();
         if (threadIdx.x == 0 && prev_row >= 0) emit_argmax(prev_row, par ^ 1);   // slots of the previous row are complete
-        float mx = lds_m[par][0];
-#pragma unroll
-        for (int w = 1; w < kCeWaves; ++w) mx = fmaxf(mx, lds_m[par][w]);
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < kCeWaves; ++w) {
-            const float m_w = lds_m[par][w];
-            sum += (m_w == -INFINITY) ? 0.f : lds_s[par][w] * __builtin_amdgcn_exp2f((m_w - mx) * kLog2e);
-        }
+        // every row of 16 lanes merges the 16 slots, one slot per lane
+        static_assert(kCeWaves == 16, "one slot per lane of a 16-lane row");
+        const float m_w = lds_m[par][threadIdx.x & 15], s_w = lds_s[par][threadIdx.x & 15];
+        const float mx = group_max<16>(m_w);
+        const float sum = group_sum<16>((m_w == -INFINITY) ? 0.f : s_w * __builtin_amdgcn_exp2f((m_w - mx) * kLog2e));
         // first position of the maximum: only the wavefronts with a thread that holds it look, walking their register
         // copy once more (a few hundred instructions for one wavefront; re-reading the vectors from memory instead
         // put a chain of dependent loads, each behind everything else in flight, on the critical path of the row)
@@ -271,9 +265,8 @@ __global__ __launch_bounds__(kCeBlock) void ce_row_kernel(const CeArgs a, int n_
                     if (f[i] == mx) arg = e0 + i;
                 if (j & 1) __builtin_amdgcn_sched_barrier(0);
             }
+            arg = group_min<64>(arg);
         }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) arg = min(arg, __shfl_xor(arg, off, MI_WAVE));
         if (lane0) lds_i[par][wave] = arg;
 
         // ---- gradient pass.  Everything requested so far is waited for here: the staged part of the next row, the
