@@ -86,9 +86,9 @@ template <> struct Elem<float> {
 // Non-temporal hint for tensors a launch touches exactly once.  Which side to hint was measured per kernel
 // (8192 x 4096 and 8192 x 14336 bf16 tensors): kernels that read more streams than they write gain from hinted
 // loads (SwiGLU forward 5.7 -> 6.6 TB/s, GELU backward 5.6 -> 6.7, decode attention 5.8 -> 6.3), one-in one-out
-// kernels from hinted stores (GELU forward 5.8 -> 6.8, RMSNorm forward 5.9 -> 6.4), hinting both sides is
-// worse than the better single side except where noted at the call site, and the norm backward kernels
-// lose with any hint.
+// kernels from hinted stores (GELU forward 5.8 -> 6.8, RMSNorm forward 5.9 -> 6.4) and, for the norm forward
+// kernels and rotary, from hinted loads on top (+ 1 - 5 %; a plain 1 GiB copy: 5.6 TB/s without hints, 5.75 with
+// hinted stores, 6.2 with both), and the norm backward kernels lose with any hint.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uint4 ldg_nt(const uint4* p) {

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int v = c * TPR + tr;
-        raw[c] = (row_ok && v < vecs) ? xr[v] : make_uint4(0, 0, 0, 0);
+        raw[c] = (row_ok && v < vecs) ? (ADD ? xr[v] : ldg_nt(xr + v)) : make_uint4(0, 0, 0, 0);
         if constexpr (ADD) {
             if (row_ok && v < vecs) {
                 float a[V], r[V];
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_fwd_kernel(const T* __restri
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int v = c * TPR + tr;
-        const uint4 raw = (row_ok && v < vecs) ? xr[v] : make_uint4(0, 0, 0, 0);
+        const uint4 raw = (row_ok && v < vecs) ? ldg_nt(xr + v) : make_uint4(0, 0, 0, 0);
         Elem<T>::unpack(raw, f[c]);
 #pragma unroll
         for (int i = 0; i < V; ++i) sum += f[c][i];

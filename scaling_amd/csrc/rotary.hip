@@ -62,8 +62,8 @@ __global__ __launch_bounds__(kBlock) void rotary_vec_kernel(RotaryParams p) {
     const TT* cr = (const TT*)p.cos + r * p.rot_dim;
     const TT* sr = (const TT*)p.sin + r * p.rot_dim;
     float x0[V], x1[V], o0[V], o1[V], cA[V], sA[V], cB[V], sB[V];
-    Elem<T>::unpack(*reinterpret_cast<const uint4*>(xrow + c0), x0);
-    Elem<T>::unpack(*reinterpret_cast<const uint4*>(xrow + c1), x1);
+    Elem<T>::unpack(ldg_nt(reinterpret_cast<const uint4*>(xrow + c0)), x0);
+    Elem<T>::unpack(ldg_nt(reinterpret_cast<const uint4*>(xrow + c1)), x1);
     load_table<TT, V>(cr + c0, cA);
     load_table<TT, V>(sr + c0, sA);
     load_table<TT, V>(cr + c1, cB);
