@@ -5,7 +5,8 @@
 // Three kernels:
 //   ce_row_kernel     gradient asked for: 1024-thread workgroups (one per compute unit) walk the rows; a row stays in
 //                     registers (up to 16 x 128-bit vectors per thread, i.e. 131072 16-bit or 65536 fp32 logits), so
-//                     max, sum of exponentials and the gradient all come from the single read
+//                     max, sum of exponentials and the gradient all come from the single read; of rows longer than
+//                     9216 vectors the first 9 vectors per thread of the next row are fetched into LDS meanwhile
 //   ce_fwd_kernel     no gradient: 512-thread workgroups stream a row once with a running (max, sum)
 //   ce_stream_kernel  anything else (rows that do not fit, unaligned rows, vocab not a multiple of the vector width):
 //                     scalar accesses, the row is re-read for each of three passes
