@@ -249,6 +249,7 @@ typedef struct mi_attn_args {
                                       mi_attn_bwd takes as q; NULL = not stored */
 } mi_attn_args;
 
+/* total_q == 0 and total_k == 0 (an empty batch) is not an error: nothing is launched, MI_OK (mi_attn_bwd likewise). */
 int mi_attn_fwd(const mi_attn_args* args);
 
 /* Backward of mi_attn_fwd.  Extra inputs: o and lse from the forward, d_o (layout/strides of o).

@@ -15,12 +15,14 @@ int mi_attn_decode_impl_f16(const mi_decode_args* a, bool static_ws);
 
 extern "C" int mi_attn_fwd(const mi_attn_args* a) {
     if (!a) return mi_fail(MI_E_NULL, "attn_fwd: args is null");
+    if (a->total_q == 0 && a->total_k == 0) return MI_OK;     // no tokens (an empty tensor may come with a null pointer)
     if (a->dtype == MI_F32) return mi_attn_fwd_impl_f32(a);
     return a->dtype == MI_F16 ? mi_attn_fwd_impl_f16(a) : mi_attn_fwd_impl_bf16(a);
 }
 
 extern "C" int mi_attn_bwd(const mi_attn_bwd_args* b) {
     if (!b) return mi_fail(MI_E_NULL, "attn_bwd: args is null");
+    if (b->fwd.total_q == 0 && b->fwd.total_k == 0) return MI_OK;
     if (b->fwd.dtype == MI_F32) return mi_attn_bwd_impl_f32(b);
     return b->fwd.dtype == MI_F16 ? mi_attn_bwd_impl_f16(b) : mi_attn_bwd_impl_bf16(b);
 }

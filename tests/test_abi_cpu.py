@@ -65,6 +65,8 @@ def test_null_and_shape_errors_are_status_codes(lib):
     assert lib.mi_rotary(base, base, base, base, None, 4, 2, 8, 3, 16, 8, 16, 8, 4, 4, 0, 0, 0, None) == -3  # odd rot_dim
     assert lib.mi_attn_fwd(None) == -1
     a = _lib.MiAttnArgs()
+    assert lib.mi_attn_fwd(ctypes.byref(a)) == 0                                                    # no tokens: nothing to do
+    a.total_q = a.total_k = 4
     assert lib.mi_attn_fwd(ctypes.byref(a)) == -1
     a.q = a.k = a.v = a.o = base
     a.cu_seqlens_q = base
@@ -86,12 +88,15 @@ def test_null_and_shape_errors_are_status_codes(lib):
     a = _lib.MiAttnArgs()
     a.q = a.k = a.v = a.o = base
     a.cu_seqlens_q = base
+    a.total_q = a.total_k = 4
     a.dtype = _lib.MI_BF16
     a.head_dim = 80
     assert lib.mi_attn_fwd(ctypes.byref(a)) == -3
     a.head_dim, a.n_q_heads, a.n_kv_heads = 128, 6, 4
     assert lib.mi_attn_fwd(ctypes.byref(a)) == -3                                                   # heads not divisible
     b = _lib.MiAttnBwdArgs()
+    assert lib.mi_attn_bwd(ctypes.byref(b)) == 0                                                    # no tokens
+    b.fwd.total_q = b.fwd.total_k = 4
     assert lib.mi_attn_bwd(ctypes.byref(b)) == -1
     d = _lib.MiDecodeArgs()
     assert lib.mi_attn_decode(ctypes.byref(d)) == -1

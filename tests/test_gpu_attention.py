@@ -38,6 +38,8 @@ CASES = [
     (1, 1300, 4, 4, 64, True, (100, 450, 451, 1000)),
     (1, 1300, 8, 2, 128, True, (300, 1100)),
     (1, 1100, 4, 4, 64, False, (64, 700)),
+    # every token a document of its own (each one an end-of-document token): 300 documents of length 1
+    (1, 300, 4, 2, 64, True, tuple(range(1, 300))),
 ]
 
 
@@ -58,6 +60,17 @@ def test_attention_fwd_bwd_parity(b, s, nq, nkv, d, causal, cuts):
     check("attn.dq", qg.grad, ref[1], ref_o[1], kind="grad")
     check("attn.dk", kg.grad, ref[2], ref_o[2], kind="grad")
     check("attn.dv", vg.grad, ref[3], ref_o[3], kind="grad")
+
+
+def test_attention_of_no_tokens_is_empty():
+    """An empty batch (no tokens at all) is not an error: empty output, empty gradients, no launch."""
+    q = torch.zeros(0, 4, 64, dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    k = torch.zeros(0, 2, 64, dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    v = torch.zeros(0, 2, 64, dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    o = ops.attention(q, k, v, torch.zeros(1, dtype=torch.int32, device=DEV), None, True, 0.125)
+    assert o.shape == (0, 4, 64)
+    o.backward(torch.zeros_like(o))
+    assert q.grad.shape == q.shape and k.grad.shape == k.shape and v.grad.shape == v.shape
 
 
 @pytest.mark.parametrize("b,s,nq,nkv,d,causal,cuts", [
