@@ -1044,22 +1044,22 @@ extern "C" {
 
 int mi_rmsnorm_fwd(const void* x, const void* weight, void* y, float* rstd, int64_t n_rows, int64_t hidden, float eps,
                    int dtype, void* stream) {
+    if (n_rows == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!x || !weight || !y) return mi_fail(MI_E_NULL, "rmsnorm_fwd: null pointer");
     if (n_rows < 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "rmsnorm_fwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
     if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(y)) return mi_fail(MI_E_ALIGN, "rmsnorm_fwd: pointers must be 16-byte aligned");
-    if (n_rows == 0) return MI_OK;
     MI_DISPATCH_DTYPE(dtype, return launch_fwd<T>(x, weight, y, rstd, n_rows, hidden, eps, (hipStream_t)stream));
     return MI_OK;
 }
 
 int mi_add_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* sum_out, void* y, int64_t n_rows,
                        int64_t hidden, float eps, int dtype, void* stream) {
+    if (n_rows == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!x || !residual || !weight || !sum_out || !y) return mi_fail(MI_E_NULL, "add_rmsnorm_fwd: null pointer");
     if (n_rows < 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "add_rmsnorm_fwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
     if (!mi_aligned16(x) || !mi_aligned16(residual) || !mi_aligned16(weight) || !mi_aligned16(sum_out) || !mi_aligned16(y))
         return mi_fail(MI_E_ALIGN, "add_rmsnorm_fwd: pointers must be 16-byte aligned");
     if (y == sum_out || y == x || y == residual) return mi_fail(MI_E_SHAPE, "add_rmsnorm_fwd: y must not alias the other tensors");
-    if (n_rows == 0) return MI_OK;
     MI_DISPATCH_DTYPE(dtype, return launch_fwd<T>(x, weight, y, nullptr, n_rows, hidden, eps, (hipStream_t)stream, residual, sum_out));
     return MI_OK;
 }
@@ -1083,12 +1083,12 @@ int mi_rmsnorm_bwd(const void* x, const void* weight, const void* dy, void* dx, 
 
 int mi_layernorm_fwd(const void* x, const void* weight, const void* bias, void* y, float* mean, float* rstd,
                      int64_t n_rows, int64_t hidden, float eps, int dtype, void* stream) {
+    if (n_rows == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!x || !weight || !y) return mi_fail(MI_E_NULL, "layernorm_fwd: null pointer");
     if ((mean == nullptr) != (rstd == nullptr)) return mi_fail(MI_E_NULL, "layernorm_fwd: mean and rstd go together");
     if (n_rows < 0 || hidden <= 0) return mi_fail(MI_E_SHAPE, "layernorm_fwd: bad shape [%lld, %lld]", (long long)n_rows, (long long)hidden);
     if (!mi_aligned16(x) || !mi_aligned16(weight) || !mi_aligned16(y) || (bias && !mi_aligned16(bias)))
         return mi_fail(MI_E_ALIGN, "layernorm_fwd: pointers must be 16-byte aligned");
-    if (n_rows == 0) return MI_OK;
     MI_DISPATCH_DTYPE(dtype, return launch_ln_fwd<T>(x, weight, bias, y, mean, rstd, n_rows, hidden, eps, (hipStream_t)stream));
     return MI_OK;
 }

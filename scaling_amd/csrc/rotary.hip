@@ -155,13 +155,13 @@ extern "C" int mi_rotary(const void* x, void* out, const void* cos, const void* 
                          int64_t n_tokens, int32_t n_heads, int32_t head_dim, int32_t rot_dim, int64_t x_stride_token,
                          int64_t x_stride_head, int64_t out_stride_token, int64_t out_stride_head, int64_t table_rows,
                          int64_t seq_len_for_null_ids, int inverse, int dtype, int table_dtype, void* stream) {
+    if (n_tokens == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!x || !out || !cos || !sin) return mi_fail(MI_E_NULL, "rotary: null pointer");
     if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0 || rot_dim <= 1 || rot_dim > head_dim || (rot_dim & 1) || table_rows <= 0)
         return mi_fail(MI_E_SHAPE, "rotary: bad shape tokens=%lld heads=%d head_dim=%d rot_dim=%d table_rows=%lld",
                        (long long)n_tokens, n_heads, head_dim, rot_dim, (long long)table_rows);
     if (!position_ids && seq_len_for_null_ids <= 0) return mi_fail(MI_E_SHAPE, "rotary: need position ids or a sequence length");
     if (table_dtype != dtype && table_dtype != MI_F32) return mi_fail(MI_E_DTYPE, "rotary: table dtype must equal the data dtype or be fp32");
-    if (n_tokens == 0) return MI_OK;
     RotaryParams p{x, out, cos, sin, position_ids, n_tokens, n_heads, head_dim, rot_dim, x_stride_token, x_stride_head,
                    out_stride_token, out_stride_head, table_rows, seq_len_for_null_ids, inverse ? -1.0f : 1.0f};
     MI_DISPATCH_DTYPE(dtype, {
@@ -175,11 +175,11 @@ extern "C" int mi_rotary_complex(const void* x, void* out, const float* cos, con
                                  int64_t n_tokens, int32_t n_heads, int32_t head_dim, int64_t x_stride_token,
                                  int64_t x_stride_head, int64_t out_stride_token, int64_t out_stride_head,
                                  int64_t table_rows, int64_t seq_len_for_null_ids, int inverse, int dtype, void* stream) {
+    if (n_tokens == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!x || !out || !cos || !sin) return mi_fail(MI_E_NULL, "rotary_complex: null pointer");
     if (n_tokens < 0 || n_heads <= 0 || head_dim <= 0 || table_rows <= 0)
         return mi_fail(MI_E_SHAPE, "rotary_complex: bad shape tokens=%lld heads=%d head_dim=%d", (long long)n_tokens, n_heads, head_dim);
     if (!position_ids && seq_len_for_null_ids <= 0) return mi_fail(MI_E_SHAPE, "rotary_complex: need position ids or a sequence length");
-    if (n_tokens == 0) return MI_OK;
     RotaryParams p{x, out, cos, sin, position_ids, n_tokens, n_heads, head_dim, head_dim, x_stride_token, x_stride_head,
                    out_stride_token, out_stride_head, table_rows, seq_len_for_null_ids, inverse ? -1.0f : 1.0f};
     MI_DISPATCH_DTYPE(dtype, {

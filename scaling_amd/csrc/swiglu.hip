@@ -174,10 +174,10 @@ template <typename T> unsigned grid_for(int64_t n_elem, int64_t* n_vec) {
 extern "C" {
 
 int mi_swiglu_fwd(const void* a, const void* gate, void* out, int64_t n_elem, int dtype, void* stream) {
+    if (n_elem == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!a || !gate || !out) return mi_fail(MI_E_NULL, "swiglu_fwd: null pointer");
     if (n_elem < 0) return mi_fail(MI_E_SHAPE, "swiglu_fwd: negative size");
     if (!mi_aligned16(a) || !mi_aligned16(gate) || !mi_aligned16(out)) return mi_fail(MI_E_ALIGN, "swiglu_fwd: pointers must be 16-byte aligned");
-    if (n_elem == 0) return MI_OK;
     if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "swiglu_fwd: too many elements");
     MI_DISPATCH_DTYPE(dtype, {
         int64_t n_vec;
@@ -189,11 +189,11 @@ int mi_swiglu_fwd(const void* a, const void* gate, void* out, int64_t n_elem, in
 
 int mi_swiglu_bwd(const void* a, const void* gate, const void* dout, void* da, void* dgate, int64_t n_elem, int dtype,
                   void* stream) {
+    if (n_elem == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!a || !gate || !dout || !da || !dgate) return mi_fail(MI_E_NULL, "swiglu_bwd: null pointer");
     if (n_elem < 0) return mi_fail(MI_E_SHAPE, "swiglu_bwd: negative size");
     if (!mi_aligned16(a) || !mi_aligned16(gate) || !mi_aligned16(dout) || !mi_aligned16(da) || !mi_aligned16(dgate))
         return mi_fail(MI_E_ALIGN, "swiglu_bwd: pointers must be 16-byte aligned");
-    if (n_elem == 0) return MI_OK;
     if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "swiglu_bwd: too many elements");
     MI_DISPATCH_DTYPE(dtype, {
         int64_t n_vec;
@@ -205,10 +205,10 @@ int mi_swiglu_bwd(const void* a, const void* gate, const void* dout, void* da, v
 }
 
 int mi_gelu_fwd(const void* x, void* y, int64_t n_elem, int dtype, void* stream) {
+    if (n_elem == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!x || !y) return mi_fail(MI_E_NULL, "gelu_fwd: null pointer");
     if (n_elem < 0) return mi_fail(MI_E_SHAPE, "gelu_fwd: negative size");
     if (!mi_aligned16(x) || !mi_aligned16(y)) return mi_fail(MI_E_ALIGN, "gelu_fwd: pointers must be 16-byte aligned");
-    if (n_elem == 0) return MI_OK;
     if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "gelu_fwd: too many elements");
     MI_DISPATCH_DTYPE(dtype, {
         int64_t n_vec;
@@ -219,10 +219,10 @@ int mi_gelu_fwd(const void* x, void* y, int64_t n_elem, int dtype, void* stream)
 }
 
 int mi_gelu_bwd(const void* x, const void* dy, void* dx, int64_t n_elem, int dtype, void* stream) {
+    if (n_elem == 0) return MI_OK;       // nothing to do (an empty tensor may come with a null pointer)
     if (!x || !dy || !dx) return mi_fail(MI_E_NULL, "gelu_bwd: null pointer");
     if (n_elem < 0) return mi_fail(MI_E_SHAPE, "gelu_bwd: negative size");
     if (!mi_aligned16(x) || !mi_aligned16(dy) || !mi_aligned16(dx)) return mi_fail(MI_E_ALIGN, "gelu_bwd: pointers must be 16-byte aligned");
-    if (n_elem == 0) return MI_OK;
     if (n_elem / 4 / (kBlock * kUnroll) > 0x7fffffffLL) return mi_fail(MI_E_SHAPE, "gelu_bwd: too many elements");
     MI_DISPATCH_DTYPE(dtype, {
         int64_t n_vec;

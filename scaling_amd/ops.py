@@ -58,6 +58,8 @@ def rms_norm_forward(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch
 def rms_norm_backward(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor, eps: float):
     _need_cuda(x, weight, dy)
     lib = _lib.load()
+    if x.numel() == 0:                   # no rows: no launch, the weight gradient is a sum over nothing
+        return torch.empty_like(x), torch.zeros_like(weight)
     x2 = x.contiguous().view(-1, x.shape[-1])
     dy2 = dy.contiguous().view(-1, x.shape[-1])
     w = weight.contiguous()
@@ -115,6 +117,8 @@ def layer_norm_backward(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor,
     None to have the statistics recomputed."""
     _need_cuda(x, weight, dy)
     lib = _lib.load()
+    if x.numel() == 0:                   # no rows: no launch, the parameter gradients are sums over nothing
+        return torch.empty_like(x), torch.zeros_like(weight), (torch.zeros_like(weight) if need_bias_grad else None)
     if stats is not None:
         assert stats.dtype == torch.float32 and stats.is_contiguous() and stats.shape == (2, x.numel() // x.shape[-1])
     x2 = x.contiguous().view(-1, x.shape[-1])

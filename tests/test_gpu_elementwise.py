@@ -306,3 +306,19 @@ def test_add_rmsnorm_equals_separate_add_and_norm(rows, hidden, dtype):
     ref = oracle.rms_norm((x.float() + r.float()).to(dtype).float().cpu(), w.float().cpu(), 1e-5)
     check("add_rmsnorm.y", y, ref, max_abs_tol=1e-5 if dtype == torch.float32 else 2e-2,
           mean_rel_tol=1e-5 if dtype == torch.float32 else 1e-3)
+
+
+def test_empty_tensors_pass_through_every_elementwise_op():
+    """No rows / no tokens is not an error: outputs of the input's shape, zero parameter gradients, no launch."""
+    w = torch.ones(256, dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    b = torch.zeros(256, dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    x = torch.zeros(0, 256, dtype=torch.bfloat16, device=DEV, requires_grad=True)
+    for y in (ops.rms_norm(x, w, 1e-5), ops.layer_norm(x, w, b, 1e-5), ops.swiglu(x, x.clone()), ops.gelu(x)):
+        assert y.shape == x.shape
+        y.sum().backward()
+    assert x.grad.shape == x.shape and float(w.grad.abs().sum()) == 0.0 and float(b.grad.abs().sum()) == 0.0
+    total, normed = ops.add_rms_norm(x.detach(), x.detach(), w.detach(), 1e-5)
+    assert total.shape == normed.shape == x.shape
+    q = torch.zeros(0, 4, 64, dtype=torch.bfloat16, device=DEV)
+    tables = torch.zeros(16, 64, dtype=torch.bfloat16, device=DEV)
+    assert ops.rotary_embedding(q, tables, tables, torch.zeros(0, dtype=torch.int64, device=DEV)).shape == q.shape
