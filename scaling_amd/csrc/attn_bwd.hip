@@ -117,11 +117,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkdv_kernel(const AttnParams 
     int qlo, qhi;
     query_range(p, key, qlo, qhi);
     int wmin = qhi > qlo ? qlo : 0x7fffffff, wmax = qhi > qlo ? qhi : 0;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        wmin = min(wmin, __shfl_xor(wmin, off, 64));
-        wmax = max(wmax, __shfl_xor(wmax, off, 64));
-    }
+    wmin = group_min<64>(wmin);           // DPP lane reductions: no trips through the LDS crossbar
+    wmax = group_max<64>(wmax);
     if (lane == 0) { range_lds[wave] = wmin; range_lds[8 + wave] = wmax; }
 
     // K / V rows of this key block: loaded once, global -> LDS directly; wavefronts 0-3 fetch K, 4-7 fetch V
@@ -485,11 +482,8 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dq_kernel(const AttnParams p)
     int klo, khi;
     key_range(p, tq, klo, khi);
     int wmin = khi > klo ? klo : 0x7fffffff, wmax = khi > klo ? khi : 0;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        wmin = min(wmin, __shfl_xor(wmin, off, 64));
-        wmax = max(wmax, __shfl_xor(wmax, off, 64));
-    }
+    wmin = group_min<64>(wmin);           // DPP lane reductions: no trips through the LDS crossbar
+    wmax = group_max<64>(wmax);
     if (lane == 0) { range_lds[wave] = wmin; range_lds[8 + wave] = wmax; }
 
     const int tl = tq < p.total_q ? tq : p.total_q - 1;

@@ -124,11 +124,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_kernel(const AttnParams p
     // entry, and every use inside the loop waits for the K/V prefetch issued just before it.
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        wmin = min(wmin, __shfl_xor(wmin, off, 64));
-        wmax = max(wmax, __shfl_xor(wmax, off, 64));
-    }
+    wmin = group_min<64>(wmin);           // DPP lane reductions: no trips through the LDS crossbar
+    wmax = group_max<64>(wmax);
     if (lane == 0) { range_lds[wave] = wmin; range_lds[NW + wave] = wmax; }
     __syncthreads();
     int bmin = 0x7fffffff, bmax = 0;

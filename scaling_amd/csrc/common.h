@@ -164,6 +164,9 @@ template <int WIDTH> __device__ __forceinline__ float group_max(float v) {
 template <int WIDTH> __device__ __forceinline__ int group_min(int v) {
     return (int)group_reduce_bits<WIDTH>((uint32_t)v, [](uint32_t a, uint32_t b) { return (uint32_t)min((int)a, (int)b); });
 }
+template <int WIDTH> __device__ __forceinline__ int group_max(int v) {
+    return (int)group_reduce_bits<WIDTH>((uint32_t)v, [](uint32_t a, uint32_t b) { return (uint32_t)max((int)a, (int)b); });
+}
 
 #define MI_DISPATCH_DTYPE(dtype, ...)                                       \
     switch (dtype) {                                                        \
